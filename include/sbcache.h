@@ -1,0 +1,213 @@
+/*
+ * sbcache.h — C ABI of libsbcache.so: the decode-time cache hot path of a
+ * SpikingBrain-7B-shaped hybrid model (sliding-window paged KV cache, window-bounded
+ * paged decode attention, GLA recurrent-state update) as hand-written HIP kernels for
+ * gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every pointer named in an args struct is a DEVICE pointer unless stated otherwise;
+ *   - strides are in ELEMENTS of the tensor's dtype, sizes are element counts;
+ *   - no entry point allocates, frees or synchronises; kernels are enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL = the null stream);
+ *   - return value: 0 = launched; negative = rejected before launch (SB_ERR_*);
+ *     positive = the hipError_t reported by the launch. sb_last_error() gives the text
+ *     of the most recent failure on the calling thread;
+ *   - no global mutable state: entry points are re-entrant.
+ *
+ * Each entry point cites the reference interface it replaces (paths relative to the
+ * BICLab/SpikingBrain-7B tree).
+ */
+#ifndef SBCACHE_H
+#define SBCACHE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SB_ABI_VERSION 1
+
+enum sb_dtype { SB_BF16 = 0, SB_F16 = 1, SB_F32 = 2 };
+
+enum sb_status {
+  SB_OK = 0,
+  SB_ERR_INVALID = -1,     /* malformed argument (null pointer, bad size, misalignment) */
+  SB_ERR_UNSUPPORTED = -2, /* a shape / dtype the kernels are not instantiated for */
+  SB_ERR_WORKSPACE = -3    /* caller workspace too small */
+};
+
+/* ABI version of the loaded library (== SB_ABI_VERSION of the header it was built from). */
+int sb_abi_version(void);
+
+/* Text of the last failure on this thread ("" if none). Host pointer, valid until the next call. */
+const char *sb_last_error(void);
+
+/* ------------------------------------------------------------------------------------
+ * KV append — scatter new key/value rows into the paged cache at slot_mapping.
+ * Replaces torch.ops._C_cache_ops.reshape_and_cache_flash as called from
+ * vllm_hymeta/attention/meta_attention.py:790-799.
+ *   key/value     [num_tokens, num_kv_heads, head_size]   (token and head strides given)
+ *   k_cache/v_cache [num_blocks, block_size, num_kv_heads, head_size] (strides given;
+ *                 the two halves of the (2, nb, bs, Hkv, D) tensor of meta_attention.py:92)
+ *   slot_mapping  [num_tokens] int64; slot = block*block_size + offset; slot < 0 skips the
+ *                 token (PAD_SLOT_ID, meta_attention.py:558).
+ * Pure byte copy: bit-exact. head_size*sizeof(dtype) must be a multiple of 16 and all
+ * row starts 16-byte aligned.
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_kv_append_args {
+  const void *key;
+  const void *value;
+  void *k_cache;
+  void *v_cache;
+  const int64_t *slot_mapping;
+  int64_t num_tokens;
+  int32_t num_kv_heads;
+  int32_t head_size;
+  int32_t block_size;
+  int32_t dtype; /* enum sb_dtype */
+  int64_t key_stride_token, key_stride_head;
+  int64_t value_stride_token, value_stride_head;
+  int64_t cache_stride_block, cache_stride_row, cache_stride_head;
+  int64_t num_blocks; /* bound for host-side validation only */
+  void *stream;
+} sb_kv_append_args;
+
+int sb_kv_append(const sb_kv_append_args *args);
+
+/* ------------------------------------------------------------------------------------
+ * Window-bounded single-query attention over the paged (or a dense) KV cache.
+ * Replaces flash_attn_2_cuda.fwd_kvcache as called from
+ * vllm_hymeta/attention/fa_kernel_metatoken.py:84-105 (via :157-168 and
+ * meta_attention.py:965-981), with causal=True and window_size=(window_left, -1); and the
+ * decode step of hf_7B_model/window_attention_sdpa.py:186-214 on a dense cache.
+ *
+ * One "query row" r = one query token. Its keys are indices i in [0, seq_lens[r]) of
+ * sequence row_seq[r]; the query sits at index seq_lens[r]-1; key i is visible iff
+ *     max(seq_lens[r]-1-window_left, key_lo[r]) <= i <= seq_lens[r]-1
+ * (window_left < 0 = unbounded; key_lo NULL = 0). A row with no visible key yields zeros
+ * (and lse = -inf), which is what nan_to_num gives at window_attention_sdpa.py:213-214.
+ *
+ * Key addressing, element offset of key i / kv-head h of sequence s:
+ *   paged  (block_table != NULL): blk = block_table[s*block_table_stride + i/block_size]
+ *          blk*kv_stride_block + (i%block_size)*kv_stride_row + h*kv_stride_head
+ *   dense  (block_table == NULL): (kv_start[s] + i)*kv_stride_row + h*kv_stride_head
+ * block_size must be a multiple of 16 in paged mode (meta_attention.py:88-91).
+ *
+ * out[r, hq, :] = softmax_i(scale * q[r,hq,:]·K[i,hq/G,:]) · V[i,hq/G,:], fp32 accumulate,
+ * rounded once to dtype. lse (optional, fp32 [num_rows, num_q_heads], natural log) is the
+ * log-sum-exp of the scaled scores, the quantity fa_kernel_metatoken.py:110-122 merges on.
+ *
+ * The kernel splits each row's window into n_split parts and merges them; partials live
+ * in `workspace` (sb_swa_decode_workspace_bytes). n_split = 0 picks a split count from
+ * the shapes alone (never from device data), so the call is graph-capturable.
+ * head_size must be 128; num_q_heads/num_kv_heads in {1,2,4,7,8}.
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_swa_decode_args {
+  const void *q;   /* [num_rows, num_q_heads, head_size] */
+  const void *k_cache;
+  const void *v_cache;
+  void *out;       /* [num_rows, num_q_heads, head_size] */
+  float *lse;      /* optional */
+  const int32_t *block_table; /* [num_seqs, block_table_stride] or NULL */
+  const int64_t *kv_start;    /* dense mode: first row of each sequence, or NULL (= 0) */
+  const int32_t *row_seq;     /* [num_rows] sequence of each query row, or NULL (= r) */
+  const int32_t *seq_lens;    /* [num_rows] */
+  const int32_t *key_lo;      /* [num_rows] or NULL */
+  void *workspace;
+  size_t workspace_bytes;
+  int64_t num_rows;
+  int32_t num_q_heads, num_kv_heads, head_size, block_size;
+  int32_t window_left;
+  int32_t max_seq_len; /* upper bound of seq_lens (host knowledge); sizes the split */
+  int32_t n_split;     /* 0 = auto */
+  int32_t dtype;
+  float scale;
+  int64_t q_stride_row, q_stride_head;
+  int64_t out_stride_row, out_stride_head;
+  int64_t kv_stride_block, kv_stride_row, kv_stride_head;
+  int64_t block_table_stride;
+  void *stream;
+} sb_swa_decode_args;
+
+/* Split count the auto rule (n_split = 0) would use for these shapes. */
+int32_t sb_swa_decode_auto_split(int64_t num_rows, int32_t num_kv_heads, int32_t max_seq_len,
+                                 int32_t window_left);
+/* Bytes of workspace sb_swa_decode needs for a given split count (0 when n_split == 1). */
+size_t sb_swa_decode_workspace_bytes(int64_t num_rows, int32_t num_q_heads, int32_t head_size,
+                                     int32_t n_split);
+int sb_swa_decode(const sb_swa_decode_args *args);
+
+/* ------------------------------------------------------------------------------------
+ * GLA recurrent step(s) with in-place, slot-indexed state.
+ * Replaces my_fused_recurrent_gla (vllm_hymeta/model_for_7B/my_fused_recurrent.py:9-153,
+ * called from vllm_hymeta/model_for_7B/gla_attention.py:232) for T = 1, and
+ * fla.ops.gla.fused_recurrent_gla as called from hf_7B_model/gla_attention.py:153 for T >= 1.
+ * Per (b, h), for t = 0..T-1:
+ *     S  <- exp(g_t)[:,None] * S + k_t[:,None] * v_t[None,:]        (S is [dk, dv])
+ *     o_t = sum_dk (q_t*scale)[:,None] * S                          (uses the updated S)
+ * State of batch row b is state[slot_idx[b]] (slot_idx NULL = b); slot_idx[b] == -1 leaves
+ * state and output of that row untouched (my_fused_recurrent.py:32-36). fp32 math; state
+ * is read once and written once per call whatever T is. dk = dv = 128.
+ *   q,k,v  [B, H, T, 128] dtype `dtype` (batch/head/time strides given)
+ *   g      [B, H, T, 128] dtype `g_dtype` (log-space gate per key dim)
+ *   state  [num_slots, H, 128, 128] dtype `state_dtype` (SB_F32 or SB_BF16)
+ *   out    [B, H, T, 128] dtype `dtype`
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_gla_recurrent_args {
+  const void *q, *k, *v, *g;
+  void *state;
+  void *out;
+  const int32_t *slot_idx;
+  int64_t batch;
+  int32_t num_heads, seq_len, head_dim;
+  int32_t dtype, g_dtype, state_dtype;
+  float scale;
+  int64_t q_stride_b, q_stride_h, q_stride_t;
+  int64_t k_stride_b, k_stride_h, k_stride_t;
+  int64_t v_stride_b, v_stride_h, v_stride_t;
+  int64_t g_stride_b, g_stride_h, g_stride_t;
+  int64_t out_stride_b, out_stride_h, out_stride_t;
+  int64_t state_stride_slot, state_stride_head;
+  int64_t num_slots; /* bound for documentation; slot_idx values are trusted */
+  void *stream;
+} sb_gla_recurrent_args;
+
+int sb_gla_recurrent(const sb_gla_recurrent_args *args);
+
+/* ------------------------------------------------------------------------------------
+ * Block copy inside one device (copy-on-write of cache blocks).
+ * Replaces ops.copy_blocks as called from meta_attention.py:115-126, for ONE cache
+ * tensor half per call.  pairs = [num_pairs, 2] int64 (src block, dst block).
+ * ------------------------------------------------------------------------------------ */
+int sb_copy_blocks(void *cache, const int64_t *pairs, int64_t num_pairs, int64_t block_bytes,
+                   int64_t stride_block_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Dense sliding-window append for the HuggingFace-style cache.
+ * Replaces the roll + slice-assign of hf_7B_model/cache.py:96-104: dst holds, per (b, h),
+ * the last (keep) rows of src followed by the n new rows, in chronological order.
+ * src/dst rows are [rows, D] planes addressed as plane p = b*H + h:
+ *     src + p*src_stride_plane + (src_row0 + r)*D,  dst likewise. Byte copy, bit-exact.
+ * Used by the cache's amortised compaction (one call per `capacity - window` appends).
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_window_shift_args {
+  const void *src; /* old storage */
+  void *dst;       /* new storage (must not overlap src rows being read) */
+  const void *fresh; /* new rows [planes, n_new, D] with stride fresh_stride_plane / fresh_stride_row, may be NULL */
+  int64_t planes;
+  int64_t keep_rows, src_row0, dst_row0;
+  int64_t n_new;
+  int64_t row_bytes;
+  int64_t src_stride_plane_bytes, dst_stride_plane_bytes;
+  int64_t fresh_stride_plane_bytes, fresh_stride_row_bytes;
+  void *stream;
+} sb_window_shift_args;
+
+int sb_window_shift(const sb_window_shift_args *args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SBCACHE_H */

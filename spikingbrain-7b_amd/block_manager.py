@@ -1,0 +1,201 @@
+"""Host-side bookkeeping of the paged sliding-window KV cache: physical block allocation,
+window eviction / block recycling, slot mapping and the windowed block-table view.
+
+In the reference this work is done by vLLM's v0 block manager and model runner (not vendored
+there); the reference's own files fix the call pattern: the metadata builder takes the last
+`curr_sliding_window_block` entries of each table and computes slots with
+`compute_slot_mapping_start_idx` / `compute_slot_mapping`
+(vllm_hymeta/attention/meta_attention.py:474-494), pads tables with 0 and slots with
+PAD_SLOT_ID (:556-569), and one block table is shared by all SWA layers.
+
+Policy of this manager (its own specification, deterministic):
+  * free blocks form a LIFO stack that initially pops 0, 1, 2, ...;
+  * per engine step and per sequence, in batch-row order: first evict every resident logical
+    block that lies wholly before the window of the FIRST new token
+    (logical block < (p0 - window_left) // block_size), lowest first, pushing each on the
+    stack; then allocate, in position order, a block for every stored token whose logical
+    block has none. With window_left a multiple of block_size a decoding sequence therefore
+    recycles its own oldest block: a fixed ring of window_left/block_size + 1 blocks;
+  * a prompt stores only tokens i >= query_len - window_left (older ones get PAD_SLOT_ID).
+Per-sequence tables are rings indexed by logical block modulo the ring size, so a step costs
+O(events) Python work plus vectorised numpy, independent of the context length.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+PAD_SLOT_ID = -1
+
+
+def compute_slot_mapping_start_idx(is_prompt: bool, query_len: int, context_len: int,
+                                   sliding_window: Optional[int]) -> int:
+    """First token index of a prompt that is cached at all (call site meta_attention.py:489-491)."""
+    start_idx = 0
+    if is_prompt and sliding_window is not None:
+        start_idx = max(0, query_len - sliding_window)
+    return start_idx
+
+
+def compute_slot_mapping(is_profile_run: bool, slot_mapping: List[int], seq_id, seq_len: int, context_len: int,
+                         start_idx: int, block_size: int, block_tables) -> None:
+    """Append one slot per new token i in [context_len, seq_len) (call site meta_attention.py:492-494):
+    PAD_SLOT_ID below start_idx, else block_tables[seq_id][i // block_size] * block_size + i % block_size.
+    `block_tables[seq_id]` must be indexable by ABSOLUTE logical block (a list, or the
+    `LogicalTable` view of this module)."""
+    if is_profile_run:
+        slot_mapping.extend([PAD_SLOT_ID] * seq_len)
+        return
+    slot_mapping.extend([PAD_SLOT_ID] * max(0, start_idx - context_len))
+    table = block_tables[seq_id]
+    first = max(start_idx, context_len)
+    if seq_len > first:
+        pos = np.arange(first, seq_len, dtype=np.int64)
+        blocks = np.asarray([table[j] for j in range(first // block_size, (seq_len - 1) // block_size + 1)],
+                            dtype=np.int64)
+        slot_mapping.extend((blocks[pos // block_size - first // block_size] * block_size + pos % block_size).tolist())
+
+
+class LogicalTable:
+    """Read-only view of one sequence's ring as a table indexed by absolute logical block."""
+
+    def __init__(self, mgr: "WindowBlockManager", row: int):
+        self._mgr, self._row = mgr, row
+
+    def __getitem__(self, j: int) -> int:
+        m, r = self._mgr, self._row
+        if j < m.lo[r] or j > m.hi[r]:
+            raise IndexError(f"logical block {j} is not resident (resident {m.lo[r]}..{m.hi[r]})")
+        return int(m.ring[r, j % m.ring_blocks])
+
+
+class WindowBlockManager:
+    """Block allocator + per-sequence window rings for up to `max_seqs` live sequences."""
+
+    def __init__(self, num_blocks: int, block_size: int, window_left: int, max_seqs: int,
+                 max_chunk_tokens: int = 0):
+        if block_size % 16 != 0 or block_size < 16:
+            raise ValueError(f"Invalid block size {block_size}. Must be a multiple of 16 and at least 16.")
+        if window_left < 0:
+            raise ValueError("window_left must be >= 0 (an unbounded window needs no eviction)")
+        self.num_blocks, self.block_size, self.window_left = num_blocks, block_size, window_left
+        # most blocks a sequence can hold: window + the tokens of one step, unaligned at both ends
+        self.ring_blocks = (window_left + max(1, max_chunk_tokens)) // block_size + 2
+        self.ring = np.zeros((max_seqs, self.ring_blocks), dtype=np.int32)
+        self.n_tokens = np.zeros(max_seqs, dtype=np.int64)
+        self.lo = np.zeros(max_seqs, dtype=np.int64)        # lowest resident logical block
+        self.hi = np.full(max_seqs, -1, dtype=np.int64)     # highest resident logical block (-1: none)
+        self._stack = np.arange(num_blocks - 1, -1, -1, dtype=np.int32)
+        self._top = num_blocks                              # number of free blocks
+        self._rows: Dict[object, int] = {}
+        self._free_rows = list(range(max_seqs - 1, -1, -1))
+
+    # -- sequences ------------------------------------------------------------------
+    def add_seq(self, seq_id) -> int:
+        if seq_id in self._rows:
+            raise KeyError(f"sequence {seq_id!r} already exists")
+        if not self._free_rows:
+            raise RuntimeError("no free sequence row")
+        r = self._free_rows.pop()
+        self._rows[seq_id] = r
+        self.n_tokens[r], self.lo[r], self.hi[r] = 0, 0, -1
+        return r
+
+    def free_seq(self, seq_id) -> None:
+        r = self._rows.pop(seq_id)
+        for j in range(int(self.lo[r]), int(self.hi[r]) + 1):
+            self._push(int(self.ring[r, j % self.ring_blocks]))
+        self.lo[r], self.hi[r], self.n_tokens[r] = 0, -1, 0
+        self._free_rows.append(r)
+
+    def row_of(self, seq_id) -> int:
+        return self._rows[seq_id]
+
+    @property
+    def num_free_blocks(self) -> int:
+        return self._top
+
+    def free_stack(self) -> List[int]:
+        """Free physical blocks, bottom of the stack first (the next allocation takes the last)."""
+        return self._stack[:self._top].tolist()
+
+    def _push(self, blk: int) -> None:
+        self._stack[self._top] = blk
+        self._top += 1
+
+    def _pop(self) -> int:
+        if self._top == 0:
+            raise RuntimeError("out of KV cache blocks")
+        self._top -= 1
+        return int(self._stack[self._top])
+
+    # -- one engine step ------------------------------------------------------------
+    def _advance_row(self, r: int, count: int, is_prompt: bool) -> Tuple[int, int]:
+        """Evict + allocate for `count` new tokens of row r; returns (p0, first stored position)."""
+        bs, wl, R = self.block_size, self.window_left, self.ring_blocks
+        p0 = int(self.n_tokens[r])
+        lo_new = max(0, (p0 - wl) // bs)
+        lo, hi = int(self.lo[r]), int(self.hi[r])
+        for j in range(lo, min(lo_new, hi + 1)):
+            self._push(int(self.ring[r, j % R]))
+        if hi >= lo:
+            lo = max(lo, lo_new)
+            if lo > hi:  # everything evicted
+                lo, hi = 0, -1
+        start_idx = compute_slot_mapping_start_idx(is_prompt, count, p0, wl)
+        first = max(p0, start_idx)
+        end = p0 + count
+        if end > first:
+            jb, je = first // bs, (end - 1) // bs
+            if hi < lo:
+                lo, hi = jb, jb - 1
+            if je - lo + 1 > R:
+                raise RuntimeError(f"{je - lo + 1} resident blocks exceed the ring of {R}; raise max_chunk_tokens")
+            for j in range(max(jb, hi + 1), je + 1):
+                self.ring[r, j % R] = self._pop()
+            hi = max(hi, je)
+        self.lo[r], self.hi[r] = lo, hi
+        self.n_tokens[r] = end
+        return p0, first
+
+    def append_tokens(self, seq_id, count: int, is_prompt: bool) -> List[int]:
+        """Slots of `count` new tokens of one sequence (one prompt chunk or one decode token)."""
+        r = self._rows[seq_id]
+        p0, first = self._advance_row(r, count, is_prompt)
+        slots: List[int] = []
+        compute_slot_mapping(False, slots, r, p0 + count, p0, first, self.block_size, {r: LogicalTable(self, r)})
+        return slots
+
+    def decode_step(self, seq_ids: Sequence) -> np.ndarray:
+        """One new token for every sequence of `seq_ids` (batch-row order); returns slot_mapping
+        int64 [len(seq_ids)]. Only rows that cross a block boundary do Python work."""
+        bs, wl, R = self.block_size, self.window_left, self.ring_blocks
+        rows = np.fromiter((self._rows[s] for s in seq_ids), dtype=np.int64, count=len(seq_ids))
+        p = self.n_tokens[rows]
+        need_evict = (np.maximum(0, (p - wl) // bs) > self.lo[rows]) & (self.hi[rows] >= self.lo[rows])
+        need_alloc = (p // bs) > self.hi[rows]
+        for i in np.nonzero(need_evict | need_alloc)[0]:
+            self._advance_row(int(rows[i]), 1, False)
+        quiet = ~(need_evict | need_alloc)
+        self.n_tokens[rows[quiet]] += 1
+        return self.ring[rows, (p // bs) % R].astype(np.int64) * bs + p % bs
+
+    # -- kernel view ----------------------------------------------------------------
+    def kernel_view(self, seq_ids: Sequence, pad_blocks: Optional[int] = None) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+        """(block_tables int32 [B, max_blocks] padded with 0, cache_seqlens int32 [B], first resident
+        position int64 [B]). Key index k of row b is absolute position first[b] + k; the newest
+        token sits at index cache_seqlens[b] - 1."""
+        R, bs = self.ring_blocks, self.block_size
+        rows = np.fromiter((self._rows[s] for s in seq_ids), dtype=np.int64, count=len(seq_ids))
+        lo, hi = self.lo[rows], self.hi[rows]
+        nblk = np.maximum(hi - lo + 1, 0)
+        width = int(nblk.max()) if len(rows) else 0
+        if pad_blocks is not None:
+            if pad_blocks < width:
+                raise ValueError(f"pad_blocks {pad_blocks} < widest table {width}")
+            width = pad_blocks
+        j = lo[:, None] + np.arange(width, dtype=np.int64)[None, :]
+        tables = np.where(j <= hi[:, None], self.ring[rows[:, None], j % R], 0).astype(np.int32)
+        seqlens = np.where(nblk > 0, self.n_tokens[rows] - lo * bs, 0).astype(np.int32)
+        return tables, seqlens, lo * bs

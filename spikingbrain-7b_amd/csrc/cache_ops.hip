@@ -1,0 +1,159 @@
+// Byte-moving kernels of the cache path: slot-mapped KV append, block copy, and the
+// dense-window shift used by the HuggingFace-style cache. All are pure copies in 16-byte
+// lanes (one wavefront moves 1 KiB per instruction), so results are bit-exact.
+#include "common.h"
+
+namespace {
+
+// One wavefront per (token, K|V). A row of num_kv_heads*head_size elements is moved as
+// 16-byte chunks; chunk c belongs to head c / chunks_per_head.
+__global__ __launch_bounds__(256) void kv_append_kernel(
+    const char *__restrict__ key, const char *__restrict__ value, char *__restrict__ k_cache,
+    char *__restrict__ v_cache, const int64_t *__restrict__ slot_mapping, int64_t num_tokens,
+    int chunks_per_head, int n_chunks, int block_size, int64_t key_tok_b, int64_t key_head_b,
+    int64_t val_tok_b, int64_t val_head_b, int64_t blk_b, int64_t row_b, int64_t head_b) {
+  const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int lane = threadIdx.x & 63;
+  const int64_t tok = wave >> 1;
+  const int which = (int)(wave & 1);
+  if (tok >= num_tokens) return;
+  const int64_t slot = slot_mapping[tok];
+  if (slot < 0) return;  // padded lane / token older than the window
+  const int64_t blk = slot / block_size;
+  const int64_t off = slot - blk * block_size;
+  const char *src = which ? value + tok * val_tok_b : key + tok * key_tok_b;
+  const int64_t src_head_b = which ? val_head_b : key_head_b;
+  char *dst = (which ? v_cache : k_cache) + blk * blk_b + off * row_b;
+  for (int c = lane; c < n_chunks; c += 64) {
+    const int h = c / chunks_per_head;
+    const int w = c - h * chunks_per_head;
+    const uint4 x = *reinterpret_cast<const uint4 *>(src + h * src_head_b + (int64_t)w * 16);
+    *reinterpret_cast<uint4 *>(dst + h * head_b + (int64_t)w * 16) = x;
+  }
+}
+
+// One workgroup per (pair, 4 KiB segment of the block).
+__global__ __launch_bounds__(256) void copy_blocks_kernel(char *__restrict__ cache,
+                                                          const int64_t *__restrict__ pairs,
+                                                          int64_t block_bytes,
+                                                          int64_t stride_block_bytes) {
+  const int64_t pair = blockIdx.y;
+  const int64_t src = pairs[2 * pair], dst = pairs[2 * pair + 1];
+  const int64_t byte0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 16;
+  if (byte0 >= block_bytes || src == dst) return;
+  const uint4 x = *reinterpret_cast<const uint4 *>(cache + src * stride_block_bytes + byte0);
+  *reinterpret_cast<uint4 *>(cache + dst * stride_block_bytes + byte0) = x;
+}
+
+// Dense window shift: per plane, dst rows [dst_row0, dst_row0+keep) <- src rows
+// [src_row0, src_row0+keep), then n_new fresh rows behind them.
+// grid: (ceil(rows*chunks / 256), planes)
+__global__ __launch_bounds__(256) void window_shift_kernel(
+    const char *__restrict__ src, char *__restrict__ dst, const char *__restrict__ fresh,
+    int64_t keep_rows, int64_t src_row0, int64_t dst_row0, int64_t n_new, int64_t row_bytes,
+    int64_t src_plane_b, int64_t dst_plane_b, int64_t fresh_plane_b, int64_t fresh_row_b) {
+  const int64_t plane = blockIdx.y;
+  const int64_t chunks_per_row = row_bytes >> 4;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = idx / chunks_per_row;
+  const int64_t c = idx - row * chunks_per_row;
+  if (row >= keep_rows + n_new) return;
+  uint4 x;
+  if (row < keep_rows) {
+    x = *reinterpret_cast<const uint4 *>(src + plane * src_plane_b + (src_row0 + row) * row_bytes +
+                                         c * 16);
+  } else {
+    x = *reinterpret_cast<const uint4 *>(fresh + plane * fresh_plane_b +
+                                         (row - keep_rows) * fresh_row_b + c * 16);
+  }
+  *reinterpret_cast<uint4 *>(dst + plane * dst_plane_b + (dst_row0 + row) * row_bytes + c * 16) = x;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+extern "C" int sb_kv_append(const sb_kv_append_args *a) {
+  using namespace sb_host;
+  if (!a) return fail(SB_ERR_INVALID, "sb_kv_append: null args");
+  if (a->num_tokens < 0) return fail(SB_ERR_INVALID, "sb_kv_append: negative num_tokens");
+  if (a->num_tokens == 0) return SB_OK;
+  if (!a->key || !a->value || !a->k_cache || !a->v_cache || !a->slot_mapping)
+    return fail(SB_ERR_INVALID, "sb_kv_append: null tensor pointer");
+  int esz;
+  switch (a->dtype) {
+    case SB_BF16:
+    case SB_F16: esz = 2; break;
+    case SB_F32: esz = 4; break;
+    default: return fail(SB_ERR_UNSUPPORTED, "sb_kv_append: unknown dtype %d", a->dtype);
+  }
+  if (a->num_kv_heads <= 0 || a->head_size <= 0 || a->block_size <= 0)
+    return fail(SB_ERR_INVALID, "sb_kv_append: non-positive shape");
+  const int64_t head_bytes = (int64_t)a->head_size * esz;
+  if (head_bytes % 16 != 0)
+    return fail(SB_ERR_UNSUPPORTED, "sb_kv_append: head_size*elem (%lld B) not a multiple of 16",
+                (long long)head_bytes);
+  const int64_t strides[] = {a->key_stride_token,   a->key_stride_head,  a->value_stride_token,
+                             a->value_stride_head,  a->cache_stride_block, a->cache_stride_row,
+                             a->cache_stride_head};
+  for (int64_t s : strides)
+    if ((s * esz) % 16 != 0)
+      return fail(SB_ERR_INVALID, "sb_kv_append: stride %lld elements is not 16-byte aligned",
+                  (long long)s);
+  if (!aligned16(a->key) || !aligned16(a->value) || !aligned16(a->k_cache) || !aligned16(a->v_cache))
+    return fail(SB_ERR_INVALID, "sb_kv_append: tensor base not 16-byte aligned");
+  const int chunks_per_head = (int)(head_bytes / 16);
+  const int n_chunks = chunks_per_head * a->num_kv_heads;
+  const int64_t waves = a->num_tokens * 2;
+  const int64_t blocks = (waves + 3) / 4;
+  if (blocks > 0x7fffffffLL) return fail(SB_ERR_UNSUPPORTED, "sb_kv_append: too many tokens");
+  hipLaunchKernelGGL(kv_append_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)a->stream,
+                     (const char *)a->key, (const char *)a->value, (char *)a->k_cache,
+                     (char *)a->v_cache, a->slot_mapping, a->num_tokens, chunks_per_head, n_chunks,
+                     a->block_size, a->key_stride_token * esz, a->key_stride_head * esz,
+                     a->value_stride_token * esz, a->value_stride_head * esz,
+                     a->cache_stride_block * esz, a->cache_stride_row * esz,
+                     a->cache_stride_head * esz);
+  return check_launch("kv_append_kernel");
+}
+
+extern "C" int sb_copy_blocks(void *cache, const int64_t *pairs, int64_t num_pairs,
+                              int64_t block_bytes, int64_t stride_block_bytes, void *stream) {
+  using namespace sb_host;
+  if (num_pairs < 0) return fail(SB_ERR_INVALID, "sb_copy_blocks: negative num_pairs");
+  if (num_pairs == 0) return SB_OK;
+  if (!cache || !pairs) return fail(SB_ERR_INVALID, "sb_copy_blocks: null pointer");
+  if (block_bytes <= 0 || block_bytes % 16 != 0 || stride_block_bytes % 16 != 0 || !aligned16(cache))
+    return fail(SB_ERR_INVALID, "sb_copy_blocks: sizes must be positive multiples of 16 bytes");
+  if (num_pairs > 65535) return fail(SB_ERR_UNSUPPORTED, "sb_copy_blocks: more than 65535 pairs");
+  const unsigned gx = (unsigned)((block_bytes / 16 + 255) / 256);
+  hipLaunchKernelGGL(copy_blocks_kernel, dim3(gx, (unsigned)num_pairs), dim3(256), 0,
+                     (hipStream_t)stream, (char *)cache, pairs, block_bytes, stride_block_bytes);
+  return check_launch("copy_blocks_kernel");
+}
+
+extern "C" int sb_window_shift(const sb_window_shift_args *a) {
+  using namespace sb_host;
+  if (!a) return fail(SB_ERR_INVALID, "sb_window_shift: null args");
+  if (a->planes < 0 || a->keep_rows < 0 || a->n_new < 0)
+    return fail(SB_ERR_INVALID, "sb_window_shift: negative size");
+  const int64_t rows = a->keep_rows + a->n_new;
+  if (a->planes == 0 || rows == 0) return SB_OK;
+  if (!a->dst || (a->keep_rows > 0 && !a->src) || (a->n_new > 0 && !a->fresh))
+    return fail(SB_ERR_INVALID, "sb_window_shift: null pointer");
+  if (a->row_bytes <= 0 || a->row_bytes % 16 != 0 || a->src_stride_plane_bytes % 16 != 0 ||
+      a->dst_stride_plane_bytes % 16 != 0 || a->fresh_stride_plane_bytes % 16 != 0 ||
+      a->fresh_stride_row_bytes % 16 != 0 || !aligned16(a->dst) || !aligned16(a->src) ||
+      !aligned16(a->fresh))
+    return fail(SB_ERR_INVALID, "sb_window_shift: rows and strides must be 16-byte multiples");
+  if (a->planes > 65535) return fail(SB_ERR_UNSUPPORTED, "sb_window_shift: more than 65535 planes");
+  const int64_t work = rows * (a->row_bytes / 16);
+  const int64_t gx = (work + 255) / 256;
+  if (gx > 0x7fffffffLL) return fail(SB_ERR_UNSUPPORTED, "sb_window_shift: too many rows");
+  hipLaunchKernelGGL(window_shift_kernel, dim3((unsigned)gx, (unsigned)a->planes), dim3(256), 0,
+                     (hipStream_t)a->stream, (const char *)a->src, (char *)a->dst,
+                     (const char *)a->fresh, a->keep_rows, a->src_row0, a->dst_row0, a->n_new,
+                     a->row_bytes, a->src_stride_plane_bytes, a->dst_stride_plane_bytes,
+                     a->fresh_stride_plane_bytes, a->fresh_stride_row_bytes);
+  return check_launch("window_shift_kernel");
+}

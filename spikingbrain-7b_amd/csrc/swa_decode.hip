@@ -1,0 +1,452 @@
+// Window-bounded single-query attention over a paged (or dense) KV cache, split-K.
+//
+// Work decomposition
+//   grid = (query rows, kv heads, splits); one 256-thread workgroup (4 wavefronts) handles
+//   one kv head of one query row over one contiguous part of the visible window, for all G
+//   query heads of the GQA group at once, so every K/V byte is fetched from HBM once and
+//   used G times.
+//   The window is cut into tiles of 16 keys (a vLLM cache block is a whole number of tiles).
+//   Inside a wavefront lane = (g, c): c = lane%16 owns head dims [8c, 8c+8) (one 16-byte
+//   vector of a bf16 row), g = lane/16 picks one of the 4 key rows a load instruction covers,
+//   so one instruction fetches 4 whole 256-byte rows. Partial dot products are all-reduced
+//   over the 16 lanes of a row with DPP; each of the 4 row groups keeps its own online-softmax
+//   state (m, l, acc[G][8]) and the 16 row groups of a workgroup are merged once at the end
+//   (registers -> LDS), then either normalised and stored (n_split == 1) or written as an
+//   fp32 partial (m, l, acc) that swa_decode_merge_kernel combines.
+//   Scores are kept in log2 units: p = exp2(s*scale*log2e - m).
+#include "common.h"
+
+namespace {
+
+using namespace sb;
+
+struct DecodeParams {
+  const char *q;
+  const char *k;
+  const char *v;
+  char *out;
+  float *lse;
+  const int32_t *block_table;
+  const int64_t *kv_start;
+  const int32_t *row_seq;
+  const int32_t *seq_lens;
+  const int32_t *key_lo;
+  float *ws_acc;  // [rows, Hq, n_split, 128]
+  float *ws_ml;   // [rows, Hq, n_split, 2]
+  int Hq, block_size, window_left, n_split;
+  float scale_log2;
+  int64_t q_sr, q_sh, o_sr, o_sh;  // elements
+  int64_t kv_sb, kv_sr, kv_sh;     // bytes
+  int64_t bt_stride;
+};
+
+template <typename E>
+struct Pack {
+  uint32_t w[E::kPackWords];
+};
+
+template <typename E>
+__device__ __forceinline__ Pack<E> load_pack(const char *p) {
+  Pack<E> r;
+  const uint4 a = *reinterpret_cast<const uint4 *>(p);
+  r.w[0] = a.x; r.w[1] = a.y; r.w[2] = a.z; r.w[3] = a.w;
+  if constexpr (E::kPackWords == 8) {
+    const uint4 b = *reinterpret_cast<const uint4 *>(p + 16);
+    r.w[4] = b.x; r.w[5] = b.y; r.w[6] = b.z; r.w[7] = b.w;
+  }
+  return r;
+}
+
+template <typename E>
+__device__ __forceinline__ float dot_pack(const Pack<E> &a, const Pack<E> &b) {
+  float s = 0.f;
+  if constexpr (E::kPackWords == 8) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s = fmaf(__uint_as_float(a.w[i]), __uint_as_float(b.w[i]), s);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s = E::dot2(a.w[i], b.w[i], s);
+  }
+  return s;
+}
+
+template <typename E>
+__device__ __forceinline__ void unpack(const Pack<E> &a, float (&f)[8]) {
+  if constexpr (E::kPackWords == 8) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = __uint_as_float(a.w[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = E::lo(a.w[i]);
+      f[2 * i + 1] = E::hi(a.w[i]);
+    }
+  }
+}
+
+template <typename E>
+__device__ __forceinline__ void store_out(char *out, int64_t idx, float x) {
+  if constexpr (E::kPackWords == 8) {
+    reinterpret_cast<float *>(out)[idx] = x;
+  } else {
+    reinterpret_cast<uint16_t *>(out)[idx] = (uint16_t)(E::pack(x, 0.f) & 0xffffu);
+  }
+}
+
+constexpr float kNegInf = -__builtin_inff();
+
+template <typename E, int G>
+__global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParams p) {
+  constexpr int kPackBytes = 8 * E::kBytes;
+  constexpr bool kPrefetch = (E::kBytes == 2);
+
+  const int64_t r = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int split = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+
+  const int64_t seq = p.row_seq ? (int64_t)p.row_seq[r] : r;
+  const int hi = p.seq_lens[r];
+  int lo = p.window_left >= 0 ? max(0, hi - 1 - p.window_left) : 0;
+  if (p.key_lo) lo = max(lo, p.key_lo[r]);
+
+  const int first_tile = lo >> 4;
+  const int n_tiles = hi > lo ? ((hi - 1) >> 4) - first_tile + 1 : 0;
+  const int tps = (n_tiles + p.n_split - 1) / p.n_split;
+  const int tb = first_tile + split * tps;
+  const int te = min(tb + tps, first_tile + n_tiles);
+
+  // query vectors of the group, this lane's 8 dims
+  Pack<E> qp[G];
+#pragma unroll
+  for (int h = 0; h < G; ++h)
+    qp[h] = load_pack<E>(p.q + (r * p.q_sr + (int64_t)(kvh * G + h) * p.q_sh + c * 8) * E::kBytes);
+
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    m[h] = kNegInf;
+    l[h] = 0.f;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc[h][d] = 0.f;
+  }
+
+  const bool paged = p.block_table != nullptr;
+  const int64_t dense_row0 = (!paged && p.kv_start) ? p.kv_start[seq] : 0;
+  const int64_t lane_off = (int64_t)kvh * p.kv_sh + c * kPackBytes;
+
+  // byte offset of the first row of tile t (uniform over the wavefront)
+  auto tile_base = [&](int t) -> int64_t {
+    if (t >= te) return 0;
+    const int i0 = t << 4;
+    if (paged) {
+      const int bi = i0 / p.block_size;
+      const int64_t blk = p.block_table[seq * p.bt_stride + bi];
+      return blk * p.kv_sb + (int64_t)(i0 - bi * p.block_size) * p.kv_sr;
+    }
+    return (dense_row0 + i0) * p.kv_sr;
+  };
+  // rows past the last key are clamped onto it (never read outside the sequence)
+  auto load_tile = [&](int t, int64_t base, Pack<E> (&kb)[4], Pack<E> (&vb)[4]) {
+    const int i0 = t << 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = min(4 * j + g, hi - 1 - i0);
+      const int64_t off = base + (int64_t)row * p.kv_sr + lane_off;
+      kb[j] = load_pack<E>(p.k + off);
+      vb[j] = load_pack<E>(p.v + off);
+    }
+  };
+
+  auto compute_tile = [&](int t, const Pack<E> (&kb)[4], const Pack<E> (&vb)[4]) {
+    const int i0 = t << 4;
+    float s[G][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int h = 0; h < G; ++h) s[h][j] = row16_allreduce_sum(dot_pack<E>(qp[h], kb[j]));
+    if (i0 < lo || i0 + 16 > hi) {  // edge tile: mask keys outside [lo, hi)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = i0 + 4 * j + g;
+        if (i < lo || i >= hi) {
+#pragma unroll
+          for (int h = 0; h < G; ++h) s[h][j] = kNegInf;
+        }
+      }
+    }
+    float alpha[G];
+    bool grew = false;
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      const float mx = fmaxf(fmaxf(s[h][0], s[h][1]), fmaxf(s[h][2], s[h][3])) * p.scale_log2;
+      const float m_new = fmaxf(m[h], mx);
+      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+      grew |= (m_new > m[h]);
+      alpha[h] = fast_exp2(m[h] - m_safe);
+      float psum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s[h][j] = fast_exp2(fmaf(s[h][j], p.scale_log2, -m_safe));
+        psum += s[h][j];
+      }
+      l[h] = fmaf(l[h], alpha[h], psum);
+      m[h] = m_new;
+    }
+    if (__builtin_amdgcn_ballot_w64(grew) != 0) {
+#pragma unroll
+      for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int d = 0; d < 8; ++d) acc[h][d] *= alpha[h];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float vf[8];
+      unpack<E>(vb[j], vf);
+#pragma unroll
+      for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int d = 0; d < 8; ++d) acc[h][d] = fmaf(s[h][j], vf[d], acc[h][d]);
+    }
+  };
+
+  int t = tb + wave;
+  if constexpr (kPrefetch) {
+    Pack<E> kb[4], vb[4];
+    int64_t base1 = tile_base(t + 4);
+    if (t < te) load_tile(t, tile_base(t), kb, vb);
+    while (t < te) {
+      const int64_t base2 = tile_base(t + 8);
+      Pack<E> kn[4], vn[4];
+      const bool more = (t + 4 < te);
+      if (more) load_tile(t + 4, base1, kn, vn);
+      compute_tile(t, kb, vb);
+      if (more) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          kb[j] = kn[j];
+          vb[j] = vn[j];
+        }
+      }
+      base1 = base2;
+      t += 4;
+    }
+  } else {
+    for (; t < te; t += 4) {
+      Pack<E> kb[4], vb[4];
+      load_tile(t, tile_base(t), kb, vb);
+      compute_tile(t, kb, vb);
+    }
+  }
+
+  // ---- merge the 4 row groups of this wavefront ------------------------------------
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    const float mo = m[h];
+    float M = fmaxf(mo, __shfl_xor(mo, 16));
+    M = fmaxf(M, __shfl_xor(M, 32));
+    const float f = (mo == kNegInf) ? 0.f : fast_exp2(mo - M);
+    float lv = l[h] * f;
+    lv += __shfl_xor(lv, 16);
+    lv += __shfl_xor(lv, 32);
+    l[h] = lv;
+    m[h] = M;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+      float a = acc[h][d] * f;
+      a += __shfl_xor(a, 16);
+      a += __shfl_xor(a, 32);
+      acc[h][d] = a;
+    }
+  }
+
+  // ---- merge the 4 wavefronts through LDS ---------------------------------------------
+  __shared__ float s_m[4][G], s_l[4][G];
+  __shared__ __attribute__((aligned(16))) float s_acc[4][G][128];
+  if (g == 0) {
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      if (c == 0) {
+        s_m[wave][h] = m[h];
+        s_l[wave][h] = l[h];
+      }
+      float4 *dst = reinterpret_cast<float4 *>(&s_acc[wave][h][c * 8]);
+      dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+      dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * 128; idx += 256) {
+    const int h = idx >> 7, d = idx & 127;
+    const float M = fmaxf(fmaxf(s_m[0][h], s_m[1][h]), fmaxf(s_m[2][h], s_m[3][h]));
+    float tot = 0.f, L = 0.f;
+    if (M != kNegInf) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float mw = s_m[w][h];
+        const float f = (mw == kNegInf) ? 0.f : fast_exp2(mw - M);
+        tot = fmaf(s_acc[w][h][d], f, tot);
+        L = fmaf(s_l[w][h], f, L);
+      }
+    }
+    const int hq = kvh * G + h;
+    if (p.n_split == 1) {
+      store_out<E>(p.out, r * p.o_sr + (int64_t)hq * p.o_sh + d, L > 0.f ? tot / L : 0.f);
+      if (d == 0 && p.lse) p.lse[r * p.Hq + hq] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
+    } else {
+      const int64_t part = (r * p.Hq + hq) * p.n_split + split;
+      p.ws_acc[part * 128 + d] = tot;
+      if (d == 0) {
+        p.ws_ml[part * 2] = M;
+        p.ws_ml[part * 2 + 1] = L;
+      }
+    }
+  }
+}
+
+// One 128-thread workgroup per (query row, query head): log-sum-exp merge of the splits.
+template <typename E>
+__global__ __launch_bounds__(128) void swa_decode_merge_kernel(const DecodeParams p) {
+  const int64_t rh = blockIdx.x;  // r*Hq + hq
+  const int64_t r = rh / p.Hq;
+  const int hq = (int)(rh - r * p.Hq);
+  const int d = threadIdx.x;
+  const float *ml = p.ws_ml + rh * p.n_split * 2;
+  float M = kNegInf;
+  for (int s = 0; s < p.n_split; ++s) M = fmaxf(M, ml[2 * s]);
+  float tot = 0.f, L = 0.f;
+  if (M != kNegInf) {
+    const float *acc = p.ws_acc + rh * p.n_split * 128 + d;
+    for (int s = 0; s < p.n_split; ++s) {
+      const float ms = ml[2 * s];
+      const float f = (ms == kNegInf) ? 0.f : fast_exp2(ms - M);
+      tot = fmaf(acc[(int64_t)s * 128], f, tot);
+      L = fmaf(ml[2 * s + 1], f, L);
+    }
+  }
+  store_out<E>(p.out, r * p.o_sr + (int64_t)hq * p.o_sh + d, L > 0.f ? tot / L : 0.f);
+  if (d == 0 && p.lse) p.lse[rh] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
+}
+
+template <typename E>
+int launch_for_group(int G, dim3 grid, hipStream_t st, const DecodeParams &p) {
+  switch (G) {
+    case 1: hipLaunchKernelGGL((swa_decode_split_kernel<E, 1>), grid, dim3(256), 0, st, p); return 0;
+    case 2: hipLaunchKernelGGL((swa_decode_split_kernel<E, 2>), grid, dim3(256), 0, st, p); return 0;
+    case 4: hipLaunchKernelGGL((swa_decode_split_kernel<E, 4>), grid, dim3(256), 0, st, p); return 0;
+    case 7: hipLaunchKernelGGL((swa_decode_split_kernel<E, 7>), grid, dim3(256), 0, st, p); return 0;
+    case 8: hipLaunchKernelGGL((swa_decode_split_kernel<E, 8>), grid, dim3(256), 0, st, p); return 0;
+    default: return -1;
+  }
+}
+
+inline int64_t round_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace
+
+extern "C" int32_t sb_swa_decode_auto_split(int64_t num_rows, int32_t num_kv_heads,
+                                            int32_t max_seq_len, int32_t window_left) {
+  if (num_rows <= 0 || num_kv_heads <= 0 || max_seq_len <= 0) return 1;
+  int64_t keys = max_seq_len;
+  if (window_left >= 0 && keys > (int64_t)window_left + 1) keys = (int64_t)window_left + 1;
+  const int64_t tiles = (keys + 15) / 16 + 1;  // +1: an unaligned window touches one more tile
+  // aim at ~2048 workgroups (8 per CU on 256 CUs), at least 4 tiles (one per wavefront) each
+  const int64_t groups = num_rows * num_kv_heads;
+  int64_t n = (2048 + groups - 1) / groups;
+  const int64_t cap = (tiles + 3) / 4;
+  if (n > cap) n = cap;
+  if (n > 64) n = 64;
+  if (n < 1) n = 1;
+  return (int32_t)n;
+}
+
+extern "C" size_t sb_swa_decode_workspace_bytes(int64_t num_rows, int32_t num_q_heads,
+                                                int32_t head_size, int32_t n_split) {
+  if (n_split <= 1 || num_rows <= 0 || num_q_heads <= 0 || head_size <= 0) return 0;
+  const int64_t parts = num_rows * num_q_heads * (int64_t)n_split;
+  return (size_t)(round_up(parts * head_size * 4, 256) + round_up(parts * 2 * 4, 256));
+}
+
+extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
+  using namespace sb_host;
+  if (!a) return fail(SB_ERR_INVALID, "sb_swa_decode: null args");
+  if (a->num_rows < 0) return fail(SB_ERR_INVALID, "sb_swa_decode: negative num_rows");
+  if (a->num_rows == 0) return SB_OK;
+  if (!a->q || !a->k_cache || !a->v_cache || !a->out || !a->seq_lens)
+    return fail(SB_ERR_INVALID, "sb_swa_decode: null tensor pointer");
+  if (a->head_size != 128)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: head_size %d (only 128 is built)", a->head_size);
+  if (a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_q_heads % a->num_kv_heads != 0)
+    return fail(SB_ERR_INVALID, "sb_swa_decode: num_q_heads must be a positive multiple of num_kv_heads");
+  if (!(a->scale > 0.f)) return fail(SB_ERR_INVALID, "sb_swa_decode: scale must be positive");
+  if (a->block_table && (a->block_size < 16 || a->block_size % 16 != 0))
+    return fail(SB_ERR_INVALID, "sb_swa_decode: block_size %d must be a multiple of 16", a->block_size);
+  if (a->num_rows > 0x7fffffffLL || a->num_kv_heads > 65535)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: grid too large");
+  int esz;
+  switch (a->dtype) {
+    case SB_BF16:
+    case SB_F16: esz = 2; break;
+    case SB_F32: esz = 4; break;
+    default: return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: unknown dtype %d", a->dtype);
+  }
+  const int64_t es[] = {a->q_stride_row, a->q_stride_head, a->kv_stride_block, a->kv_stride_row,
+                        a->kv_stride_head};
+  for (int64_t s : es)
+    if ((s * esz) % 16 != 0)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: stride %lld elements is not 16-byte aligned",
+                  (long long)s);
+  if ((reinterpret_cast<uintptr_t>(a->q) | reinterpret_cast<uintptr_t>(a->k_cache) |
+       reinterpret_cast<uintptr_t>(a->v_cache)) & 15u)
+    return fail(SB_ERR_INVALID, "sb_swa_decode: q/k/v base not 16-byte aligned");
+
+  int n_split = a->n_split;
+  if (n_split < 0) return fail(SB_ERR_INVALID, "sb_swa_decode: negative n_split");
+  if (n_split == 0)
+    n_split = sb_swa_decode_auto_split(a->num_rows, a->num_kv_heads, a->max_seq_len, a->window_left);
+  if (n_split > 65535) return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: n_split > 65535");
+  const size_t need = sb_swa_decode_workspace_bytes(a->num_rows, a->num_q_heads, 128, n_split);
+  if (need > 0 && (!a->workspace || a->workspace_bytes < need))
+    return fail(SB_ERR_WORKSPACE, "sb_swa_decode: workspace of %zu bytes needed for n_split=%d, got %zu",
+                need, n_split, a->workspace ? a->workspace_bytes : (size_t)0);
+  if (need > 0 && (reinterpret_cast<uintptr_t>(a->workspace) & 15u))
+    return fail(SB_ERR_INVALID, "sb_swa_decode: workspace not 16-byte aligned");
+
+  DecodeParams p;
+  p.q = (const char *)a->q; p.k = (const char *)a->k_cache; p.v = (const char *)a->v_cache;
+  p.out = (char *)a->out; p.lse = a->lse;
+  p.block_table = a->block_table; p.kv_start = a->kv_start; p.row_seq = a->row_seq;
+  p.seq_lens = a->seq_lens; p.key_lo = a->key_lo;
+  const int64_t parts = a->num_rows * a->num_q_heads * (int64_t)n_split;
+  p.ws_acc = (float *)a->workspace;
+  p.ws_ml = need ? (float *)((char *)a->workspace + round_up(parts * 128 * 4, 256)) : nullptr;
+  p.Hq = a->num_q_heads; p.block_size = a->block_size > 0 ? a->block_size : 16;
+  p.window_left = a->window_left; p.n_split = n_split;
+  p.scale_log2 = a->scale * sb::kLog2e;
+  p.q_sr = a->q_stride_row; p.q_sh = a->q_stride_head;
+  p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
+  p.kv_sb = a->kv_stride_block * esz; p.kv_sr = a->kv_stride_row * esz; p.kv_sh = a->kv_stride_head * esz;
+  p.bt_stride = a->block_table_stride;
+
+  const int G = a->num_q_heads / a->num_kv_heads;
+  const dim3 grid((unsigned)a->num_rows, (unsigned)a->num_kv_heads, (unsigned)n_split);
+  hipStream_t st = (hipStream_t)a->stream;
+  int rc;
+  if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
+  else if (a->dtype == SB_F16) rc = launch_for_group<F16>(G, grid, st, p);
+  else rc = launch_for_group<F32>(G, grid, st, p);
+  if (rc != 0)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: GQA group size %d (built: 1, 2, 4, 7, 8)", G);
+  rc = check_launch("swa_decode_split_kernel");
+  if (rc != SB_OK || n_split == 1) return rc;
+
+  const dim3 mgrid((unsigned)(a->num_rows * a->num_q_heads));
+  if (a->dtype == SB_BF16) hipLaunchKernelGGL(swa_decode_merge_kernel<BF16>, mgrid, dim3(128), 0, st, p);
+  else if (a->dtype == SB_F16) hipLaunchKernelGGL(swa_decode_merge_kernel<F16>, mgrid, dim3(128), 0, st, p);
+  else hipLaunchKernelGGL(swa_decode_merge_kernel<F32>, mgrid, dim3(128), 0, st, p);
+  return check_launch("swa_decode_merge_kernel");
+}

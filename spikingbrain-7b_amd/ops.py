@@ -1,0 +1,259 @@
+"""Tensor-level wrappers over the C ABI: validate shapes the way the reference's callers expect,
+then enqueue the HIP kernel on torch's current stream. No wrapper computes anything itself.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _native as N
+
+PAD_SLOT_ID = -1
+
+_workspaces: Dict[torch.device, torch.Tensor] = {}
+
+
+def _workspace(dev: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+    """Per-device scratch for split-K partials, grown on demand and reused by every call on
+    the device (calls on one device are stream-ordered, so they never overlap)."""
+    if nbytes == 0:
+        return None
+    ws = _workspaces.get(dev)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _workspaces[dev] = ws
+    return ws
+
+
+def _inner_contiguous(t: torch.Tensor, name: str) -> None:
+    if t.stride(-1) != 1:
+        raise ValueError(f"{name} must have a contiguous last dimension, got strides {t.stride()}")
+
+
+def kv_append(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+              slot_mapping: torch.Tensor) -> None:
+    """Scatter key/value [T, Hkv, D] into the paged caches [nb, bs, Hkv, D] at slot_mapping [T]
+    (int64; negative = skip). Same contract as reshape_and_cache_flash at
+    vllm_hymeta/attention/meta_attention.py:790-799 with an unquantised kv_cache_dtype."""
+    dev = N.require_gpu(key, value, key_cache, value_cache, slot_mapping)
+    if key.dim() != 3 or value.shape != key.shape:
+        raise ValueError(f"key/value must both be [num_tokens, num_kv_heads, head_size], got {tuple(key.shape)} "
+                         f"and {tuple(value.shape)}")
+    if key_cache.dim() != 4 or value_cache.shape != key_cache.shape:
+        raise ValueError("key_cache/value_cache must both be [num_blocks, block_size, num_kv_heads, head_size]")
+    T, Hkv, D = key.shape
+    nb, bs, Hc, Dc = key_cache.shape
+    if (Hc, Dc) != (Hkv, D):
+        raise ValueError(f"cache heads/head_size {(Hc, Dc)} do not match key {(Hkv, D)}")
+    if not (key.dtype == value.dtype == key_cache.dtype == value_cache.dtype):
+        raise ValueError("key, value and caches must share one dtype (quantised KV is not supported)")
+    if slot_mapping.dtype != torch.int64:
+        raise ValueError(f"slot_mapping must be int64, got {slot_mapping.dtype}")
+    slot_mapping = slot_mapping.flatten()
+    if slot_mapping.numel() < T:
+        raise ValueError(f"slot_mapping has {slot_mapping.numel()} entries for {T} tokens")
+    if not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.contiguous()
+    for t, n in ((key, "key"), (value, "value"), (key_cache, "key_cache"), (value_cache, "value_cache")):
+        _inner_contiguous(t, n)
+    if key_cache.stride() != value_cache.stride():
+        raise ValueError("key_cache and value_cache must have identical strides")
+    a = N.KvAppendArgs(
+        key=N.ptr(key), value=N.ptr(value), k_cache=N.ptr(key_cache), v_cache=N.ptr(value_cache),
+        slot_mapping=N.ptr(slot_mapping), num_tokens=T, num_kv_heads=Hkv, head_size=D, block_size=bs,
+        dtype=N.dtype_code(key.dtype),
+        key_stride_token=key.stride(0), key_stride_head=key.stride(1),
+        value_stride_token=value.stride(0), value_stride_head=value.stride(1),
+        cache_stride_block=key_cache.stride(0), cache_stride_row=key_cache.stride(1),
+        cache_stride_head=key_cache.stride(2), num_blocks=nb, stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_kv_append(C.byref(a)), "kv_append")
+
+
+def swa_decode_attention(
+    q: torch.Tensor,
+    key_cache: torch.Tensor,
+    value_cache: torch.Tensor,
+    seq_lens: torch.Tensor,
+    *,
+    block_table: Optional[torch.Tensor] = None,
+    kv_start: Optional[torch.Tensor] = None,
+    row_seq: Optional[torch.Tensor] = None,
+    key_lo: Optional[torch.Tensor] = None,
+    kv_strides: Optional[Tuple[int, int, int]] = None,
+    block_size: Optional[int] = None,
+    num_kv_heads: Optional[int] = None,
+    window_left: int = -1,
+    scale: Optional[float] = None,
+    out: Optional[torch.Tensor] = None,
+    return_lse: bool = False,
+    max_seq_len: Optional[int] = None,
+    n_split: int = 0,
+):
+    """Single-query window attention for each row of q [R, Hq, D].
+
+    paged mode (block_table [S, max_blocks] int32): key_cache/value_cache are
+    [num_blocks, block_size, Hkv, D] and strides are taken from them.
+    dense mode (block_table None): key_cache/value_cache are any tensors whose element offset
+    for (sequence s, key i, head h) is (kv_start[s] + i)*kv_strides[1] + h*kv_strides[2];
+    kv_strides = (block, row, head) in elements and num_kv_heads must be given.
+    The query of row r sits at key index seq_lens[r]-1 of sequence row_seq[r] (default r) and sees
+    keys in [max(seq_lens[r]-1-window_left, key_lo[r]), seq_lens[r]-1].
+    max_seq_len (a host int bounding seq_lens) only sizes the split; it defaults to a bound
+    derived from the table/window shapes so that no device value is read back."""
+    dev = N.require_gpu(q, key_cache, value_cache, seq_lens, block_table, kv_start, row_seq, key_lo, out)
+    if q.dim() != 3:
+        raise ValueError(f"q must be [rows, num_heads, head_size], got {tuple(q.shape)}")
+    R, Hq, D = q.shape
+    _inner_contiguous(q, "q")
+    if key_cache.dtype != q.dtype or value_cache.dtype != q.dtype:
+        raise ValueError("q and the caches must share one dtype")
+    if block_table is not None:
+        if key_cache.dim() != 4 or value_cache.shape != key_cache.shape:
+            raise ValueError("paged caches must be [num_blocks, block_size, num_kv_heads, head_size]")
+        if key_cache.stride() != value_cache.stride():
+            raise ValueError("key_cache and value_cache must have identical strides")
+        _inner_contiguous(key_cache, "key_cache")
+        nb, bs, Hkv, Dc = key_cache.shape
+        kv_strides = (key_cache.stride(0), key_cache.stride(1), key_cache.stride(2))
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+            raise ValueError("block_table must be a 2-D int32 tensor with contiguous rows")
+        bt_stride = block_table.stride(0)
+        bound = block_table.shape[1] * bs
+    else:
+        if kv_strides is None or num_kv_heads is None:
+            raise ValueError("dense mode needs kv_strides and num_kv_heads")
+        Hkv, Dc, bs, bt_stride = num_kv_heads, D, 16, 0
+        if kv_start is not None and (kv_start.dtype != torch.int64 or not kv_start.is_contiguous()):
+            raise ValueError("kv_start must be a contiguous int64 tensor")
+        bound = max_seq_len if max_seq_len is not None else (window_left + 1 if window_left >= 0 else 1 << 20)
+    if Dc != D:
+        raise ValueError(f"head_size mismatch: q {D}, cache {Dc}")
+    for t, n in ((seq_lens, "seq_lens"), (row_seq, "row_seq"), (key_lo, "key_lo")):
+        if t is not None and (t.dtype != torch.int32 or t.dim() != 1 or not t.is_contiguous() or t.numel() < R):
+            raise ValueError(f"{n} must be a contiguous int32 vector with one entry per query row")
+    if scale is None:
+        scale = D ** -0.5
+    if out is None:
+        out = torch.empty((R, Hq, D), dtype=q.dtype, device=dev)
+    else:
+        if out.shape != q.shape or out.dtype != q.dtype:
+            raise ValueError("out must match q in shape and dtype")
+        _inner_contiguous(out, "out")
+    lse = torch.empty((R, Hq), dtype=torch.float32, device=dev) if return_lse else None
+    if max_seq_len is None:
+        max_seq_len = bound
+    if window_left >= 0:
+        max_seq_len = max(1, max_seq_len)
+    L = N.lib()
+    if n_split == 0:
+        n_split = L.sb_swa_decode_auto_split(R, Hkv, int(max_seq_len), int(window_left))
+    ws_bytes = L.sb_swa_decode_workspace_bytes(R, Hq, D, n_split)
+    ws = _workspace(dev, ws_bytes)
+    a = N.SwaDecodeArgs(
+        q=N.ptr(q), k_cache=N.ptr(key_cache), v_cache=N.ptr(value_cache), out=N.ptr(out), lse=N.ptr(lse),
+        block_table=N.ptr(block_table), kv_start=N.ptr(kv_start), row_seq=N.ptr(row_seq),
+        seq_lens=N.ptr(seq_lens), key_lo=N.ptr(key_lo),
+        workspace=N.ptr(ws), workspace_bytes=0 if ws is None else ws.numel(),
+        num_rows=R, num_q_heads=Hq, num_kv_heads=Hkv, head_size=D, block_size=bs,
+        window_left=int(window_left), max_seq_len=int(min(max_seq_len, 2**31 - 1)), n_split=int(n_split),
+        dtype=N.dtype_code(q.dtype), scale=float(scale),
+        q_stride_row=q.stride(0), q_stride_head=q.stride(1),
+        out_stride_row=out.stride(0), out_stride_head=out.stride(1),
+        kv_stride_block=kv_strides[0], kv_stride_row=kv_strides[1], kv_stride_head=kv_strides[2],
+        block_table_stride=bt_stride, stream=N.stream_ptr(dev))
+    N.check(L.sb_swa_decode(C.byref(a)), "swa_decode")
+    return (out, lse) if return_lse else out
+
+
+def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
+                  slot_idx: Optional[torch.Tensor] = None, scale: Optional[float] = None,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q, k, v, g [B, H, T, D] (any batch/head/time strides, contiguous D); state
+    [slots, H, D, D] fp32 or bf16, updated in place; returns o [B, H, T, D] in q's dtype.
+    Rows with slot_idx == -1 are skipped (state and output untouched)."""
+    dev = N.require_gpu(q, k, v, g, state, slot_idx, out)
+    if q.dim() != 4 or k.shape != q.shape or v.shape != q.shape or g.shape != q.shape:
+        raise ValueError(f"q, k, v, g must all be [B, H, T, D]; got {tuple(q.shape)}, {tuple(k.shape)}, "
+                         f"{tuple(v.shape)}, {tuple(g.shape)}")
+    B, H, T, D = q.shape
+    if not (k.dtype == q.dtype and v.dtype == q.dtype):
+        raise ValueError("q, k, v must share one dtype")
+    if state.dim() != 4 or state.shape[1:] != (H, D, D):
+        raise ValueError(f"state must be [slots, {H}, {D}, {D}], got {tuple(state.shape)}")
+    if state.stride(3) != 1 or state.stride(2) != D:
+        raise ValueError("each [dk, dv] state matrix must be contiguous")
+    for t, n in ((q, "q"), (k, "k"), (v, "v"), (g, "g")):
+        _inner_contiguous(t, n)
+    if slot_idx is not None:
+        if slot_idx.dtype != torch.int32 or slot_idx.dim() != 1 or slot_idx.numel() < B or not slot_idx.is_contiguous():
+            raise ValueError("slot_idx must be a contiguous int32 vector with one entry per batch row")
+    elif state.shape[0] < B:
+        raise ValueError(f"state has {state.shape[0]} slots for a batch of {B} and no slot_idx")
+    if scale is None:
+        scale = D ** -0.5
+    if out is None:
+        out = torch.empty((B, H, T, D), dtype=q.dtype, device=dev)
+    else:
+        if out.shape != q.shape or out.dtype != q.dtype:
+            raise ValueError("out must match q in shape and dtype")
+        _inner_contiguous(out, "out")
+    a = N.GlaRecurrentArgs(
+        q=N.ptr(q), k=N.ptr(k), v=N.ptr(v), g=N.ptr(g), state=N.ptr(state), out=N.ptr(out),
+        slot_idx=N.ptr(slot_idx), batch=B, num_heads=H, seq_len=T, head_dim=D,
+        dtype=N.dtype_code(q.dtype), g_dtype=N.dtype_code(g.dtype), state_dtype=N.dtype_code(state.dtype),
+        scale=float(scale),
+        q_stride_b=q.stride(0), q_stride_h=q.stride(1), q_stride_t=q.stride(2),
+        k_stride_b=k.stride(0), k_stride_h=k.stride(1), k_stride_t=k.stride(2),
+        v_stride_b=v.stride(0), v_stride_h=v.stride(1), v_stride_t=v.stride(2),
+        g_stride_b=g.stride(0), g_stride_h=g.stride(1), g_stride_t=g.stride(2),
+        out_stride_b=out.stride(0), out_stride_h=out.stride(1), out_stride_t=out.stride(2),
+        state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
+        num_slots=state.shape[0], stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
+    return out
+
+
+def copy_blocks(cache_half: torch.Tensor, pairs: torch.Tensor) -> None:
+    """cache_half [num_blocks, ...] with contiguous blocks; pairs [n, 2] int64 (src, dst) on the
+    same device. One half (K or V) per call, as ops.copy_blocks does per layer at
+    vllm_hymeta/attention/meta_attention.py:115-126."""
+    dev = N.require_gpu(cache_half, pairs)
+    if pairs.dtype != torch.int64 or pairs.dim() != 2 or pairs.shape[1] != 2:
+        raise ValueError("pairs must be an int64 [n, 2] tensor")
+    pairs = pairs.contiguous()
+    if not cache_half[0].is_contiguous():
+        raise ValueError("each cache block must be contiguous")
+    esz = cache_half.element_size()
+    N.check(N.lib().sb_copy_blocks(N.ptr(cache_half), N.ptr(pairs), pairs.shape[0],
+                                   cache_half[0].numel() * esz, cache_half.stride(0) * esz,
+                                   N.stream_ptr(dev)), "copy_blocks")
+
+
+def window_shift(src: Optional[torch.Tensor], dst: torch.Tensor, fresh: Optional[torch.Tensor], *, keep_rows: int,
+                 src_row0: int, dst_row0: int) -> None:
+    """dst[..., dst_row0 : dst_row0+keep_rows, :] = src[..., src_row0 : src_row0+keep_rows, :] and the
+    n rows of fresh behind them; src/dst are [B, H, cap, D] contiguous, fresh is [B, H, n, D]."""
+    dev = N.require_gpu(src, dst, fresh)
+    B, H, cap_d, D = dst.shape
+    if not dst.is_contiguous() or (src is not None and not src.is_contiguous()):
+        raise ValueError("window_shift needs contiguous [B, H, cap, D] storage")
+    esz = dst.element_size()
+    n_new = 0 if fresh is None else fresh.shape[2]
+    if fresh is not None:
+        if fresh.shape[:2] != (B, H) or fresh.shape[3] != D or fresh.dtype != dst.dtype or fresh.stride(3) != 1:
+            raise ValueError("fresh must be [B, H, n, D] of the cache dtype with contiguous rows")
+        if fresh.stride(0) != H * fresh.stride(1):
+            fresh = fresh.contiguous()
+    if dst_row0 + keep_rows + n_new > cap_d:
+        raise ValueError("window_shift would write past the destination capacity")
+    a = N.WindowShiftArgs(
+        src=N.ptr(src), dst=N.ptr(dst), fresh=N.ptr(fresh), planes=B * H, keep_rows=keep_rows,
+        src_row0=src_row0, dst_row0=dst_row0, n_new=n_new, row_bytes=D * esz,
+        src_stride_plane_bytes=0 if src is None else src.stride(1) * esz,
+        dst_stride_plane_bytes=dst.stride(1) * esz,
+        fresh_stride_plane_bytes=0 if fresh is None else fresh.stride(1) * esz,
+        fresh_stride_row_bytes=0 if fresh is None else fresh.stride(2) * esz,
+        stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_window_shift(C.byref(a)), "window_shift")

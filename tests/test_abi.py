@@ -1,0 +1,78 @@
+"""The C-ABI library loads and exports every symbol include/sbcache.h declares; argument
+rejection that happens before any HIP call works without a GPU."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sbcache.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sb_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_all_exported(sb):
+    names = declared_symbols()
+    assert "sb_kv_append" in names and "sb_swa_decode" in names and "sb_gla_recurrent" in names
+    lib = C.CDLL(sb._native.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/sbcache.h but not exported"
+    assert set(names) == set(sb._native.EXPORTS), "ctypes table and header disagree"
+
+
+def test_abi_version(sb):
+    assert sb._native.lib().sb_abi_version() == sb._native.ABI_VERSION
+
+
+def test_null_args_rejected(sb):
+    L = sb._native.lib()
+    assert L.sb_kv_append(None) == sb._native.SB_ERR_INVALID
+    assert b"null" in L.sb_last_error()
+    assert L.sb_swa_decode(None) == sb._native.SB_ERR_INVALID
+    assert L.sb_gla_recurrent(None) == sb._native.SB_ERR_INVALID
+    assert L.sb_window_shift(None) == sb._native.SB_ERR_INVALID
+
+
+def test_bad_shapes_rejected_before_launch(sb):
+    N = sb._native
+    L = N.lib()
+    a = N.SwaDecodeArgs(q=16, k_cache=16, v_cache=16, out=16, seq_lens=16, num_rows=1, num_q_heads=28,
+                        num_kv_heads=4, head_size=64, block_size=16, scale=1.0, dtype=0)
+    assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_UNSUPPORTED  # head_size 64 is not built
+    a.head_size = 128
+    a.num_q_heads = 27
+    assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_INVALID
+    a.num_q_heads = 28
+    a.scale = 0.0
+    assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_INVALID
+    a.scale = 1.0
+    a.block_table = 16
+    a.block_size = 24
+    assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_INVALID
+    a.block_size = 16
+    a.n_split = 4  # needs a workspace
+    assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_WORKSPACE
+    g = N.GlaRecurrentArgs(q=16, k=16, v=16, g=16, state=16, out=16, batch=1, num_heads=1, seq_len=1, head_dim=64)
+    assert L.sb_gla_recurrent(C.byref(g)) == N.SB_ERR_UNSUPPORTED
+
+
+def test_auto_split_and_workspace(sb):
+    L = sb._native.lib()
+    n = L.sb_swa_decode_auto_split(64, 4, 32768, 4096)
+    assert n == 8
+    assert L.sb_swa_decode_auto_split(4096, 4, 32768, 4096) == 1
+    assert L.sb_swa_decode_workspace_bytes(64, 28, 128, 1) == 0
+    need = L.sb_swa_decode_workspace_bytes(64, 28, 128, 8)
+    assert need >= 64 * 28 * 8 * 130 * 4
+
+
+def test_wrappers_refuse_cpu_tensors(sb):
+    import torch
+    k = torch.zeros(2, 4, 128, dtype=torch.bfloat16)
+    cache = torch.zeros(4, 16, 4, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        sb.ops.kv_append(k, k, cache, cache, torch.zeros(2, dtype=torch.int64))

@@ -1,0 +1,138 @@
+"""GLA recurrent kernel vs the float64 oracle. Tolerances (BASELINE): state 1e-4 relative to
+the largest state entry, output 2e-2 max-abs for bf16 q/k/v."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gla as G
+
+pytestmark = pytest.mark.gpu
+
+STATE_RTOL = 1e-4
+OUT_ATOL = 2e-2
+
+
+def make(B, H, T, D, seed, dtype=torch.bfloat16, relu=False):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(B, H, T, D, generator=g).to(dtype) for _ in range(3))
+    if relu:
+        q, k = q.relu(), k.relu()
+    gate = F.logsigmoid(torch.randn(B, H, T, D, generator=g)) / 16
+    return q, k, v, gate
+
+
+def rel(a, b):
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+@pytest.mark.parametrize("state_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,H,slots", [(5, 28, 9), (1, 4, 1), (64, 7, 64)])
+def test_decode_step_vs_oracle(sb, dev, state_dtype, B, H, slots):
+    D = 128
+    q, k, v, gate = make(B, H, 1, D, B * 31 + H)
+    g = torch.Generator().manual_seed(7)
+    state = (torch.randn(slots, H, D, D, generator=g) * 0.02).to(state_dtype)
+    slot_idx = torch.randperm(slots, generator=g)[:B].to(torch.int32)
+    if B > 2:
+        slot_idx[1] = -1
+    ref_state = state.double().numpy().copy()
+    ref_o = G.gla_step(q[:, :, 0].float().numpy(), k[:, :, 0].float().numpy(), v[:, :, 0].float().numpy(),
+                       gate[:, :, 0].numpy(), ref_state, slot_idx.tolist())
+    st = state.to(dev)
+    o = sb.my_fused_recurrent_gla(q.to(dev), k.to(dev), v.to(dev), gate.to(dev), st, slot_idx.to(dev))
+    torch.cuda.synchronize()
+    assert o.shape == (B, H, D) and o.dtype == q.dtype
+    got_state = st.double().cpu().numpy()
+    live = [b for b in range(B) if slot_idx[b] >= 0]
+    skipped_slots = sorted(set(range(slots)) - {int(slot_idx[b]) for b in live})
+    tol = STATE_RTOL if state_dtype == torch.float32 else 2 ** -8   # bf16 storage rounds to 8 bits
+    assert rel(got_state[[int(slot_idx[b]) for b in live]], ref_state[[int(slot_idx[b]) for b in live]]) <= tol
+    # untouched slots are bit-identical
+    assert np.array_equal(got_state[skipped_slots], state.double().numpy()[skipped_slots])
+    assert np.abs(o.float().cpu().numpy()[live] - ref_o[live]).max() <= OUT_ATOL
+    if B > 2:
+        assert (o[1] == 0).all()        # skipped row: output buffer left as allocated (zeros)
+
+
+def test_special_cases_on_device(sb, dev):
+    B, H, D = 2, 3, 128
+    q, k, v, gate = make(B, H, 1, D, 5, dtype=torch.float32)
+    S0 = torch.randn(B, H, D, D) * 0.1
+    # k = 0, g = 0 leaves the state bit-identical and o = scale * q S
+    st = S0.clone().to(dev)
+    o = sb.my_fused_recurrent_gla(q.to(dev), torch.zeros_like(k).to(dev), v.to(dev), torch.zeros_like(gate).to(dev), st, None, scale=0.5)
+    assert torch.equal(st.cpu(), S0)
+    np.testing.assert_allclose(o.cpu().numpy(), 0.5 * torch.einsum("bhk,bhkv->bhv", q[:, :, 0], S0).numpy(), rtol=1e-4, atol=1e-5)
+    # q = e_i / scale reads row i of the updated state exactly
+    e = torch.zeros(B, H, 1, D); e[..., 5] = 4.0
+    st = S0.clone().to(dev)
+    o = sb.my_fused_recurrent_gla(e.to(dev), k.to(dev), v.to(dev), gate.to(dev), st, None, scale=0.25)
+    assert torch.equal(o.cpu(), st.cpu()[:, :, 5, :])
+
+
+@pytest.mark.parametrize("T", [1, 2, 17])
+def test_multi_step_vs_oracle_and_layouts(sb, dev, T):
+    B, H, D = 3, 4, 128
+    q, k, v, gate = make(B, H, T, D, 11 + T, relu=True)
+    S0 = torch.randn(B, H, D, D) * 0.02
+    ref_o, ref_S = G.gla_recurrent(q.float().numpy(), k.float().numpy(), v.float().numpy(), gate.numpy(), S0.numpy())
+    # head-first views of token-major projections, as the HF layer produces them
+    qd, kd, vd, gd = (x.transpose(1, 2).contiguous().to(dev).transpose(1, 2) for x in (q, k, v, gate))
+    o, S = sb.fused_recurrent_gla(qd, kd, vd, gd, initial_state=S0.to(dev), output_final_state=True)
+    assert rel(S.double().cpu().numpy(), ref_S) <= STATE_RTOL
+    assert np.abs(o.float().cpu().numpy() - ref_o).max() <= OUT_ATOL
+    # stepping T times with T=1 gives the same state as one call with T steps (same fp32 op order)
+    st = S0.clone().to(dev)
+    for t in range(T):
+        sb.fused_recurrent_gla(qd[:, :, t:t + 1], kd[:, :, t:t + 1], vd[:, :, t:t + 1], gd[:, :, t:t + 1],
+                               initial_state=st, output_final_state=True, inplace_state=True)
+    assert torch.equal(st, S)
+    o2, S2 = sb.fused_recurrent_gla(qd, kd, vd, gd, initial_state=None, output_final_state=False)
+    assert S2 is None
+    ref_o0, _ = G.gla_recurrent(q.float().numpy(), k.float().numpy(), v.float().numpy(), gate.numpy(), None)
+    assert np.abs(o2.float().cpu().numpy() - ref_o0).max() <= OUT_ATOL
+
+
+def test_full_size_config3_properties(sb, dev):
+    """BASELINE config 3 (B=64, H=28, fp32 state): properties that need no CPU-sized oracle pass.
+    (1) a random sample of (b, h) pairs matches the oracle; (2) linearity of the state update in
+    (S, k): step(S1 + S2, k1 + k2) == step(S1, k1) + step(S2, k2) to fp32 rounding."""
+    B, H, D = 64, 28, 128
+    q, k, v, gate = make(B, H, 1, D, 3)
+    g = torch.Generator().manual_seed(9)
+    S = torch.randn(B, H, D, D, generator=g) * 0.02
+    st = S.clone().to(dev)
+    o = sb.my_fused_recurrent_gla(q.to(dev), k.to(dev), v.to(dev), gate.to(dev), st,
+                                  torch.arange(B, dtype=torch.int32, device=dev))
+    torch.cuda.synchronize()
+    pairs = [(0, 0), (63, 27), (17, 5), (40, 13)]
+    for b, h in pairs:
+        ref_S = S[b:b + 1, h:h + 1].double().numpy().copy()
+        ref_o = G.gla_step(q[b:b + 1, h:h + 1, 0].float().numpy(), k[b:b + 1, h:h + 1, 0].float().numpy(),
+                           v[b:b + 1, h:h + 1, 0].float().numpy(), gate[b:b + 1, h:h + 1, 0].numpy(), ref_S)
+        assert rel(st[b, h].double().cpu().numpy(), ref_S[0, 0]) <= STATE_RTOL
+        assert np.abs(o[b, h].float().cpu().numpy() - ref_o[0, 0]).max() <= OUT_ATOL
+    S2 = torch.randn(B, H, D, D, generator=g) * 0.02
+    k2 = torch.randn(B, H, 1, D, generator=g).bfloat16()
+    ksum = (k.float() + k2.float())
+    a = S.clone().to(dev); b_ = S2.clone().to(dev); c = (S + S2).to(dev)
+    qf, vf = q.float().to(dev), v.float().to(dev)
+    sb.my_fused_recurrent_gla(qf, k.float().to(dev), vf, gate.to(dev), a, None)
+    sb.my_fused_recurrent_gla(qf, k2.float().to(dev), vf, gate.to(dev), b_, None)
+    sb.my_fused_recurrent_gla(qf, ksum.to(dev), vf, gate.to(dev), c, None)
+    assert ((a + b_ - c).abs().max() / c.abs().max()).item() <= 1e-5
+
+
+def test_argument_errors(sb, dev):
+    q = torch.zeros(2, 4, 1, 128, device=dev, dtype=torch.bfloat16)
+    st = torch.zeros(2, 4, 128, 128, device=dev)
+    with pytest.raises(ValueError):
+        sb.ops.gla_recurrent(q, q[:, :2], q, q, st)
+    with pytest.raises(ValueError, match="state must be"):
+        sb.ops.gla_recurrent(q, q, q, q, st[:, :2])
+    with pytest.raises(NotImplementedError):
+        q64 = torch.zeros(2, 4, 1, 64, device=dev, dtype=torch.bfloat16)
+        sb.ops.gla_recurrent(q64, q64, q64, q64, torch.zeros(2, 4, 64, 64, device=dev))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        sb.ops.gla_recurrent(q.cpu(), q.cpu(), q.cpu(), q.cpu(), st.cpu())

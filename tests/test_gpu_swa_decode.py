@@ -1,0 +1,176 @@
+"""Window-bounded paged/dense single-query attention vs the float64 oracle.
+Tolerance (BASELINE): max-abs 2e-2 for bf16, 1e-5 for fp32, against fp32/fp64 mathematics."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as A
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3, torch.float32: 1e-5}
+
+
+def paged_problem(lens, bs, Hkv, D, dtype, seed, slack=5, resident_from=None):
+    """Random paged cache holding `lens[b]` keys per sequence in a seeded block permutation."""
+    g = torch.Generator().manual_seed(seed)
+    need = [(n + bs - 1) // bs for n in lens]
+    nb = sum(need) + slack
+    perm = torch.randperm(nb, generator=g)
+    kv = torch.randn(2, nb, bs, Hkv, D, generator=g).to(dtype)
+    tables = torch.zeros(len(lens), max(max(need), 1), dtype=torch.int32)
+    p = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[p:p + n]; p += n
+    return kv, tables
+
+
+def run_paged(sb, dev, q, kv, tables, lens, wl, scale, **kw):
+    return sb.ops.swa_decode_attention(q.to(dev), kv[0].to(dev), kv[1].to(dev),
+                                       torch.tensor(lens, dtype=torch.int32, device=dev),
+                                       block_table=tables.to(dev), window_left=wl, scale=scale, **kw)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("Hq,Hkv", [(28, 4), (8, 8), (8, 2), (16, 2)])
+@pytest.mark.parametrize("wl,n_split", [(64, 1), (64, 3), (37, 0), (-1, 2), (0, 1)])
+def test_paged_decode_vs_oracle(sb, dev, dtype, Hq, Hkv, wl, n_split):
+    D, bs = 128, 16
+    lens = [1, 15, 16, 17, 64, 65, 100, 129, 200]
+    kv, tables = paged_problem(lens, bs, Hkv, D, dtype, seed=Hq * 7 + (wl % 5))
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(len(lens), Hq, D, generator=g).to(dtype)
+    scale = D ** -0.5
+    out, lse = run_paged(sb, dev, q, kv, tables, lens, wl, scale, n_split=n_split, return_lse=True)
+    ref, ref_lse = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(),
+                                            tables.numpy(), lens, scale, wl, return_lse=True)
+    assert np.abs(out.float().cpu().numpy() - ref).max() <= TOL[dtype]
+    assert np.abs(lse.cpu().numpy() - ref_lse).max() <= 1e-3
+
+
+def test_block_size_64_and_large_scores(sb, dev):
+    # run_model_vllm.py uses block_size 64; scores up to ~|40| exercise the running-max rescale
+    D, bs, Hq, Hkv = 128, 64, 28, 4
+    lens = [300, 64, 5]
+    kv, tables = paged_problem(lens, bs, Hkv, D, torch.bfloat16, seed=3)
+    q = (torch.randn(3, Hq, D, generator=torch.Generator().manual_seed(1)) * 4).bfloat16()
+    out = run_paged(sb, dev, q, kv, tables, lens, 100, 1.0 / 3, n_split=2)
+    ref = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(),
+                                   tables.numpy(), lens, 1.0 / 3, 100)
+    assert np.abs(out.float().cpu().numpy() - ref).max() <= 2e-2
+
+
+def test_empty_rows_key_lo_and_row_seq(sb, dev):
+    """seq_len 0 and key_lo beyond the query give zeros; several query rows may share a sequence
+    (varlen decode): row r sees the first seq_lens[r] keys of sequence row_seq[r]."""
+    D, bs, Hq, Hkv, wl = 128, 16, 28, 4, 20
+    lens = [50, 33]
+    kv, tables = paged_problem(lens, bs, Hkv, D, torch.bfloat16, seed=5)
+    row_seq = [0, 0, 0, 1, 1, 0]
+    row_len = [48, 49, 50, 33, 0, 50]
+    key_lo = [0, 40, 0, 0, 0, 50]
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(len(row_seq), Hq, D, generator=g).bfloat16()
+    out, lse = sb.ops.swa_decode_attention(
+        q.to(dev), kv[0].to(dev), kv[1].to(dev), torch.tensor(row_len, dtype=torch.int32, device=dev),
+        block_table=tables.to(dev), row_seq=torch.tensor(row_seq, dtype=torch.int32, device=dev),
+        key_lo=torch.tensor(key_lo, dtype=torch.int32, device=dev), window_left=wl, n_split=2, return_lse=True)
+    out = out.float().cpu().numpy()
+    k_np, v_np = kv[0].float().numpy(), kv[1].float().numpy()
+    for r in range(len(row_seq)):
+        n, s = row_len[r], row_seq[r]
+        lo = max(max(0, n - 1 - wl), key_lo[r])
+        if n == 0 or lo >= n:
+            assert (out[r] == 0).all() and torch.isinf(lse[r]).all() and (lse[r] < 0).all()
+            continue
+        kk = A.gather_paged(k_np, tables[s].numpy(), n); vv = A.gather_paged(v_np, tables[s].numpy(), n)
+        masked = (np.arange(n) < lo)[None]
+        for h in range(Hq):
+            ref = A.masked_softmax_attention(q[r, h].float().numpy()[None], kk[:, h // 7], vv[:, h // 7], masked, D ** -0.5)
+            assert np.abs(out[r, h] - ref[0]).max() <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dense_mode_matches_paged_semantics(sb, dev, dtype):
+    """Dense [B, Hkv, cap, D] storage with a row window (the HF cache layout)."""
+    B, Hq, Hkv, D, cap, start, L, W = 3, 28, 4, 128, 96, 11, 70, 32
+    g = torch.Generator().manual_seed(6)
+    store_k = torch.randn(B, Hkv, cap, D, generator=g).to(dtype).to(dev)
+    store_v = torch.randn(B, Hkv, cap, D, generator=g).to(dtype).to(dev)
+    k, v = store_k[:, :, start:start + L], store_v[:, :, start:start + L]
+    q = torch.randn(B, Hq, D, generator=g).to(dtype)
+    kv_start = torch.arange(B, dtype=torch.int64, device=dev) * (Hkv * cap)
+    out = sb.ops.swa_decode_attention(
+        q.to(dev), k, v, torch.full((B,), L, dtype=torch.int32, device=dev), kv_start=kv_start,
+        kv_strides=(0, k.stride(2), k.stride(1)), num_kv_heads=Hkv, window_left=W - 1, max_seq_len=L)
+    ref = A.sdpa_window_attention(q.float().numpy()[:, :, None], k.float().cpu().numpy(), v.float().cpu().numpy(), W)
+    assert np.abs(out.float().cpu().numpy() - ref[:, :, 0]).max() <= TOL[dtype]
+
+
+def config2_problem(dev, B=64, seed=0):
+    """BASELINE config 2: B=64, 28q/4kv, D=128, bs=16, window_left=4096, ctx ~ U[1024, 32768],
+    only in-window blocks resident, seeded block permutation, bf16 N(0,1)."""
+    Hq, Hkv, D, bs, wl = 28, 4, 128, 16, 4096
+    g = torch.Generator().manual_seed(seed)
+    ctx = torch.randint(1024, 32769, (B,), generator=g)
+    pos = ctx                                   # position of the new token
+    lo_blk = torch.clamp((pos - wl) // bs, min=0)
+    hi_blk = pos // bs
+    nblk = (hi_blk - lo_blk + 1)
+    nb = int(nblk.sum() * 1.1) + 1
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(B, int(nblk.max()), dtype=torch.int32)
+    p = 0
+    for b in range(B):
+        tables[b, :nblk[b]] = perm[p:p + nblk[b]]; p += int(nblk[b])
+    seqlens = (pos + 1 - lo_blk * bs).to(torch.int32)
+    kv = torch.randn(2, nb, bs, Hkv, D, device=dev, dtype=torch.bfloat16)
+    q = torch.randn(B, Hq, D, device=dev, dtype=torch.bfloat16)
+    return dict(q=q, kv=kv, tables=tables.to(dev), seqlens=seqlens.to(dev), wl=wl, D=D, Hq=Hq, Hkv=Hkv, bs=bs)
+
+
+def test_config2_full_size_properties(sb, dev):
+    """Full BASELINE config 2 through size-independent properties plus a sampled oracle check."""
+    p = config2_problem(dev)
+    q, kv, tables, seqlens, wl = p["q"], p["kv"], p["tables"], p["seqlens"], p["wl"]
+    base = sb.ops.swa_decode_attention(q, kv[0], kv[1], seqlens, block_table=tables, window_left=wl)
+    # (1) the split count does not change the result beyond fp32 merge rounding
+    one = sb.ops.swa_decode_attention(q, kv[0], kv[1], seqlens, block_table=tables, window_left=wl, n_split=1)
+    many = sb.ops.swa_decode_attention(q, kv[0], kv[1], seqlens, block_table=tables, window_left=wl, n_split=16)
+    assert (base.float() - one.float()).abs().max() <= 4e-3 and (base.float() - many.float()).abs().max() <= 4e-3
+    # (2) relabelling physical blocks leaves the result bit-identical
+    nb = kv.shape[1]
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(1)).to(dev)
+    inv = torch.argsort(perm)
+    moved = sb.ops.swa_decode_attention(q, kv[0][perm], kv[1][perm], seqlens, block_table=inv[tables.long()].int(),
+                                        window_left=wl)
+    assert torch.equal(moved, base)
+    # (3) constant V gives that constant
+    const_v = torch.full_like(kv[1], 0.75)
+    out = sb.ops.swa_decode_attention(q, kv[0], const_v, seqlens, block_table=tables, window_left=wl)
+    assert (out.float() - 0.75).abs().max() <= 4e-3
+    # (4) a few sequences against the oracle (shortest, longest, first), on their own blocks only
+    sl = seqlens.cpu()
+    for b in sorted({0, int(sl.argmin()), int(sl.argmax())}):
+        n = int(sl[b])
+        nblk = (n + p["bs"] - 1) // p["bs"]
+        blocks = tables[b, :nblk].long()
+        kk, vv = kv[0][blocks].float().cpu().numpy(), kv[1][blocks].float().cpu().numpy()
+        ref = A.paged_decode_attention(q[b:b + 1].float().cpu().numpy(), kk, vv, np.arange(nblk)[None], [n],
+                                       p["D"] ** -0.5, wl)
+        assert np.abs(base[b:b + 1].float().cpu().numpy() - ref).max() <= 2e-2
+
+
+def test_argument_errors(sb, dev):
+    q = torch.zeros(2, 28, 128, device=dev, dtype=torch.bfloat16)
+    kv = torch.zeros(2, 4, 16, 4, 128, device=dev, dtype=torch.bfloat16)
+    sl = torch.ones(2, dtype=torch.int32, device=dev)
+    bt = torch.zeros(2, 1, dtype=torch.int32, device=dev)
+    with pytest.raises(ValueError, match="int32"):
+        sb.ops.swa_decode_attention(q, kv[0], kv[1], sl.long(), block_table=bt)
+    with pytest.raises(ValueError, match="share one dtype"):
+        sb.ops.swa_decode_attention(q.float(), kv[0], kv[1], sl, block_table=bt)
+    with pytest.raises(NotImplementedError, match="group size"):
+        sb.ops.swa_decode_attention(torch.zeros(2, 12, 128, device=dev, dtype=torch.bfloat16), kv[0], kv[1], sl, block_table=bt)
+    with pytest.raises(ValueError, match="dense mode"):
+        sb.ops.swa_decode_attention(q, kv[0], kv[1], sl)

@@ -1,0 +1,135 @@
+"""Pins oracle.attention against a library routine (torch SDPA) and against special cases the
+mathematics fixes."""
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from oracle import attention as A
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def test_mask_is_W_keys_including_self_bottom_right_aligned():
+    m = ~A.sliding_causal_mask(3, 7, 3)  # allowed
+    # queries sit at absolute positions 4, 5, 6; each sees itself and the two keys before it
+    assert [np.nonzero(r)[0].tolist() for r in m] == [[2, 3, 4], [3, 4, 5], [4, 5, 6]]
+    assert (~A.sliding_causal_mask(1, 5, 100))[0].all()          # window wider than the cache: all keys
+    assert (~A.sliding_causal_mask(4, 4, 1)).sum() == 4           # W=1: only self
+
+
+def test_repeat_kv_matches_repeat_interleave():
+    x = rng(0).standard_normal((2, 4, 5, 3))
+    np.testing.assert_array_equal(A.repeat_kv(x, 7), np.repeat(x, 7, axis=1))
+
+
+def test_sdpa_window_attention_vs_torch_sdpa_with_left_padding():
+    B, Hq, Hkv, Q, K, D, W = 3, 8, 2, 5, 11, 16, 4
+    r = rng(1)
+    q = r.standard_normal((B, Hq, Q, D)); k = r.standard_normal((B, Hkv, K, D)); v = r.standard_normal((B, Hkv, K, D))
+    am = np.ones((B, K + 2), np.int64); am[1, :5] = 0; am[2, :9] = 0      # left padding, row 2 pads into the queries
+    got = A.sdpa_window_attention(q, k, v, W, am)
+    kp = np.arange(K); qa = (K - Q) + np.arange(Q)
+    allowed = (kp[None] <= qa[:, None]) & (kp[None] > qa[:, None] - W)
+    mask = (~allowed)[None, None] | (am[:, -K:] == 0)[:, None, None, :]
+    add = torch.where(torch.from_numpy(mask), -torch.inf, 0.0).double()
+    ref = F.scaled_dot_product_attention(torch.from_numpy(q), torch.from_numpy(np.repeat(k, Hq // Hkv, 1)),
+                                         torch.from_numpy(np.repeat(v, Hq // Hkv, 1)), attn_mask=add)
+    ref = torch.nan_to_num(ref, nan=0.0).numpy()
+    np.testing.assert_allclose(got, ref, rtol=1e-10, atol=1e-12)
+    assert (got[2, :, :1] == 0).all() and (got[2, :, 1:] != 0).any()   # the pad query of row 2 is fully masked -> zeros
+
+
+def dense_reference(q, kk, vv, scale, window_left):
+    """torch SDPA on one sequence's gathered keys; q [Hq, D], kk/vv [n, Hkv, D]."""
+    n, Hkv, D = kk.shape
+    Hq = q.shape[0]
+    i = np.arange(n)
+    masked = i < (n - 1 - window_left) if window_left >= 0 else np.zeros(n, bool)
+    add = torch.where(torch.from_numpy(masked), -torch.inf, 0.0).double()[None, None, None, :]
+    kr = torch.from_numpy(np.repeat(kk.transpose(1, 0, 2), Hq // Hkv, 0))[None]
+    vr = torch.from_numpy(np.repeat(vv.transpose(1, 0, 2), Hq // Hkv, 0))[None]
+    return F.scaled_dot_product_attention(torch.from_numpy(q)[None, :, None, :], kr, vr, attn_mask=add,
+                                          scale=scale)[0, :, 0].numpy()
+
+
+def make_paged(B, lens, bs, Hkv, D, seed, nb_extra=5):
+    r = rng(seed)
+    need = [(n + bs - 1) // bs for n in lens]
+    nb = sum(need) + nb_extra
+    perm = r.permutation(nb)
+    kc = r.standard_normal((nb, bs, Hkv, D)); vc = r.standard_normal((nb, bs, Hkv, D))
+    tables = np.zeros((B, max(need)), np.int32)
+    p = 0
+    for b in range(B):
+        tables[b, :need[b]] = perm[p:p + need[b]]; p += need[b]
+    return kc, vc, tables
+
+
+def test_paged_decode_vs_torch_sdpa_on_gathered_keys():
+    B, Hq, Hkv, D, bs, wl = 4, 14, 2, 16, 16, 20
+    lens = [1, 17, 48, 50]
+    kc, vc, tables = make_paged(B, lens, bs, Hkv, D, 2)
+    q = rng(3).standard_normal((B, Hq, D))
+    out, lse = A.paged_decode_attention(q, kc, vc, tables, lens, 0.3, wl, return_lse=True)
+    for b, n in enumerate(lens):
+        kk = np.concatenate([kc[t] for t in tables[b]])[:n]   # independent gather: concatenate blocks in order
+        vv = np.concatenate([vc[t] for t in tables[b]])[:n]
+        np.testing.assert_allclose(out[b], dense_reference(q[b], kk, vv, 0.3, wl), rtol=1e-10, atol=1e-12)
+        lo = max(0, n - 1 - wl)
+        s = np.einsum("hd,nhd->hn", q[b].reshape(Hkv, -1, D).reshape(Hq, D), np.repeat(kk, Hq // Hkv, 1))[:, lo:] * 0.3
+        np.testing.assert_allclose(lse[b], np.log(np.exp(s).sum(1)), rtol=1e-10)
+
+
+def test_paged_decode_special_cases_and_invariants():
+    B, Hq, Hkv, D, bs = 2, 4, 2, 8, 16
+    lens = [40, 33]
+    kc, vc, tables = make_paged(B, lens, bs, Hkv, D, 4)
+    q = rng(5).standard_normal((B, Hq, D))
+    # window_left = 0: only the newest key is visible -> output is exactly that V row
+    out = A.paged_decode_attention(q, kc, vc, tables, lens, 1.0, 0)
+    for b, n in enumerate(lens):
+        vrow = vc[tables[b, (n - 1) // bs], (n - 1) % bs]
+        np.testing.assert_allclose(out[b], np.repeat(vrow, Hq // Hkv, 0), rtol=1e-12)
+    # constant V -> constant output whatever the scores
+    vconst = np.full_like(vc, 2.5)
+    np.testing.assert_allclose(A.paged_decode_attention(q, kc, vconst, tables, lens, 1.0, 12), 2.5, rtol=1e-12)
+    # relabelling physical blocks (permute cache rows, rewrite the table) changes nothing
+    nb = kc.shape[0]
+    perm = rng(6).permutation(nb)
+    inv = np.argsort(perm)
+    base = A.paged_decode_attention(q, kc, vc, tables, lens, 0.5, 12)
+    moved = A.paged_decode_attention(q, kc[perm], vc[perm], inv[tables].astype(np.int32), lens, 0.5, 12)
+    np.testing.assert_allclose(moved, base, rtol=1e-12)
+    # a wider window never loses keys: window >= n equals unbounded
+    np.testing.assert_allclose(A.paged_decode_attention(q, kc, vc, tables, lens, 0.5, 1000),
+                               A.paged_decode_attention(q, kc, vc, tables, lens, 0.5, -1), rtol=1e-12)
+
+
+def test_varlen_vs_torch_sdpa_and_decode_consistency():
+    Hq, Hkv, D, wl = 4, 2, 8, 5
+    cu_q = [0, 6, 6, 9]; cu_k = [0, 6, 10, 21]          # seq0: plain prompt; seq1: no queries; seq2: 3 new of 11
+    r = rng(7)
+    q = r.standard_normal((9, Hq, D)); k = r.standard_normal((21, Hkv, D)); v = r.standard_normal((21, Hkv, D))
+    out = A.varlen_window_attention(q, k, v, cu_q, cu_k, 0.4, wl)
+    for s in range(3):
+        Lq, Lk = cu_q[s + 1] - cu_q[s], cu_k[s + 1] - cu_k[s]
+        for j in range(Lq):
+            n = Lk - Lq + j + 1                            # this query as a decode over the first n keys
+            ref = dense_reference(q[cu_q[s] + j], k[cu_k[s]:cu_k[s] + n], v[cu_k[s]:cu_k[s] + n], 0.4, wl)
+            np.testing.assert_allclose(out[cu_q[s] + j], ref, rtol=1e-10, atol=1e-12)
+
+
+def test_lse_merge_equals_attention_over_union():
+    D, nA, nB = 8, 5, 7
+    r = rng(8)
+    q = r.standard_normal((3, D)); kA = r.standard_normal((nA, D)); vA = r.standard_normal((nA, D))
+    kB = r.standard_normal((nB, D)); vB = r.standard_normal((nB, D))
+    none = np.zeros((1, 1), bool)
+    oA, lA = A.masked_softmax_attention(q, kA, vA, none, 0.5, return_lse=True)
+    oB, lB = A.masked_softmax_attention(q, kB, vB, none, 0.5, return_lse=True)
+    oU, lU = A.masked_softmax_attention(q, np.concatenate([kA, kB]), np.concatenate([vA, vB]), none, 0.5, return_lse=True)
+    o, l = A.lse_merge(oA, lA, oB, lB)
+    np.testing.assert_allclose(o, oU, rtol=1e-10)
+    np.testing.assert_allclose(l, lU, rtol=1e-10)

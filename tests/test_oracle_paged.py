@@ -1,0 +1,146 @@
+"""Pins oracle.paged (append, slot mapping, the window block-manager model) by brute force, then
+checks the product's vectorised WindowBlockManager against that model bit for bit."""
+import numpy as np
+import pytest
+
+from oracle import paged as P
+
+
+def test_kv_append_closed_form_and_sentinels():
+    r = np.random.default_rng(0)
+    nb, bs, H, D, T = 6, 16, 2, 4, 9
+    kc = np.full((nb, bs, H, D), -7.0); vc = np.full((nb, bs, H, D), -9.0)
+    key = r.standard_normal((T, H, D)); val = r.standard_normal((T, H, D))
+    slots = [5, 16, -1, 95, 0, 17, -1, 40, 41]
+    P.kv_append(key, val, kc, vc, slots)
+    flat_k = kc.reshape(nb * bs, H, D); flat_v = vc.reshape(nb * bs, H, D)
+    written = [s for s in slots if s >= 0]
+    for t, s in enumerate(slots):
+        if s >= 0:
+            assert np.array_equal(flat_k[s], key[t]) and np.array_equal(flat_v[s], val[t])
+    untouched = np.setdiff1d(np.arange(nb * bs), written)
+    assert (flat_k[untouched] == -7.0).all() and (flat_v[untouched] == -9.0).all()
+
+
+def test_slot_mapping_functions():
+    assert P.compute_slot_mapping_start_idx(True, 100, 0, 32) == 68
+    assert P.compute_slot_mapping_start_idx(True, 10, 0, 32) == 0
+    assert P.compute_slot_mapping_start_idx(False, 1, 500, 32) == 0      # decode: never skipped
+    assert P.compute_slot_mapping_start_idx(True, 100, 0, None) == 0
+    bt = {7: [9, 3, 5]}
+    out = []
+    P.compute_slot_mapping(False, out, 7, 40, 0, 20, 16, bt)             # tokens 0..19 PAD, 20..39 mapped
+    assert out[:20] == [-1] * 20
+    assert out[20:] == [bt[7][i // 16] * 16 + i % 16 for i in range(20, 40)]
+    out = []
+    P.compute_slot_mapping(False, out, 7, 41, 40, 0, 16, bt)             # one decode token at position 40
+    assert out == [5 * 16 + 8]
+    out = []
+    P.compute_slot_mapping(True, out, 7, 5, 0, 0, 16, bt)                # profile run: all PAD
+    assert out == [-1] * 5
+
+
+@pytest.mark.parametrize("bs,wl", [(16, 32), (16, 40), (32, 64), (16, 0)])
+def test_model_residency_invariant_brute_force(bs, wl):
+    """After every token: every position a query at the newest position may see is resident, at
+    the slot the closed form gives, and nothing older than one block before the window is kept."""
+    m = P.WindowCacheModel(64, bs, wl)
+    m.add_seq(0)
+    where = {}                                   # absolute position -> slot, filled from returned slots
+    prompt = 3 * wl // 2 + 7
+    slots = m.append_tokens(0, prompt, True)
+    assert slots[:max(0, prompt - wl)] == [-1] * max(0, prompt - wl)
+    for i, s in enumerate(slots):
+        if s >= 0:
+            where[i] = s
+    n = prompt
+    for step in range(5 * bs + 3):
+        (s,) = m.append_tokens(0, 1, False)
+        where[n] = s
+        n += 1
+        table, seqlen, first = m.view(0)
+        p = n - 1
+        assert first % bs == 0 and seqlen == n - first
+        for pos in range(max(0, p - wl), p + 1):                         # the whole window is resident ...
+            k = pos - first
+            assert k >= 0
+            assert table[k // bs] * bs + k % bs == where[pos]            # ... at the slot it was written to
+        assert first >= max(0, (p - wl) // bs * bs - 0)                  # and no whole block before the window stays
+        assert first <= max(0, p - wl)
+        live = set(table)
+        assert len(live) == len(table) and not live & set(m.free)        # no block both resident and free
+    assert len(m.free) + len(m.view(0)[0]) == 64                         # nothing leaked
+
+
+def test_model_recycles_own_block_when_window_is_block_aligned():
+    m = P.WindowCacheModel(32, 16, 64)
+    m.add_seq("a")
+    m.append_tokens("a", 64, True)
+    used = set()
+    for _ in range(200):
+        m.append_tokens("a", 1, False)
+        used |= set(m.view("a")[0])
+    assert len(used) == 64 // 16 + 1                                     # a fixed ring of wl/bs + 1 blocks
+
+
+def run_schedule(mgr, model, seed, n_seqs, steps, bs, wl):
+    r = np.random.default_rng(seed)
+    live = []
+    next_id = 0
+    for step in range(steps):
+        if len(live) < n_seqs and r.random() < 0.3:                      # a new prompt arrives
+            sid = next_id; next_id += 1
+            mgr.add_seq(sid); model.add_seq(sid)
+            L = int(r.integers(1, 3 * wl + 5))
+            chunks = [L] if r.random() < 0.5 else [L // 2, L - L // 2]
+            for c in chunks:
+                if c:
+                    assert mgr.append_tokens(sid, c, True) == model.append_tokens(sid, c, True)
+            live.append(sid)
+        if live and r.random() < 0.1:
+            sid = live.pop(int(r.integers(len(live))))
+            mgr.free_seq(sid); model.free_seq(sid)
+        if live:
+            order = list(r.permutation(live))
+            got = mgr.decode_step(order)
+            exp = [model.append_tokens(s, 1, False)[0] for s in order]
+            assert got.tolist() == exp
+            tables, seqlens, first = mgr.kernel_view(order)
+            for i, s in enumerate(order):
+                t, n, f = model.view(s)
+                assert tables[i, :len(t)].tolist() == t and (tables[i, len(t):] == 0).all()
+                assert int(seqlens[i]) == n and int(first[i]) == f
+        assert mgr.free_stack() == model.free
+
+
+@pytest.mark.parametrize("seed,bs,wl", [(0, 16, 32), (1, 16, 48), (2, 32, 64), (3, 16, 40)])
+def test_product_block_manager_matches_model(sb, seed, bs, wl):
+    nb = 256
+    mgr = sb.WindowBlockManager(nb, bs, wl, max_seqs=6, max_chunk_tokens=3 * wl + 5)
+    model = P.WindowCacheModel(nb, bs, wl)
+    run_schedule(mgr, model, seed, n_seqs=6, steps=120, bs=bs, wl=wl)
+
+
+def test_product_slot_mapping_functions_match(sb):
+    for args in [(True, 100, 0, 32), (True, 10, 0, 32), (False, 1, 500, 32), (True, 9, 4, None)]:
+        assert sb.compute_slot_mapping_start_idx(*args) == P.compute_slot_mapping_start_idx(*args)
+    bt = {0: list(range(50, 60))}
+    for seq_len, ctx, start in [(40, 0, 20), (41, 40, 0), (100, 30, 50), (17, 16, 0)]:
+        a, b = [], []
+        sb.compute_slot_mapping(False, a, 0, seq_len, ctx, start, 16, bt)
+        P.compute_slot_mapping(False, b, 0, seq_len, ctx, start, 16, bt)
+        assert a == b
+    a = []
+    sb.compute_slot_mapping(True, a, 0, 5, 0, 0, 16, bt)
+    assert a == [-1] * 5
+
+
+def test_block_manager_errors(sb):
+    with pytest.raises(ValueError, match="multiple of 16"):
+        sb.WindowBlockManager(8, 24, 32, max_seqs=1)
+    m = sb.WindowBlockManager(2, 16, 64, max_seqs=1, max_chunk_tokens=64)
+    m.add_seq(0)
+    with pytest.raises(RuntimeError, match="out of KV cache blocks"):
+        m.append_tokens(0, 64, True)
+    with pytest.raises(KeyError):
+        m.add_seq(0)
