@@ -1,0 +1,201 @@
+"""Benchmark of the decode-time cache hot path on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input at BASELINE config 2
+(paged SWA decode at the 7B layer shape): KV append of one new token per sequence through
+slot_mapping, then window-bounded paged decode attention (split kernel + merge kernel).
+  B=64, 28 q / 4 kv heads, head_dim 128, block_size 16, window_left 4096, bf16,
+  context lengths ~ U[1024, 32768] (seed 0), seeded block permutation, only in-window blocks
+  resident, K/V ~ N(0,1).
+`value` is algorithmic bytes of a step / wall time of a step, inputs resident in HBM.
+Between steps the bench rotates over several copies of the KV cache whose total size exceeds
+the 256 MB on-die cache, so every step reads its K/V from HBM.
+
+Prints ONE JSON line (rank 0 is the only rank: this build is single-GPU).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+HQ, HKV, D, BS, WL = 28, 4, 128, 16, 4096
+E = 2  # bf16
+
+
+def build_config2(dev, B=64, seed=0, copies=3):
+    g = torch.Generator().manual_seed(seed)
+    ctx = torch.randint(1024, 32769, (B,), generator=g)          # tokens already cached
+    pos = ctx                                                    # position of the new token
+    lo_blk = torch.clamp((pos - WL) // BS, min=0)
+    hi_blk = pos // BS
+    nblk = hi_blk - lo_blk + 1
+    nb = int(int(nblk.sum()) * 1.1) + 1
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(B, int(nblk.max()), dtype=torch.int32)
+    p = 0
+    for b in range(B):
+        tables[b, :nblk[b]] = perm[p:p + int(nblk[b])]
+        p += int(nblk[b])
+    seqlens = (pos + 1 - lo_blk * BS).to(torch.int32)            # view-relative length incl. the new token
+    k_idx = pos - lo_blk * BS                                    # view-relative index of the new token
+    slots = tables[torch.arange(B), (k_idx // BS).long()].to(torch.int64) * BS + k_idx % BS
+    n_keys = torch.minimum(pos + 1, torch.tensor(WL + 1))        # keys each query attends to
+    kv = [torch.randn(2, nb, BS, HKV, D, device=dev, dtype=torch.bfloat16) for _ in range(copies)]
+    prob = dict(
+        B=B, nb=nb, kv=kv, tables=tables.to(dev), seqlens=seqlens.to(dev), slots=slots.to(dev),
+        q=torch.randn(B, HQ, D, device=dev, dtype=torch.bfloat16),
+        k=torch.randn(B, HKV, D, device=dev, dtype=torch.bfloat16),
+        v=torch.randn(B, HKV, D, device=dev, dtype=torch.bfloat16),
+        out=torch.empty(B, HQ, D, device=dev, dtype=torch.bfloat16),
+        n_keys=n_keys, max_seq_len=int(seqlens.max()), resident_blocks=int(nblk.sum()))
+    # algorithmic bytes of one layer-step (formula of the measurement plan):
+    kv_read = int(n_keys.sum()) * HKV * D * 2 * E               # K and V rows inside the window
+    qo = 2 * B * HQ * D * E                                      # q read, o write
+    new_kv = 2 * B * HKV * D * E * 2                             # new k,v read + written to the cache
+    tables_b = int(nblk.sum()) * 4 + B * (8 + 4)                 # block ids, slot, seq_len
+    prob["bytes_step"] = kv_read + qo + new_kv + tables_b
+    prob["bytes_split_kernel"] = kv_read + qo + int(nblk.sum()) * 4 + B * 4
+    return prob
+
+
+def cpu_baseline(seconds_budget=12.0, sample_B=8):
+    """The reference's PyTorch CPU path (oracle/cpu_path.py, a port) on a bounded sample of the
+    same workload: sample_B sequences, window-saturated dense fp32 caches [B, 4, 4097, 128], one
+    decode token: roll + slice-assign update, repeat_kv, SDPA with the sliding-causal mask."""
+    from oracle import cpu_path
+
+    threads = torch.get_num_threads()
+    g = torch.Generator().manual_seed(0)
+    W = WL + 1
+    k_state = torch.randn(sample_B, HKV, W, D, generator=g)
+    v_state = torch.randn(sample_B, HKV, W, D, generator=g)
+    q = torch.randn(sample_B, HQ, 1, D, generator=g)
+    k_new = torch.randn(sample_B, HKV, 1, D, generator=g)
+    v_new = torch.randn(sample_B, HKV, 1, D, generator=g)
+    times = []
+    t_end = time.perf_counter() + seconds_budget
+    it = 0
+    while it < 3 or (time.perf_counter() < t_end and it < 200):
+        t0 = time.perf_counter()
+        k_state, v_state = cpu_path.dense_window_update(k_state, v_state, k_new, v_new, W)
+        cpu_path.sdpa_window_attention(q, k_state, v_state, W)
+        dt = time.perf_counter() - t0
+        if it >= 2:
+            times.append(dt)
+        it += 1
+    med = statistics.median(times)
+    # same algorithmic-byte formula as the GPU line (bf16 element size) so the unit is comparable
+    bytes_sample = sample_B * (W * HKV * D * 2 * E + 2 * HQ * D * E + 2 * HKV * D * E * 2 + (W // BS + 1) * 4 + 12)
+    return dict(value=bytes_sample / med / 1e9, unit="GB/s", cores=threads, kind="port",
+                sample=f"{sample_B} of 64 sequences, window-saturated (4097 keys), fp32 dense cache, "
+                       f"cache.py roll update + repeat_kv + SDPA, median of {len(times)} steps, "
+                       f"{med * 1e3:.1f} ms/step")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--n-split", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import __graft_entry__ as entry
+    sb = entry.load_package()
+    sb._native.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    prob = build_config2(dev)
+    kv, n_copies = prob["kv"], len(prob["kv"])
+
+    def step(i, phases=0, append=True):
+        c = kv[i % n_copies]
+        if append:
+            sb.ops.kv_append(prob["k"], prob["v"], c[0], c[1], prob["slots"])
+        sb.ops.swa_decode_attention(prob["q"], c[0], c[1], prob["seqlens"], block_table=prob["tables"],
+                                    window_left=WL, out=prob["out"], max_seq_len=prob["max_seq_len"],
+                                    n_split=args.n_split, phases=phases)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    value = prob["bytes_step"] / (wall / args.steps) / 1e9
+
+    # dominant kernel alone (split kernel), HIP events on the launch stream, one pair per launch
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for i in range(args.steps):
+        evs[i][0].record()
+        step(i, phases=1, append=False)
+        evs[i][1].record()
+    torch.cuda.synchronize()
+    k_ms = statistics.mean(a.elapsed_time(b) for a, b in evs)
+    achieved = prob["bytes_split_kernel"] / (k_ms * 1e-3) / 1e9
+
+    n_split = args.n_split or sb._native.lib().sb_swa_decode_auto_split(prob["B"], HKV, prob["max_seq_len"], WL)
+    line = {
+        "metric": "SWA decode-attn+append GB/s (% of HBM peak) and decode tok/s, 7B shapes, 1 GPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: paged SWA decode, one layer-step (KV append + window attention)",
+                   "batch": prob["B"], "q_heads": HQ, "kv_heads": HKV, "head_dim": D, "block_size": BS,
+                   "window_left": WL, "context_lens": "U[1024,32768] seed 0", "n_split": int(n_split),
+                   "kv_cache_copies_rotated": n_copies, "bytes_per_step": prob["bytes_step"]},
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "decode_tok_per_s_layer_step": round(prob["B"] / (wall / args.steps), 1),
+        "roofline": {"bound": "hbm", "kernel": "swa_decode_split_kernel<BF16,7>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "kernel_ms": round(k_ms, 4), "bytes_per_launch": prob["bytes_split_kernel"]},
+    }
+
+    if args.extras:
+        B3, H3 = 64, 28
+        g = torch.Generator().manual_seed(0)
+        states = [(torch.randn(B3, H3, D, D, generator=g) * 0.02).to(dev) for _ in range(3)]
+        q3, k3, v3 = (torch.randn(B3, H3, 1, D, generator=g).bfloat16().to(dev) for _ in range(3))
+        g3 = (torch.nn.functional.logsigmoid(torch.randn(B3, H3, 1, D, generator=g)) / 16).to(dev)
+        o3 = torch.empty(B3, H3, 1, D, dtype=torch.bfloat16, device=dev)
+        for i in range(10):
+            sb.ops.gla_recurrent(q3, k3, v3, g3, states[i % 3], None, None, o3)
+        ev3 = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(100)]
+        for i, (a, b) in enumerate(ev3):
+            a.record()
+            sb.ops.gla_recurrent(q3, k3, v3, g3, states[i % 3], None, None, o3)
+            b.record()
+        torch.cuda.synchronize()
+        ms3 = statistics.mean(a.elapsed_time(b) for a, b in ev3)
+        bytes3 = 2 * B3 * H3 * D * D * 4 + B3 * H3 * (3 * D * 2 + D * 4 + D * 2)
+        line["gla_state_update"] = {"workload": "BASELINE config 3: B=64, H=28, fp32 state", "kernel_ms": round(ms3, 4),
+                                    "GBps": round(bytes3 / (ms3 * 1e-3) / 1e9, 1),
+                                    "frac_hbm_peak": round(bytes3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

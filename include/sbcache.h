@@ -123,6 +123,8 @@ typedef struct sb_swa_decode_args {
   int32_t max_seq_len; /* upper bound of seq_lens (host knowledge); sizes the split */
   int32_t n_split;     /* 0 = auto */
   int32_t dtype;
+  int32_t phases;      /* 0 = split then merge; 1 = split kernel only; 2 = merge kernel only
+                          (1 and 2 exist so a profiler can time the two kernels apart) */
   float scale;
   int64_t q_stride_row, q_stride_head;
   int64_t out_stride_row, out_stride_head;

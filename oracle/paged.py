@@ -67,8 +67,9 @@ class WindowCacheModel:
                   any query of this call can still see is evicted, so attention for the call
                   may read the cache after the append;
       2. store    token i is stored iff i >= start_idx (compute_slot_mapping_start_idx: for a
-                  prompt, tokens older than query_len - wl are never cached,
-                  meta_attention.py:489-494); a stored token whose logical block i // bs has
+                  prompt attended over its in-flight K/V, tokens older than query_len - wl are
+                  never cached, meta_attention.py:489-494; a chunked-prefill prompt, whose
+                  queries read the paged cache, stores all); a stored token whose logical block i // bs has
                   no physical id pops the top of the free stack;
       3. slot     phys[i // bs] * bs + i % bs, PAD_SLOT_ID when not stored;
       4. view     block_table = phys[lo_res..hi] with lo_res the lowest resident logical block;
@@ -89,14 +90,15 @@ class WindowCacheModel:
         for j in sorted(s["phys"]):
             self.free.append(s["phys"][j])
 
-    def append_tokens(self, seq_id: int, count: int, is_prompt: bool) -> List[int]:
-        """Slots for `count` new tokens of one sequence (a prompt chunk or one decode token)."""
+    def append_tokens(self, seq_id: int, count: int, is_prompt: bool, store_all: bool = False) -> List[int]:
+        """Slots for `count` new tokens of one sequence (a prompt chunk or one decode token).
+        store_all: a prompt chunk whose attention reads the paged cache keeps every token."""
         s = self.seqs[seq_id]
         p0 = s["n"]
         lo_new = max(0, (p0 - self.wl) // self.bs)
         for j in sorted(j for j in s["phys"] if j < lo_new):
             self.free.append(s["phys"].pop(j))
-        start_idx = compute_slot_mapping_start_idx(is_prompt, count, p0, self.wl)
+        start_idx = compute_slot_mapping_start_idx(is_prompt, count, p0, None if store_all else self.wl)
         slots = []
         for i in range(p0, p0 + count):
             if i < start_idx:

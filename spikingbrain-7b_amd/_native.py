@@ -43,7 +43,7 @@ class SwaDecodeArgs(C.Structure):
         ("num_rows", i64),
         ("num_q_heads", i32), ("num_kv_heads", i32), ("head_size", i32), ("block_size", i32),
         ("window_left", i32), ("max_seq_len", i32), ("n_split", i32), ("dtype", i32),
-        ("scale", f32),
+        ("phases", i32), ("scale", f32),
         ("q_stride_row", i64), ("q_stride_head", i64),
         ("out_stride_row", i64), ("out_stride_head", i64),
         ("kv_stride_block", i64), ("kv_stride_row", i64), ("kv_stride_head", i64),

@@ -16,7 +16,10 @@ Policy of this manager (its own specification, deterministic):
     stack; then allocate, in position order, a block for every stored token whose logical
     block has none. With window_left a multiple of block_size a decoding sequence therefore
     recycles its own oldest block: a fixed ring of window_left/block_size + 1 blocks;
-  * a prompt stores only tokens i >= query_len - window_left (older ones get PAD_SLOT_ID).
+  * a prompt whose attention runs over the in-flight K/V stores only tokens
+    i >= query_len - window_left (older ones get PAD_SLOT_ID); a prompt chunk whose attention
+    reads the paged cache (chunked prefill) stores every token, because its own queries read
+    them back.
 Per-sequence tables are rings indexed by logical block modulo the ring size, so a step costs
 O(events) Python work plus vectorised numpy, independent of the context length.
 """
@@ -131,7 +134,7 @@ class WindowBlockManager:
         return int(self._stack[self._top])
 
     # -- one engine step ------------------------------------------------------------
-    def _advance_row(self, r: int, count: int, is_prompt: bool) -> Tuple[int, int]:
+    def _advance_row(self, r: int, count: int, is_prompt: bool, store_all: bool = False) -> Tuple[int, int]:
         """Evict + allocate for `count` new tokens of row r; returns (p0, first stored position)."""
         bs, wl, R = self.block_size, self.window_left, self.ring_blocks
         p0 = int(self.n_tokens[r])
@@ -143,7 +146,7 @@ class WindowBlockManager:
             lo = max(lo, lo_new)
             if lo > hi:  # everything evicted
                 lo, hi = 0, -1
-        start_idx = compute_slot_mapping_start_idx(is_prompt, count, p0, wl)
+        start_idx = compute_slot_mapping_start_idx(is_prompt, count, p0, None if store_all else wl)
         first = max(p0, start_idx)
         end = p0 + count
         if end > first:
@@ -159,10 +162,11 @@ class WindowBlockManager:
         self.n_tokens[r] = end
         return p0, first
 
-    def append_tokens(self, seq_id, count: int, is_prompt: bool) -> List[int]:
-        """Slots of `count` new tokens of one sequence (one prompt chunk or one decode token)."""
+    def append_tokens(self, seq_id, count: int, is_prompt: bool, store_all: bool = False) -> List[int]:
+        """Slots of `count` new tokens of one sequence (one prompt chunk or one decode token).
+        store_all=True keeps every prompt token (chunked prefill through the paged cache)."""
         r = self._rows[seq_id]
-        p0, first = self._advance_row(r, count, is_prompt)
+        p0, first = self._advance_row(r, count, is_prompt, store_all)
         slots: List[int] = []
         compute_slot_mapping(False, slots, r, p0 + count, p0, first, self.block_size, {r: LogicalTable(self, r)})
         return slots

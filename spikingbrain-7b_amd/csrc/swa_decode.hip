@@ -435,14 +435,17 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   const int G = a->num_q_heads / a->num_kv_heads;
   const dim3 grid((unsigned)a->num_rows, (unsigned)a->num_kv_heads, (unsigned)n_split);
   hipStream_t st = (hipStream_t)a->stream;
-  int rc;
-  if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
-  else if (a->dtype == SB_F16) rc = launch_for_group<F16>(G, grid, st, p);
-  else rc = launch_for_group<F32>(G, grid, st, p);
-  if (rc != 0)
+  int rc = 0;
+  if (a->phases < 0 || a->phases > 2) return fail(SB_ERR_INVALID, "sb_swa_decode: phases must be 0, 1 or 2");
+  if (G != 1 && G != 2 && G != 4 && G != 7 && G != 8)
     return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: GQA group size %d (built: 1, 2, 4, 7, 8)", G);
-  rc = check_launch("swa_decode_split_kernel");
-  if (rc != SB_OK || n_split == 1) return rc;
+  if (a->phases != 2) {
+    if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
+    else if (a->dtype == SB_F16) rc = launch_for_group<F16>(G, grid, st, p);
+    else rc = launch_for_group<F32>(G, grid, st, p);
+    rc = check_launch("swa_decode_split_kernel");
+  }
+  if (rc != SB_OK || n_split == 1 || a->phases == 1) return rc;
 
   const dim3 mgrid((unsigned)(a->num_rows * a->num_q_heads));
   if (a->dtype == SB_BF16) hipLaunchKernelGGL(swa_decode_merge_kernel<BF16>, mgrid, dim3(128), 0, st, p);

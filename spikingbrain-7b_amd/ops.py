@@ -90,6 +90,7 @@ def swa_decode_attention(
     return_lse: bool = False,
     max_seq_len: Optional[int] = None,
     n_split: int = 0,
+    phases: int = 0,
 ):
     """Single-query window attention for each row of q [R, Hq, D].
 
@@ -101,7 +102,8 @@ def swa_decode_attention(
     The query of row r sits at key index seq_lens[r]-1 of sequence row_seq[r] (default r) and sees
     keys in [max(seq_lens[r]-1-window_left, key_lo[r]), seq_lens[r]-1].
     max_seq_len (a host int bounding seq_lens) only sizes the split; it defaults to a bound
-    derived from the table/window shapes so that no device value is read back."""
+    derived from the table/window shapes so that no device value is read back.
+    phases: 0 = whole op; 1 = split kernel only, 2 = merge kernel only (profiling aid)."""
     dev = N.require_gpu(q, key_cache, value_cache, seq_lens, block_table, kv_start, row_seq, key_lo, out)
     if q.dim() != 3:
         raise ValueError(f"q must be [rows, num_heads, head_size], got {tuple(q.shape)}")
@@ -158,7 +160,7 @@ def swa_decode_attention(
         workspace=N.ptr(ws), workspace_bytes=0 if ws is None else ws.numel(),
         num_rows=R, num_q_heads=Hq, num_kv_heads=Hkv, head_size=D, block_size=bs,
         window_left=int(window_left), max_seq_len=int(min(max_seq_len, 2**31 - 1)), n_split=int(n_split),
-        dtype=N.dtype_code(q.dtype), scale=float(scale),
+        dtype=N.dtype_code(q.dtype), phases=int(phases), scale=float(scale),
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
         kv_stride_block=kv_strides[0], kv_stride_row=kv_strides[1], kv_stride_head=kv_strides[2],

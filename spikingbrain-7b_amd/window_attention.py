@@ -36,11 +36,17 @@ def sliding_window_attention(
     layer_idx: int = 0,
     attention_mask: Optional[torch.Tensor] = None,
     flavour: str = "flash",
+    cache_window_size: Optional[int] = -1,
+    window_left: Optional[int] = None,
 ) -> torch.Tensor:
     """query_states [B, Hq, Q, D]; key_states/value_states [B, Hkv, Q, D] (new tokens only).
     Appends the new K/V to `past_key_values` exactly as the reference layer does, then attends
     causally inside the sliding window over the cached (or, on the first call, the in-flight)
     keys. `attention_mask` [B, >=K] marks left padding with 0. Returns [B, Q, Hq, D].
+    `flavour` picks the two conventions the reference files use (flash: cache bounded at W rows,
+    W keys left of the query visible; sdpa: cache unbounded, W keys including the query);
+    `cache_window_size` (None = unbounded) and `window_left` override them one by one, e.g. a
+    bounded cache with the SDPA mask.
     A fully masked query row (a pad position) comes out as zeros."""
     if flavour not in ("flash", "sdpa"):
         raise ValueError("flavour must be 'flash' or 'sdpa'")
@@ -49,7 +55,10 @@ def sliding_window_attention(
 
     if past_key_values is not None:
         cache_has_content = past_key_values.get_seq_length(layer_idx) > 0
-        cache_kwargs = {"window_size": sliding_window} if flavour == "flash" else {}
+        if cache_window_size == -1:
+            cache_kwargs = {"window_size": sliding_window} if flavour == "flash" else {}
+        else:
+            cache_kwargs = {"window_size": cache_window_size}
         key_cached, value_cached = past_key_values.update(
             attn_state=(key_states, value_states), layer_idx=layer_idx, offset=Q,
             cache_kwargs=cache_kwargs)["attn_state"]
@@ -57,7 +66,8 @@ def sliding_window_attention(
             key_states, value_states = key_cached, value_cached
 
     K = key_states.shape[2]
-    window_left = sliding_window if flavour == "flash" else sliding_window - 1
+    if window_left is None:
+        window_left = sliding_window if flavour == "flash" else sliding_window - 1
 
     k, v = key_states, value_states
     if k.stride(3) != 1 or v.stride() != k.stride() or _kv_start_rows(k) is None:
