@@ -102,8 +102,12 @@ int sb_kv_append(const sb_kv_append_args *args);
  * The kernel splits each row's window into n_split parts and merges them; partials live
  * in `workspace` (sb_swa_decode_workspace_bytes). n_split = 0 picks a split count from
  * the shapes alone (never from device data), so the call is graph-capturable.
- * head_size must be 128; num_q_heads/num_kv_heads in {1,2,4,7,8}.
+ * head_size must be 128. bf16/fp16 run on the matrix cores with any GQA group size
+ * num_q_heads/num_kv_heads <= 16; fp32 (and SB_DECODE_FORCE_VALU) runs on the vector ALUs with
+ * group sizes {1,2,4,7,8}.
  * ------------------------------------------------------------------------------------ */
+#define SB_DECODE_FORCE_VALU 1 /* bf16/fp16: use the vector-ALU split kernel instead of the matrix-core one */
+
 typedef struct sb_swa_decode_args {
   const void *q;   /* [num_rows, num_q_heads, head_size] */
   const void *k_cache;
@@ -125,6 +129,7 @@ typedef struct sb_swa_decode_args {
   int32_t dtype;
   int32_t phases;      /* 0 = split then merge; 1 = split kernel only; 2 = merge kernel only
                           (1 and 2 exist so a profiler can time the two kernels apart) */
+  int32_t flags;       /* SB_DECODE_* bits */
   float scale;
   int64_t q_stride_row, q_stride_head;
   int64_t out_stride_row, out_stride_head;

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libsbcache.so")
 
 SB_BF16, SB_F16, SB_F32 = 0, 1, 2
 SB_ERR_INVALID, SB_ERR_UNSUPPORTED, SB_ERR_WORKSPACE = -1, -2, -3
+SB_DECODE_FORCE_VALU = 1
 ABI_VERSION = 1
 
 _DTYPES = {torch.bfloat16: SB_BF16, torch.float16: SB_F16, torch.float32: SB_F32}
@@ -43,7 +44,7 @@ class SwaDecodeArgs(C.Structure):
         ("num_rows", i64),
         ("num_q_heads", i32), ("num_kv_heads", i32), ("head_size", i32), ("block_size", i32),
         ("window_left", i32), ("max_seq_len", i32), ("n_split", i32), ("dtype", i32),
-        ("phases", i32), ("scale", f32),
+        ("phases", i32), ("flags", i32), ("scale", f32),
         ("q_stride_row", i64), ("q_stride_head", i64),
         ("out_stride_row", i64), ("out_stride_head", i64),
         ("kv_stride_block", i64), ("kv_stride_row", i64), ("kv_stride_head", i64),

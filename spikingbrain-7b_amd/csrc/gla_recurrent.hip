@@ -41,21 +41,29 @@ __device__ __forceinline__ void store_scalar(void *p, int64_t i, int dtype, floa
     reinterpret_cast<_Float16 *>(p)[i] = (_Float16)x;
 }
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+
+// The state is touched once per call (one read, one write): non-temporal accesses keep it from
+// displacing anything useful in the caches and stream measurably faster from HBM.
 template <bool kStateF32>
 __device__ __forceinline__ float4 load_state4(const char *base, int idx4) {
   if (kStateF32) {
-    return reinterpret_cast<const float4 *>(base)[idx4];
+    const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(base) + idx4);
+    return make_float4(v.x, v.y, v.z, v.w);
   } else {
-    const uint2 w = reinterpret_cast<const uint2 *>(base)[idx4];
+    const u32x2_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(base) + idx4);
     return make_float4(sb::bf16_lo(w.x), sb::bf16_hi(w.x), sb::bf16_lo(w.y), sb::bf16_hi(w.y));
   }
 }
 template <bool kStateF32>
 __device__ __forceinline__ void store_state4(char *base, int idx4, float4 s) {
   if (kStateF32) {
-    reinterpret_cast<float4 *>(base)[idx4] = s;
+    const f32x4_t v = {s.x, s.y, s.z, s.w};
+    __builtin_nontemporal_store(v, reinterpret_cast<f32x4_t *>(base) + idx4);
   } else {
-    reinterpret_cast<uint2 *>(base)[idx4] = make_uint2(sb::pack_bf16(s.x, s.y), sb::pack_bf16(s.z, s.w));
+    const u32x2_t w = {sb::pack_bf16(s.x, s.y), sb::pack_bf16(s.z, s.w)};
+    __builtin_nontemporal_store(w, reinterpret_cast<u32x2_t *>(base) + idx4);
   }
 }
 

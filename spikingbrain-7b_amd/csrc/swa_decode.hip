@@ -15,30 +15,16 @@
 //   fp32 partial (m, l, acc) that swa_decode_merge_kernel combines.
 //   Scores are kept in log2 units: p = exp2(s*scale*log2e - m).
 #include "common.h"
+#include "swa_decode_params.h"
+
+namespace sb_host {
+void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
+                                  hipStream_t st, const sb::DecodeParams &p);
+}
 
 namespace {
 
 using namespace sb;
-
-struct DecodeParams {
-  const char *q;
-  const char *k;
-  const char *v;
-  char *out;
-  float *lse;
-  const int32_t *block_table;
-  const int64_t *kv_start;
-  const int32_t *row_seq;
-  const int32_t *seq_lens;
-  const int32_t *key_lo;
-  float *ws_acc;  // [rows, Hq, n_split, 128]
-  float *ws_ml;   // [rows, Hq, n_split, 2]
-  int Hq, block_size, window_left, n_split;
-  float scale_log2;
-  int64_t q_sr, q_sh, o_sr, o_sh;  // elements
-  int64_t kv_sb, kv_sr, kv_sh;     // bytes
-  int64_t bt_stride;
-};
 
 template <typename E>
 struct Pack {
@@ -139,9 +125,8 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   const int64_t dense_row0 = (!paged && p.kv_start) ? p.kv_start[seq] : 0;
   const int64_t lane_off = (int64_t)kvh * p.kv_sh + c * kPackBytes;
 
-  // byte offset of the first row of tile t (uniform over the wavefront)
+  // byte offset of the first row of tile t (uniform over the wavefront); callers pass t < te
   auto tile_base = [&](int t) -> int64_t {
-    if (t >= te) return 0;
     const int i0 = t << 4;
     if (paged) {
       const int bi = i0 / p.block_size;
@@ -150,12 +135,13 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     }
     return (dense_row0 + i0) * p.kv_sr;
   };
-  // rows past the last key are clamped onto it (never read outside the sequence)
+  // rows outside [lo, hi) are clamped onto the nearest visible key: nothing outside the window
+  // is ever read, so stale or uninitialised rows cannot leak in through 0 * NaN
   auto load_tile = [&](int t, int64_t base, Pack<E> (&kb)[4], Pack<E> (&vb)[4]) {
     const int i0 = t << 4;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int row = min(4 * j + g, hi - 1 - i0);
+      const int row = min(max(4 * j + g, lo - i0), hi - 1 - i0);
       const int64_t off = base + (int64_t)row * p.kv_sr + lane_off;
       kb[j] = load_pack<E>(p.k + off);
       vb[j] = load_pack<E>(p.v + off);
@@ -216,24 +202,27 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
 
   int t = tb + wave;
   if constexpr (kPrefetch) {
-    Pack<E> kb[4], vb[4];
-    int64_t base1 = tile_base(t + 4);
-    if (t < te) load_tile(t, tile_base(t), kb, vb);
-    while (t < te) {
-      const int64_t base2 = tile_base(t + 8);
-      Pack<E> kn[4], vn[4];
-      const bool more = (t + 4 < te);
-      if (more) load_tile(t + 4, base1, kn, vn);
-      compute_tile(t, kb, vb);
-      if (more) {
+    // Software pipeline, one tile deep: the loads of the next tile are issued before the
+    // current tile is computed. The prefetch is unconditional (past the end it re-reads the
+    // last tile of the split) so that the number of loads in flight is the same on every
+    // path and the wait before the compute only covers the current tile's loads.
+    if (t < te) {
+      const int last = te - 1;
+      Pack<E> kb[4], vb[4];
+      load_tile(t, tile_base(t), kb, vb);
+      int64_t base1 = tile_base(min(t + 4, last));
+      for (; t < te; t += 4) {
+        const int64_t base2 = tile_base(min(t + 8, last));
+        Pack<E> kn[4], vn[4];
+        load_tile(min(t + 4, last), base1, kn, vn);
+        compute_tile(t, kb, vb);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           kb[j] = kn[j];
           vb[j] = vn[j];
         }
+        base1 = base2;
       }
-      base1 = base2;
-      t += 4;
     }
   } else {
     for (; t < te; t += 4) {
@@ -348,16 +337,30 @@ inline int64_t round_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
 }  // namespace
 
+// Number of compute units of the current device (256 on MI355X); 256 if the query fails.
+static int device_cu_count() {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    return 256;
+  return cus;
+}
+
 extern "C" int32_t sb_swa_decode_auto_split(int64_t num_rows, int32_t num_kv_heads,
                                             int32_t max_seq_len, int32_t window_left) {
   if (num_rows <= 0 || num_kv_heads <= 0 || max_seq_len <= 0) return 1;
   int64_t keys = max_seq_len;
   if (window_left >= 0 && keys > (int64_t)window_left + 1) keys = (int64_t)window_left + 1;
-  const int64_t tiles = (keys + 15) / 16 + 1;  // +1: an unaligned window touches one more tile
-  // aim at ~2048 workgroups (8 per CU on 256 CUs), at least 4 tiles (one per wavefront) each
-  const int64_t groups = num_rows * num_kv_heads;
-  int64_t n = (2048 + groups - 1) / groups;
-  const int64_t cap = (tiles + 3) / 4;
+  const int64_t chunks = (keys + 31) / 32 + 1;  // +1: an unaligned window touches one more chunk
+  // A split is one workgroup per (row, group of up to 8 kv heads). All workgroups of a launch are
+  // resident at once and each streams at the same rate, so the launch is fastest when their
+  // number is a whole multiple of the CU count: take the split count that brings it nearest to
+  // one workgroup per CU, but leave every workgroup at least 8 chunks (256 keys) of work so that
+  // filling its load pipeline and writing its partial result stay small next to the streaming.
+  const int64_t wgs = num_rows * ((num_kv_heads + 7) / 8);
+  const int64_t cus = device_cu_count();
+  int64_t n = (cus + wgs / 2) / wgs;
+  const int64_t cap = chunks / 8;
   if (n > cap) n = cap;
   if (n > 64) n = 64;
   if (n < 1) n = 1;
@@ -437,10 +440,20 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   hipStream_t st = (hipStream_t)a->stream;
   int rc = 0;
   if (a->phases < 0 || a->phases > 2) return fail(SB_ERR_INVALID, "sb_swa_decode: phases must be 0, 1 or 2");
-  if (G != 1 && G != 2 && G != 4 && G != 7 && G != 8)
-    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: GQA group size %d (built: 1, 2, 4, 7, 8)", G);
+  // bf16/fp16 run on the matrix cores (any group size up to 16); fp32 runs on the vector ALUs
+  const bool mfma = (a->dtype != SB_F32) && !(a->flags & SB_DECODE_FORCE_VALU);
+  if (mfma ? (G > 16) : (G != 1 && G != 2 && G != 4 && G != 7 && G != 8))
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: GQA group size %d (built: up to 16 for bf16/fp16; 1, 2, 4, 7, 8 for fp32)", G);
+  if (mfma && (a->kv_stride_row <= 0 || a->kv_stride_row * esz * 16 >= (1LL << 31)))
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: kv row stride %lld does not fit the kernel's 32-bit in-tile offsets",
+                (long long)a->kv_stride_row);
+  if (mfma && ((reinterpret_cast<uintptr_t>(a->out) & 15u) || (a->out_stride_row * esz) % 16 ||
+               (a->out_stride_head * esz) % 16))
+    return fail(SB_ERR_INVALID, "sb_swa_decode: out rows must be 16-byte aligned");
   if (a->phases != 2) {
-    if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
+    if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
+                                           (a->flags >> 4) & 7, st, p);
+    else if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
     else if (a->dtype == SB_F16) rc = launch_for_group<F16>(G, grid, st, p);
     else rc = launch_for_group<F32>(G, grid, st, p);
     rc = check_launch("swa_decode_split_kernel");

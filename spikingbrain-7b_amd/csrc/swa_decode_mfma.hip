@@ -1,0 +1,347 @@
+// Window-bounded single-query attention, split-K, bf16/fp16, matrix-core version.
+//
+// Why matrix cores here: with a GQA group of 7 every K/V byte feeds 7 query heads, i.e. 7 flop per
+// byte; done on the vector ALUs that is ~900 VALU instructions per 16-key tile and the split kernel
+// ran VALU-bound (71 % VALU issue utilisation at 50 % of HBM peak on the 7B decode shape). The
+// group is therefore padded to the 16-wide N dimension of v_mfma_f32_16x16x32 and both
+// contractions run on the matrix cores; what is left on the VALU is the softmax of a
+// [32 keys x 16 heads] tile (8 values per lane) and an in-register 8x8 transpose of V.
+//
+// Work decomposition: grid = (query rows, kv-head groups, splits). A workgroup has one wavefront
+// per kv head (up to 8), all walking the same part of the same sequence's window: the heads of a
+// cache row are adjacent in memory (a 16-token block of 4 heads is 16 KiB contiguous), so the
+// wavefronts of a workgroup together stream whole DRAM pages instead of 256-byte pieces 1 KiB
+// apart. Wavefronts are independent (own head group, own online softmax, own partial result):
+// no LDS, no barrier. A wavefront walks over "chunks" of 32 keys (two 16-key tiles).
+// Lane = (g = lane/16, c = lane%16). K/V are read once, with non-temporal loads.
+//
+//   S^T = K Q^T   A = K tile  : lane (g,c) holds key c of the tile, dims of 16-byte chunk 4s+g
+//                 B = Q^T     : lane (g,c) holds head c (zero for c >= G), same dims
+//                 D = S^T     : lane (g,c) holds head c, keys 4g..4g+3 of the tile
+//   O^T = V^T P^T A = V^T     : lane (g,c) holds dim 8c+mt, keys kk = 8g..8g+7 of the chunk, where
+//                               kk = 8g+j is key 4g+j of tile 0 (j<4) or key 4g+j-4 of tile 1
+//                 B = P^T     : lane (g,c) holds head c, the same 8 keys: exactly the S^T results of
+//                               that lane, so P never leaves its registers
+//                 D = O^T     : lane (g,c) holds head c, dims 32g + 8i + mt (i<4, mt<8)
+//   V is loaded as 16-byte row pieces (lane (g,c): its 8 keys, dims 8c..8c+7; one instruction covers
+//   4 whole 256-byte rows) and the 8x8 (key x dim) block of a lane is transposed in registers with
+//   v_perm_b32 to give the 8 A operands. K loads cover 16 rows x 64 bytes per instruction.
+//   Softmax state (running max m, denominator l) is per lane for head c; the max is shared by the
+//   four g groups of a head through two cross-lane exchanges per chunk.
+// Rows outside [lo, hi) are never read: row indices are clamped into the visible range for the
+// address and masked by their true index for the score, so stale or uninitialised cache rows
+// cannot leak NaNs through 0 * NaN.
+#include "common.h"
+#include "swa_decode_params.h"
+
+namespace {
+
+using namespace sb;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+template <typename E>
+struct Mma;
+template <>
+struct Mma<BF16> {
+  __device__ static __forceinline__ f32x4_t run(const uint4 &a, const uint4 &b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pack(float lo, float hi) {
+    bf16x2_t v;
+    v[0] = (__bf16)lo;
+    v[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, v);
+  }
+};
+template <>
+struct Mma<F16> {
+  __device__ static __forceinline__ f32x4_t run(const uint4 &a, const uint4 &b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pack(float lo, float hi) { return pack_f16(lo, hi); }
+};
+
+constexpr float kNegInf = -__builtin_inff();
+
+__device__ __forceinline__ uint32_t perm_lo(uint32_t hi_src, uint32_t lo_src) {
+  return __builtin_amdgcn_perm(hi_src, lo_src, 0x05040100u);  // (hi_src.lo16 << 16) | lo_src.lo16
+}
+__device__ __forceinline__ uint32_t perm_hi(uint32_t hi_src, uint32_t lo_src) {
+  return __builtin_amdgcn_perm(hi_src, lo_src, 0x07060302u);  // (hi_src.hi16 << 16) | lo_src.hi16
+}
+__device__ __forceinline__ uint32_t word(const uint4 &v, int i) {
+  return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
+}
+
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+// K/V bytes are used exactly once per launch: stream them past the caches.
+__device__ __forceinline__ uint4 load_stream16(const char *p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+struct Chunk {
+  uint4 k0[4], k1[4];  // K operands of tile 0 / tile 1, one per 32-dim step
+  uint4 v[8];          // V rows of this lane's 8 keys, dims 8c..8c+7
+};
+
+// kDepth = chunks in flight per wavefront besides the one being computed; kMaxThreads bounds the
+// workgroup size, which with one workgroup per CU fixes the register budget (256 threads: one
+// wavefront per SIMD, 512 registers; 512 threads: two per SIMD, 256 registers).
+template <typename E, int kDepth, int kMaxThreads>
+__global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(const DecodeParams p, const int G,
+                                                                                const int Hkv) {
+  const int64_t r = blockIdx.x;
+  const int split = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int kvh = blockIdx.y * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (kvh >= Hkv) return;  // whole wavefront; there is no barrier in this kernel
+  const int lane = tid & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+
+  const int64_t seq = p.row_seq ? (int64_t)p.row_seq[r] : r;
+  const int hi = p.seq_lens[r];
+  int lo = p.window_left >= 0 ? max(0, hi - 1 - p.window_left) : 0;
+  if (p.key_lo) lo = max(lo, p.key_lo[r]);
+  const bool any = hi > lo;
+
+  const int first_tile = lo >> 4;
+  const int last_tile = any ? (hi - 1) >> 4 : first_tile;
+  const int first_chunk = first_tile >> 1;
+  const int n_chunks = any ? (last_tile >> 1) - first_chunk + 1 : 0;
+  const int cps = (n_chunks + p.n_split - 1) / p.n_split;
+  const int cb = first_chunk + split * cps;
+  const int ce = min(cb + cps, first_chunk + n_chunks);
+
+  // Q^T operands: head c of the group, dims of chunk 4s+g; zero rows pad the group to 16 heads
+  uint4 qb[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    qb[s] = make_uint4(0u, 0u, 0u, 0u);
+    if (c < G)
+      qb[s] = *reinterpret_cast<const uint4 *>(
+          p.q + (r * p.q_sr + (int64_t)(kvh * G + c) * p.q_sh + (4 * s + g) * 8) * 2);
+  }
+
+  f32x4_t acc[8];
+#pragma unroll
+  for (int mt = 0; mt < 8; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = kNegInf, l = 0.f;
+
+  const bool paged = p.block_table != nullptr;
+  const int64_t dense_row0 = (!paged && p.kv_start) ? p.kv_start[seq] : 0;
+  const int64_t head_off = (int64_t)kvh * p.kv_sh;
+
+  // byte offset of row 0 of tile t (t inside [first_tile, last_tile]; uniform over the wavefront)
+  auto tile_base = [&](int t) -> int64_t {
+    const int i0 = t << 4;
+    if (paged) {
+      const int bi = i0 / p.block_size;
+      const int64_t blk = p.block_table[seq * p.bt_stride + bi];
+      return blk * p.kv_sb + (int64_t)(i0 - bi * p.block_size) * p.kv_sr + head_off;
+    }
+    return (dense_row0 + i0) * p.kv_sr + head_off;
+  };
+  auto clamp_tile = [&](int t) { return min(max(t, first_tile), last_tile); };
+  // row of tile tc whose key index is the visible key nearest to (tc*16 + row)
+  auto clamp_row = [&](int tc, int row) { return min(max((tc << 4) + row, lo), hi - 1) - (tc << 4); };
+
+  // Lane offsets inside a tile (bytes, 32-bit): K row c at 16-byte piece g; V rows 4g+j at piece c.
+  // Interior chunks use these constants; edge chunks (first/last of the window) clamp their rows.
+  const uint32_t kv_sr32 = (uint32_t)p.kv_sr;
+  const uint32_t koff = c * kv_sr32 + g * 16;
+  uint32_t voff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) voff[j] = (4 * g + j) * kv_sr32 + c * 16;
+
+  auto load_chunk = [&](int cc, int t0c, int t1c, int64_t b0, int64_t b1, Chunk &ck) {
+    const char *k0p = p.k + b0, *k1p = p.k + b1, *v0p = p.v + b0, *v1p = p.v + b1;  // wave-uniform bases
+    uint32_t ko0 = koff, ko1 = koff, vo0[4], vo1[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) vo0[j] = vo1[j] = voff[j];
+    if ((cc << 5) < lo || (cc << 5) + 32 > hi) {
+      ko0 = clamp_row(t0c, c) * kv_sr32 + g * 16;
+      ko1 = clamp_row(t1c, c) * kv_sr32 + g * 16;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        vo0[j] = clamp_row(t0c, 4 * g + j) * kv_sr32 + c * 16;
+        vo1[j] = clamp_row(t1c, 4 * g + j) * kv_sr32 + c * 16;
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      ck.k0[s] = load_stream16(k0p + ko0 + s * 64);
+      ck.k1[s] = load_stream16(k1p + ko1 + s * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      ck.v[j] = load_stream16(v0p + vo0[j]);
+      ck.v[4 + j] = load_stream16(v1p + vo1[j]);
+    }
+  };
+
+  auto compute_chunk = [&](int ch, const Chunk &ck) {
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      s0 = Mma<E>::run(ck.k0[s], qb[s], s0);
+      s1 = Mma<E>::run(ck.k1[s], qb[s], s1);
+    }
+    float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+    const int i0 = ch << 5;
+    if (i0 < lo || i0 + 32 > hi) {  // edge chunk: mask keys outside [lo, hi) by their true index
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int i = i0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+        if (i < lo || i >= hi) sc[j] = kNegInf;
+      }
+    }
+    float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m, mx * p.scale_log2);
+    const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = fast_exp2(m - m_safe);
+    const bool grew = m_new > m;
+    m = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      sc[j] = fast_exp2(fmaf(sc[j], p.scale_log2, -m_safe));
+      psum += sc[j];
+    }
+    l = fmaf(l, alpha, psum);
+    if (__builtin_amdgcn_ballot_w64(grew) != 0) {
+#pragma unroll
+      for (int mt = 0; mt < 8; ++mt) acc[mt] *= alpha;
+    }
+    const uint4 pb = make_uint4(Mma<E>::pack(sc[0], sc[1]), Mma<E>::pack(sc[2], sc[3]),
+                                Mma<E>::pack(sc[4], sc[5]), Mma<E>::pack(sc[6], sc[7]));
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) {
+      const int w = mt >> 1;
+      uint4 vt;
+      if (mt & 1) {
+        vt = make_uint4(perm_hi(word(ck.v[1], w), word(ck.v[0], w)), perm_hi(word(ck.v[3], w), word(ck.v[2], w)),
+                        perm_hi(word(ck.v[5], w), word(ck.v[4], w)), perm_hi(word(ck.v[7], w), word(ck.v[6], w)));
+      } else {
+        vt = make_uint4(perm_lo(word(ck.v[1], w), word(ck.v[0], w)), perm_lo(word(ck.v[3], w), word(ck.v[2], w)),
+                        perm_lo(word(ck.v[5], w), word(ck.v[4], w)), perm_lo(word(ck.v[7], w), word(ck.v[6], w)));
+      }
+      acc[mt] = Mma<E>::run(vt, pb, acc[mt]);
+    }
+  };
+
+  // Software pipeline kDepth chunks deep over a ring of kDepth+1 register sets (the loop is unrolled
+  // over the ring so that no registers are copied). Prefetches are unconditional (past the end they
+  // re-read the last chunk of the split), so the number of loads in flight is the same on every
+  // path and the wait before a compute covers only that chunk's loads. Tile bases (block-table
+  // lookups) run one more chunk ahead of the loads.
+  int ch = cb;
+  if (ch < ce) {
+    const int lastc = ce - 1;
+    int t0, t1;
+    int64_t b0, b1;
+    auto locate = [&](int cc) {
+      t0 = clamp_tile(2 * cc);
+      t1 = clamp_tile(2 * cc + 1);
+      b0 = tile_base(t0);
+      b1 = tile_base(t1);
+    };
+    // loads chunk min(cc, lastc), whose tiles the previous call located, and locates the next one
+    auto issue = [&](int cc, Chunk &dst) {
+      const int lt0 = t0, lt1 = t1;
+      const int64_t lb0 = b0, lb1 = b1;
+      locate(min(cc + 1, lastc));
+      load_chunk(min(cc, lastc), lt0, lt1, lb0, lb1, dst);
+    };
+    Chunk ring[kDepth + 1];
+    locate(ch);
+#pragma unroll
+    for (int u = 0; u < kDepth; ++u) issue(ch + u, ring[u]);
+    bool more = true;
+    while (more) {
+#pragma unroll
+      for (int u = 0; u <= kDepth; ++u) {
+        if (more) {
+          issue(ch + kDepth, ring[(u + kDepth) % (kDepth + 1)]);
+          compute_chunk(ch, ring[u]);
+          ++ch;
+          more = ch < ce;
+        }
+      }
+    }
+  }
+
+  // ---- denominators of the four g groups -> one per head ------------------------------
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+
+  // ---- this wavefront's result: lane (g, c < G) owns head c, dims 32g + 8i + mt --------------
+  if (c < G) {
+    const int hq = kvh * G + c;
+    if (p.n_split == 1) {
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      char *dst = p.out + (r * p.o_sr + (int64_t)hq * p.o_sh + 32 * g) * 2;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint4 o;
+        o.x = E::pack(acc[0][i] * inv, acc[1][i] * inv);
+        o.y = E::pack(acc[2][i] * inv, acc[3][i] * inv);
+        o.z = E::pack(acc[4][i] * inv, acc[5][i] * inv);
+        o.w = E::pack(acc[6][i] * inv, acc[7][i] * inv);
+        *reinterpret_cast<uint4 *>(dst + 16 * i) = o;
+      }
+      if (g == 0 && p.lse) p.lse[r * p.Hq + hq] = l > 0.f ? (m + log2f(l)) * kLn2 : kNegInf;
+    } else {
+      const int64_t part = (r * p.Hq + hq) * p.n_split + split;
+      float *dst = p.ws_acc + part * 128 + 32 * g;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        reinterpret_cast<float4 *>(dst + 8 * i)[0] = make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]);
+        reinterpret_cast<float4 *>(dst + 8 * i)[1] = make_float4(acc[4][i], acc[5][i], acc[6][i], acc[7][i]);
+      }
+      if (g == 0) {
+        p.ws_ml[part * 2] = m;
+        p.ws_ml[part * 2 + 1] = l;
+      }
+    }
+  }
+}
+
+}  // namespace
+
+namespace sb_host {
+
+// Launches the matrix-core split kernel (dtype bf16 or fp16, group size <= 16).
+// `rows`, `n_split` give grid x and z; the kv heads are spread over wavefronts and grid y.
+void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
+                                  hipStream_t st, const sb::DecodeParams &p) {
+  const int waves = Hkv < 8 ? Hkv : 8;
+  const dim3 grid(rows, (unsigned)((Hkv + waves - 1) / waves), n_split), block(64 * waves);
+  // up to 4 wavefronts per workgroup: one per SIMD with the whole register file, deep pipeline;
+  // more: two per SIMD, pipeline one chunk deep
+  if (depth <= 0) depth = waves <= 4 ? 3 : 1;
+  if (waves > 4) depth = 1;
+#define SB_LAUNCH(E, D, T) hipLaunchKernelGGL((swa_decode_split_mfma_kernel<E, D, T>), grid, block, 0, st, p, G, Hkv)
+  if (dtype == SB_BF16) {
+    if (waves > 4) SB_LAUNCH(sb::BF16, 1, 512);
+    else if (depth == 1) SB_LAUNCH(sb::BF16, 1, 256);
+    else if (depth == 2) SB_LAUNCH(sb::BF16, 2, 256);
+    else SB_LAUNCH(sb::BF16, 3, 256);
+  } else {
+    if (waves > 4) SB_LAUNCH(sb::F16, 1, 512);
+    else if (depth == 1) SB_LAUNCH(sb::F16, 1, 256);
+    else if (depth == 2) SB_LAUNCH(sb::F16, 2, 256);
+    else SB_LAUNCH(sb::F16, 3, 256);
+  }
+#undef SB_LAUNCH
+}
+
+}  // namespace sb_host

@@ -1,0 +1,27 @@
+// Kernel parameter block shared by the two split kernels (VALU and matrix-core) and the merge.
+#pragma once
+#include <stdint.h>
+
+namespace sb {
+
+struct DecodeParams {
+  const char *q;
+  const char *k;
+  const char *v;
+  char *out;
+  float *lse;
+  const int32_t *block_table;
+  const int64_t *kv_start;
+  const int32_t *row_seq;
+  const int32_t *seq_lens;
+  const int32_t *key_lo;
+  float *ws_acc;  // [rows, Hq, n_split, 128]
+  float *ws_ml;   // [rows, Hq, n_split, 2]
+  int Hq, block_size, window_left, n_split;
+  float scale_log2;
+  int64_t q_sr, q_sh, o_sr, o_sh;  // elements
+  int64_t kv_sb, kv_sr, kv_sh;     // bytes
+  int64_t bt_stride;
+};
+
+}  // namespace sb

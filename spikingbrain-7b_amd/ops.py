@@ -91,6 +91,8 @@ def swa_decode_attention(
     max_seq_len: Optional[int] = None,
     n_split: int = 0,
     phases: int = 0,
+    force_valu: bool = False,
+    pipeline_depth: int = 0,
 ):
     """Single-query window attention for each row of q [R, Hq, D].
 
@@ -103,7 +105,8 @@ def swa_decode_attention(
     keys in [max(seq_lens[r]-1-window_left, key_lo[r]), seq_lens[r]-1].
     max_seq_len (a host int bounding seq_lens) only sizes the split; it defaults to a bound
     derived from the table/window shapes so that no device value is read back.
-    phases: 0 = whole op; 1 = split kernel only, 2 = merge kernel only (profiling aid)."""
+    phases: 0 = whole op; 1 = split kernel only, 2 = merge kernel only (profiling aid).
+    force_valu: run bf16/fp16 on the vector-ALU split kernel instead of the matrix-core one."""
     dev = N.require_gpu(q, key_cache, value_cache, seq_lens, block_table, kv_start, row_seq, key_lo, out)
     if q.dim() != 3:
         raise ValueError(f"q must be [rows, num_heads, head_size], got {tuple(q.shape)}")
@@ -160,7 +163,8 @@ def swa_decode_attention(
         workspace=N.ptr(ws), workspace_bytes=0 if ws is None else ws.numel(),
         num_rows=R, num_q_heads=Hq, num_kv_heads=Hkv, head_size=D, block_size=bs,
         window_left=int(window_left), max_seq_len=int(min(max_seq_len, 2**31 - 1)), n_split=int(n_split),
-        dtype=N.dtype_code(q.dtype), phases=int(phases), scale=float(scale),
+        dtype=N.dtype_code(q.dtype), phases=int(phases), flags=(N.SB_DECODE_FORCE_VALU if force_valu else 0) | ((int(pipeline_depth) & 7) << 4),
+        scale=float(scale),
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
         kv_stride_block=kv_strides[0], kv_stride_row=kv_strides[1], kv_stride_head=kv_strides[2],

@@ -63,8 +63,10 @@ def test_bad_shapes_rejected_before_launch(sb):
 def test_auto_split_and_workspace(sb):
     L = sb._native.lib()
     n = L.sb_swa_decode_auto_split(64, 4, 32768, 4096)
-    assert n == 8
+    assert n == 4                                                   # 64 workgroups per split -> 256 = one per CU
     assert L.sb_swa_decode_auto_split(4096, 4, 32768, 4096) == 1
+    assert L.sb_swa_decode_auto_split(1, 4, 300, 4096) == 1         # short windows are never split below 8 chunks
+    assert L.sb_swa_decode_auto_split(1, 4, 1 << 20, -1) == 64      # capped
     assert L.sb_swa_decode_workspace_bytes(64, 28, 128, 1) == 0
     need = L.sb_swa_decode_workspace_bytes(64, 28, 128, 8)
     assert need >= 64 * 28 * 8 * 130 * 4

@@ -31,21 +31,55 @@ def run_paged(sb, dev, q, kv, tables, lens, wl, scale, **kw):
                                        block_table=tables.to(dev), window_left=wl, scale=scale, **kw)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("dtype,force_valu", [(torch.bfloat16, False), (torch.float16, False), (torch.float32, False),
+                                              (torch.bfloat16, True)])
 @pytest.mark.parametrize("Hq,Hkv", [(28, 4), (8, 8), (8, 2), (16, 2)])
 @pytest.mark.parametrize("wl,n_split", [(64, 1), (64, 3), (37, 0), (-1, 2), (0, 1)])
-def test_paged_decode_vs_oracle(sb, dev, dtype, Hq, Hkv, wl, n_split):
+def test_paged_decode_vs_oracle(sb, dev, dtype, force_valu, Hq, Hkv, wl, n_split):
     D, bs = 128, 16
     lens = [1, 15, 16, 17, 64, 65, 100, 129, 200]
     kv, tables = paged_problem(lens, bs, Hkv, D, dtype, seed=Hq * 7 + (wl % 5))
     g = torch.Generator().manual_seed(2)
     q = torch.randn(len(lens), Hq, D, generator=g).to(dtype)
     scale = D ** -0.5
-    out, lse = run_paged(sb, dev, q, kv, tables, lens, wl, scale, n_split=n_split, return_lse=True)
+    out, lse = run_paged(sb, dev, q, kv, tables, lens, wl, scale, n_split=n_split, return_lse=True, force_valu=force_valu)
     ref, ref_lse = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(),
                                             tables.numpy(), lens, scale, wl, return_lse=True)
     assert np.abs(out.float().cpu().numpy() - ref).max() <= TOL[dtype]
     assert np.abs(lse.cpu().numpy() - ref_lse).max() <= 1e-3
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(12, 4), (5, 1), (16, 1), (26, 2)])
+def test_matrix_core_kernel_any_group_size(sb, dev, Hq, Hkv):
+    D, bs = 128, 16
+    lens = [1, 31, 32, 33, 95, 257]
+    kv, tables = paged_problem(lens, bs, Hkv, D, torch.bfloat16, seed=Hq)
+    q = torch.randn(len(lens), Hq, D, generator=torch.Generator().manual_seed(4)).bfloat16()
+    for wl, n_split in [(50, 1), (-1, 3), (31, 2)]:
+        out = run_paged(sb, dev, q, kv, tables, lens, wl, D ** -0.5, n_split=n_split)
+        ref = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(),
+                                       tables.numpy(), lens, D ** -0.5, wl)
+        assert np.abs(out.float().cpu().numpy() - ref).max() <= 2e-2
+
+
+def test_uninitialised_rows_outside_the_window_do_not_leak(sb, dev):
+    """Rows past the newest key and rows older than the window may hold anything (NaN bit
+    patterns included): they must not reach the output."""
+    D, bs, Hq, Hkv, wl = 128, 16, 28, 4, 40
+    lens = [70, 21]
+    kv, tables = paged_problem(lens, bs, Hkv, D, torch.bfloat16, seed=9)
+    q = torch.randn(2, Hq, D, generator=torch.Generator().manual_seed(5)).bfloat16()
+    ref = run_paged(sb, dev, q, kv, tables, lens, wl, D ** -0.5)
+    poisoned = kv.clone()
+    for b, n in enumerate(lens):
+        for i in list(range(0, max(0, n - 1 - wl))) + list(range(n, tables.shape[1] * bs)):
+            blk = int(tables[b, i // bs])
+            if i // bs < (n + bs - 1) // bs or i < n:
+                poisoned[:, blk, i % bs] = float("nan")
+    for fv in (False, True):
+        out = run_paged(sb, dev, q, poisoned, tables, lens, wl, D ** -0.5, force_valu=fv)
+        assert not torch.isnan(out).any()
+        assert (out.float() - ref.float()).abs().max() <= 4e-3
 
 
 def test_block_size_64_and_large_scores(sb, dev):
@@ -170,7 +204,9 @@ def test_argument_errors(sb, dev):
         sb.ops.swa_decode_attention(q, kv[0], kv[1], sl.long(), block_table=bt)
     with pytest.raises(ValueError, match="share one dtype"):
         sb.ops.swa_decode_attention(q.float(), kv[0], kv[1], sl, block_table=bt)
-    with pytest.raises(NotImplementedError, match="group size"):
-        sb.ops.swa_decode_attention(torch.zeros(2, 12, 128, device=dev, dtype=torch.bfloat16), kv[0], kv[1], sl, block_table=bt)
+    with pytest.raises(NotImplementedError, match="group size"):      # fp32 (vector-ALU kernel): group of 3 is not built
+        sb.ops.swa_decode_attention(torch.zeros(2, 12, 128, device=dev), kv[0].float(), kv[1].float(), sl, block_table=bt)
+    with pytest.raises(NotImplementedError, match="group size"):      # bf16 (matrix-core kernel): group of 17 > 16
+        sb.ops.swa_decode_attention(torch.zeros(2, 68, 128, device=dev, dtype=torch.bfloat16), kv[0], kv[1], sl, block_table=bt)
     with pytest.raises(ValueError, match="dense mode"):
         sb.ops.swa_decode_attention(q, kv[0], kv[1], sl)
