@@ -2,7 +2,8 @@
 
 A "step" is one pass of the hot path over one batch of synthetic input at BASELINE config 2
 (paged SWA decode at the 7B layer shape): KV append of one new token per sequence through
-slot_mapping, then window-bounded paged decode attention (split kernel + merge kernel).
+slot_mapping, then window-bounded paged decode attention (split kernel + merge kernel); for a pure
+decode batch the split kernel does the append itself (one launch less), as the backend's forward does.
   B=64, 28 q / 4 kv heads, head_dim 128, block_size 16, window_left 4096, bf16,
   context lengths ~ U[1024, 32768] (seed 0), seeded block permutation, only in-window blocks
   resident, K/V ~ N(0,1).
@@ -108,6 +109,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--n-split", type=int, default=0)
+    ap.add_argument("--unfused", action="store_true", help="append with a separate kv_append launch")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3)")
     args = ap.parse_args()
@@ -125,19 +127,27 @@ def main():
     prob = build_config2(dev)
     kv, n_copies = prob["kv"], len(prob["kv"])
 
-    def attend(c, phases):
+    new_kv = dict(new_key=prob["k"], new_value=prob["v"], new_slot_mapping=prob["slots"])
+
+    def attend(c, phases, **kw):
         sb.ops.swa_decode_attention(prob["q"], c[0], c[1], prob["seqlens"], block_table=prob["tables"],
                                     window_left=WL, out=prob["out"], max_seq_len=prob["max_seq_len"],
-                                    n_split=args.n_split, phases=phases)
+                                    n_split=args.n_split, phases=phases, **kw)
 
     def step(i, events=None):
+        """One layer-step as MetaAttentionImpl.forward runs a pure decode batch: the split kernel
+        appends each sequence's new K/V row at its slot and attends; the merge kernel follows.
+        --unfused runs the append as a launch of its own (what mixed prefill/decode steps do)."""
         c = kv[i % n_copies]
-        sb.ops.kv_append(prob["k"], prob["v"], c[0], c[1], prob["slots"])
+        kw = new_kv
+        if args.unfused:
+            sb.ops.kv_append(prob["k"], prob["v"], c[0], c[1], prob["slots"])
+            kw = {}
         if events is None:
-            attend(c, 0)
+            attend(c, 0, **kw)
         else:  # same launches, with the split kernel bracketed by events on the launch stream
             events[0].record()
-            attend(c, 1)
+            attend(c, 1, **kw)
             events[1].record()
             attend(c, 2)
 
@@ -177,6 +187,21 @@ def main():
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": None, "kernel_ms": round(k_ms, 4), "bytes_per_launch": prob["bytes_split_kernel"]},
     }
+
+    # plain streaming copy of 1 GiB in the same run: what this box's HBM gives a copy kernel
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        sb.ops.stream_copy(dst, src)
+    evc = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(10)]
+    for a, b in evc:
+        a.record()
+        sb.ops.stream_copy(dst, src)
+        b.record()
+    torch.cuda.synchronize()
+    copy_ms = statistics.mean(a.elapsed_time(b) for a, b in evc)
+    line["stream_copy_GBps_read_plus_write"] = round(2 * (1 << 30) / (copy_ms * 1e-3) / 1e9, 1)
+    del src, dst
 
     if args.extras:
         B3, H3 = 64, 28

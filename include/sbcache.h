@@ -135,6 +135,18 @@ typedef struct sb_swa_decode_args {
   int64_t out_stride_row, out_stride_head;
   int64_t kv_stride_block, kv_stride_row, kv_stride_head;
   int64_t block_table_stride;
+  /* Optional fused append (all three NULL = attention only). When set, row r's newest key
+   * (index seq_lens[r]-1) has not been appended yet: its K/V rows are new_key[r] / new_value[r]
+   * ([num_rows, num_kv_heads, head_size], strides below) and the call also stores them at
+   * new_slot_mapping[r] (int64; < 0 = do not store), i.e. it does what reshape_and_cache_flash
+   * (meta_attention.py:790-799) followed by the decode call (:965-981) do, in one launch.
+   * Requires paged mode, one query row per sequence (row_seq NULL); k_cache/v_cache are
+   * written. */
+  const void *new_key;
+  const void *new_value;
+  const int64_t *new_slot_mapping;
+  int64_t new_key_stride_row, new_key_stride_head;
+  int64_t new_value_stride_row, new_value_stride_head;
   void *stream;
 } sb_swa_decode_args;
 
@@ -213,6 +225,14 @@ typedef struct sb_window_shift_args {
 } sb_window_shift_args;
 
 int sb_window_shift(const sb_window_shift_args *args);
+
+/* ------------------------------------------------------------------------------------
+ * Plain device-to-device streaming copy (non-temporal 16-byte lanes), `bytes` a multiple of
+ * 16384. No counterpart in the reference: it is the measured bandwidth yardstick printed by
+ * bench.py next to the kernels, and the launch of known size that the HBM byte counters
+ * (FETCH_SIZE / WRITE_SIZE) are calibrated against.
+ * ------------------------------------------------------------------------------------ */
+int sb_stream_copy(void *dst, const void *src, int64_t bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -48,7 +48,11 @@ class SwaDecodeArgs(C.Structure):
         ("q_stride_row", i64), ("q_stride_head", i64),
         ("out_stride_row", i64), ("out_stride_head", i64),
         ("kv_stride_block", i64), ("kv_stride_row", i64), ("kv_stride_head", i64),
-        ("block_table_stride", i64), ("stream", vp),
+        ("block_table_stride", i64),
+        ("new_key", vp), ("new_value", vp), ("new_slot_mapping", vp),
+        ("new_key_stride_row", i64), ("new_key_stride_head", i64),
+        ("new_value_stride_row", i64), ("new_value_stride_head", i64),
+        ("stream", vp),
     ]
 
 
@@ -87,6 +91,7 @@ EXPORTS = {
     "sb_gla_recurrent": (C.c_int, [C.POINTER(GlaRecurrentArgs)]),
     "sb_copy_blocks": (C.c_int, [vp, vp, i64, i64, i64, vp]),
     "sb_window_shift": (C.c_int, [C.POINTER(WindowShiftArgs)]),
+    "sb_stream_copy": (C.c_int, [vp, vp, i64, vp]),
 }
 
 _lib: Optional[C.CDLL] = None

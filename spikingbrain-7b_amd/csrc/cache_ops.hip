@@ -157,3 +157,35 @@ extern "C" int sb_window_shift(const sb_window_shift_args *a) {
                      a->fresh_stride_plane_bytes, a->fresh_stride_row_bytes);
   return check_launch("window_shift_kernel");
 }
+
+// ---- plain streaming copy: the bandwidth yardstick bench.py reports next to the kernels and the
+// known-size launch that hardware byte counters are calibrated against --------------------------
+namespace {
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void stream_copy_kernel(const u32x4_t *__restrict__ src,
+                                                          u32x4_t *__restrict__ dst, int64_t n16) {
+  int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 1024;
+  for (; i + 768 < n16; i += stride) {
+    u32x4_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(src + i + 256 * u);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u], dst + i + 256 * u);
+  }
+}
+}  // namespace
+
+extern "C" int sb_stream_copy(void *dst, const void *src, int64_t bytes, void *stream) {
+  using namespace sb_host;
+  if (bytes < 0 || bytes % 16384 != 0) return fail(SB_ERR_INVALID, "sb_stream_copy: bytes must be a multiple of 16384");
+  if (bytes == 0) return SB_OK;
+  if (!dst || !src || !aligned16(dst) || !aligned16(src))
+    return fail(SB_ERR_INVALID, "sb_stream_copy: null or misaligned pointer");
+  const int64_t n16 = bytes / 16;
+  int64_t blocks = n16 / 1024;
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const u32x4_t *)src, (u32x4_t *)dst, n16);
+  return check_launch("stream_copy_kernel");
+}

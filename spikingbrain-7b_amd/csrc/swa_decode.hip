@@ -352,12 +352,12 @@ extern "C" int32_t sb_swa_decode_auto_split(int64_t num_rows, int32_t num_kv_hea
   int64_t keys = max_seq_len;
   if (window_left >= 0 && keys > (int64_t)window_left + 1) keys = (int64_t)window_left + 1;
   const int64_t chunks = (keys + 31) / 32 + 1;  // +1: an unaligned window touches one more chunk
-  // A split is one workgroup per (row, group of up to 8 kv heads). All workgroups of a launch are
+  // A split is one workgroup per (row, group of up to 4 kv heads). All workgroups of a launch are
   // resident at once and each streams at the same rate, so the launch is fastest when their
   // number is a whole multiple of the CU count: take the split count that brings it nearest to
   // one workgroup per CU, but leave every workgroup at least 8 chunks (256 keys) of work so that
   // filling its load pipeline and writing its partial result stay small next to the streaming.
-  const int64_t wgs = num_rows * ((num_kv_heads + 7) / 8);
+  const int64_t wgs = num_rows * ((num_kv_heads + 3) / 4);
   const int64_t cus = device_cu_count();
   int64_t n = (cus + wgs / 2) / wgs;
   const int64_t cap = chunks / 8;
@@ -450,6 +450,42 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   if (mfma && ((reinterpret_cast<uintptr_t>(a->out) & 15u) || (a->out_stride_row * esz) % 16 ||
                (a->out_stride_head * esz) % 16))
     return fail(SB_ERR_INVALID, "sb_swa_decode: out rows must be 16-byte aligned");
+
+  // optional fused append of the step's newest key/value row
+  p.new_k = p.new_v = nullptr;
+  p.slot_mapping = nullptr;
+  p.nk_st = p.nk_sh = p.nv_st = p.nv_sh = 0;
+  const bool want_append = a->new_key || a->new_value || a->new_slot_mapping;
+  if (want_append) {
+    if (!a->new_key || !a->new_value || !a->new_slot_mapping)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: new_key, new_value and new_slot_mapping go together");
+    if (!a->block_table || a->row_seq)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: fused append needs paged mode and one query row per sequence");
+    if (((reinterpret_cast<uintptr_t>(a->new_key) | reinterpret_cast<uintptr_t>(a->new_value)) & 15u) ||
+        (a->new_key_stride_row * esz) % 16 || (a->new_key_stride_head * esz) % 16 ||
+        (a->new_value_stride_row * esz) % 16 || (a->new_value_stride_head * esz) % 16)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: new key/value rows must be 16-byte aligned");
+    if (mfma && a->phases != 2) {
+      p.new_k = (const char *)a->new_key; p.new_v = (const char *)a->new_value;
+      p.slot_mapping = a->new_slot_mapping;
+      p.nk_st = a->new_key_stride_row * esz; p.nk_sh = a->new_key_stride_head * esz;
+      p.nv_st = a->new_value_stride_row * esz; p.nv_sh = a->new_value_stride_head * esz;
+    } else if (a->phases != 2) {
+      // vector-ALU path: same semantics as two launches
+      sb_kv_append_args ap;
+      ap.key = a->new_key; ap.value = a->new_value;
+      ap.k_cache = const_cast<void *>(a->k_cache); ap.v_cache = const_cast<void *>(a->v_cache);
+      ap.slot_mapping = a->new_slot_mapping; ap.num_tokens = a->num_rows;
+      ap.num_kv_heads = a->num_kv_heads; ap.head_size = a->head_size; ap.block_size = a->block_size;
+      ap.dtype = a->dtype;
+      ap.key_stride_token = a->new_key_stride_row; ap.key_stride_head = a->new_key_stride_head;
+      ap.value_stride_token = a->new_value_stride_row; ap.value_stride_head = a->new_value_stride_head;
+      ap.cache_stride_block = a->kv_stride_block; ap.cache_stride_row = a->kv_stride_row;
+      ap.cache_stride_head = a->kv_stride_head; ap.num_blocks = 0; ap.stream = a->stream;
+      const int arc = sb_kv_append(&ap);
+      if (arc != SB_OK) return arc;
+    }
+  }
   if (a->phases != 2) {
     if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
                                            (a->flags >> 4) & 7, st, p);

@@ -31,6 +31,8 @@
 // Rows outside [lo, hi) are never read: row indices are clamped into the visible range for the
 // address and masked by their true index for the score, so stale or uninitialised cache rows
 // cannot leak NaNs through 0 * NaN.
+#include <type_traits>
+
 #include "common.h"
 #include "swa_decode_params.h"
 
@@ -160,33 +162,58 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
 #pragma unroll
   for (int j = 0; j < 4; ++j) voff[j] = (4 * g + j) * kv_sr32 + c * 16;
 
-  auto load_chunk = [&](int cc, int t0c, int t1c, int64_t b0, int64_t b1, Chunk &ck) {
-    const char *k0p = p.k + b0, *k1p = p.k + b1, *v0p = p.v + b0, *v1p = p.v + b1;  // wave-uniform bases
-    uint32_t ko0 = koff, ko1 = koff, vo0[4], vo1[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) vo0[j] = vo1[j] = voff[j];
-    if ((cc << 5) < lo || (cc << 5) + 32 > hi) {
-      ko0 = clamp_row(t0c, c) * kv_sr32 + g * 16;
-      ko1 = clamp_row(t1c, c) * kv_sr32 + g * 16;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        vo0[j] = clamp_row(t0c, 4 * g + j) * kv_sr32 + c * 16;
-        vo1[j] = clamp_row(t1c, 4 * g + j) * kv_sr32 + c * 16;
-      }
-    }
+  // Fused append: the newest key (index hi-1) is not in the cache yet. Its K/V rows are read from
+  // the step's key/value tensors wherever a lane's (clamped) row is hi-1, and the wavefront that
+  // owns the last chunk of the window stores them into the cache slot at the very end of the
+  // kernel. (The store must stay behind every block-table lookup: a global store ahead of them
+  // would stop the compiler from proving the table unclobbered, the lookups would turn from
+  // scalar loads into vector loads, and each would then wait for all K/V loads in flight.)
+  const bool fused = p.new_k != nullptr;
+  const char *newk = fused ? p.new_k + r * p.nk_st + (int64_t)kvh * p.nk_sh : nullptr;
+  const char *newv = fused ? p.new_v + r * p.nv_st + (int64_t)kvh * p.nv_sh : nullptr;
+  // ---- loaders ---------------------------------------------------------------------------
+  // Interior chunk (every key visible): wave-uniform bases plus constant 32-bit lane offsets.
+  auto load_interior = [&](int64_t b0, int64_t b1, Chunk &ck) {
+    const char *k0p = p.k + b0, *k1p = p.k + b1, *v0p = p.v + b0, *v1p = p.v + b1;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      ck.k0[s] = load_stream16(k0p + ko0 + s * 64);
-      ck.k1[s] = load_stream16(k1p + ko1 + s * 64);
+      ck.k0[s] = load_stream16(k0p + koff + s * 64);
+      ck.k1[s] = load_stream16(k1p + koff + s * 64);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      ck.v[j] = load_stream16(v0p + vo0[j]);
-      ck.v[4 + j] = load_stream16(v1p + vo1[j]);
+      ck.v[j] = load_stream16(v0p + voff[j]);
+      ck.v[4 + j] = load_stream16(v1p + voff[j]);
+    }
+  };
+  // Edge chunk (first / last chunk of the window; also correct for any other chunk): per-lane
+  // pointers, tiles and rows clamped into the visible range, the newest row taken from the step
+  // inputs when the append is fused.
+  auto load_edge = [&](int cc, Chunk &ck) {
+    const int t0c = clamp_tile(2 * cc), t1c = clamp_tile(2 * cc + 1);
+    const char *k0p = p.k + tile_base(t0c), *k1p = p.k + tile_base(t1c);
+    const char *v0p = p.v + (k0p - p.k), *v1p = p.v + (k1p - p.k);
+    const int newest = fused ? hi - 1 : -1;
+    const int r0 = clamp_row(t0c, c), r1 = clamp_row(t1c, c);
+    const char *pk0 = ((t0c << 4) + r0 == newest) ? newk + g * 16 : k0p + r0 * kv_sr32 + g * 16;
+    const char *pk1 = ((t1c << 4) + r1 == newest) ? newk + g * 16 : k1p + r1 * kv_sr32 + g * 16;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      ck.k0[s] = load_stream16(pk0 + s * 64);
+      ck.k1[s] = load_stream16(pk1 + s * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int q0 = clamp_row(t0c, 4 * g + j), q1 = clamp_row(t1c, 4 * g + j);
+      ck.v[j] = load_stream16(((t0c << 4) + q0 == newest) ? newv + c * 16 : v0p + q0 * kv_sr32 + c * 16);
+      ck.v[4 + j] = load_stream16(((t1c << 4) + q1 == newest) ? newv + c * 16 : v1p + q1 * kv_sr32 + c * 16);
     }
   };
 
-  auto compute_chunk = [&](int ch, const Chunk &ck) {
+  // One chunk of work: S^T = K Q^T, online softmax, O^T += V^T P^T. kMask = edge chunk (keys outside
+  // [lo, hi) are masked by their true index).
+  auto compute_chunk = [&](int ch, const Chunk &ck, auto mask_tag) {
+    constexpr bool kMask = decltype(mask_tag)::value;
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -194,8 +221,8 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
       s1 = Mma<E>::run(ck.k1[s], qb[s], s1);
     }
     float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-    const int i0 = ch << 5;
-    if (i0 < lo || i0 + 32 > hi) {  // edge chunk: mask keys outside [lo, hi) by their true index
+    if constexpr (kMask) {
+      const int i0 = ch << 5;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int i = i0 + ((j >> 2) << 4) + 4 * g + (j & 3);
@@ -237,45 +264,80 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
       acc[mt] = Mma<E>::run(vt, pb, acc[mt]);
     }
   };
+  const std::true_type kMasked{};
+  const std::false_type kUnmasked{};
 
-  // Software pipeline kDepth chunks deep over a ring of kDepth+1 register sets (the loop is unrolled
-  // over the ring so that no registers are copied). Prefetches are unconditional (past the end they
-  // re-read the last chunk of the split), so the number of loads in flight is the same on every
-  // path and the wait before a compute covers only that chunk's loads. Tile bases (block-table
-  // lookups) run one more chunk ahead of the loads.
-  int ch = cb;
-  if (ch < ce) {
-    const int lastc = ce - 1;
-    int t0, t1;
-    int64_t b0, b1;
-    auto locate = [&](int cc) {
-      t0 = clamp_tile(2 * cc);
-      t1 = clamp_tile(2 * cc + 1);
-      b0 = tile_base(t0);
-      b1 = tile_base(t1);
+  // Only the first and the last chunk of a window can hold keys outside [lo, hi). They are taken
+  // out of the streaming loop: their loads go into registers of their own and they are computed
+  // before / after the loop, so the loop body has no clamping, no masking and a fixed number of
+  // loads in flight. The loop is a software pipeline kDepth chunks deep over a ring of kDepth+1
+  // register sets (unrolled over the ring, no register copies); prefetches past the end re-read
+  // the last interior chunk; tile bases (block-table lookups) run one chunk ahead of the loads.
+  // Interior chunks lie wholly inside [lo, hi), so the unclamped interior loader (and the block
+  // table lookups made for it) never leave the sequence; when a split has no interior chunk the
+  // loop and its prologue are skipped altogether.
+  if (cb < ce) {
+    // with a fused append the chunk holding the newest key is an edge chunk even when it is full:
+    // that row is not in the cache yet and only the edge loader reads it from the step inputs
+    auto is_edge = [&](int cc) {
+      return (cc << 5) < lo || (cc << 5) + 32 > hi || (fused && cc == ((hi - 1) >> 5));
     };
-    // loads chunk min(cc, lastc), whose tiles the previous call located, and locates the next one
-    auto issue = [&](int cc, Chunk &dst) {
-      const int lt0 = t0, lt1 = t1;
-      const int64_t lb0 = b0, lb1 = b1;
-      locate(min(cc + 1, lastc));
-      load_chunk(min(cc, lastc), lt0, lt1, lb0, lb1, dst);
-    };
-    Chunk ring[kDepth + 1];
-    locate(ch);
+    const bool e_head = is_edge(cb);
+    const bool e_tail = (ce - 1 > cb) && is_edge(ce - 1);
+    const int ib = cb + (e_head ? 1 : 0), ie = ce - (e_tail ? 1 : 0);  // interior chunks [ib, ie)
+    Chunk head, tail;
+    if (ib < ie) {
+      const int lastc = ie - 1;
+      int64_t b0, b1;
+      auto locate = [&](int cc) {
+        b0 = tile_base(2 * cc);
+        b1 = tile_base(2 * cc + 1);
+      };
+      // loads chunk min(cc, lastc), whose tiles the previous call located, and locates the next one
+      auto issue = [&](int cc, Chunk &dst) {
+        const int64_t lb0 = b0, lb1 = b1;
+        locate(min(cc + 1, lastc));
+        load_interior(lb0, lb1, dst);
+      };
+      Chunk ring[kDepth + 1];
+      int ch = ib;
+      locate(ch);
 #pragma unroll
-    for (int u = 0; u < kDepth; ++u) issue(ch + u, ring[u]);
-    bool more = true;
-    while (more) {
+      for (int u = 0; u < kDepth; ++u) issue(ch + u, ring[u]);
+      // edge loads go behind the prologue: by the time they have landed so has the prologue
+      load_edge(cb, head);
+      load_edge(ce - 1, tail);
+      if (e_head) compute_chunk(cb, head, kMasked);
+      bool more = true;
+      while (more) {
 #pragma unroll
-      for (int u = 0; u <= kDepth; ++u) {
-        if (more) {
-          issue(ch + kDepth, ring[(u + kDepth) % (kDepth + 1)]);
-          compute_chunk(ch, ring[u]);
-          ++ch;
-          more = ch < ce;
+        for (int u = 0; u <= kDepth; ++u) {
+          if (more) {
+            issue(ch + kDepth, ring[(u + kDepth) % (kDepth + 1)]);
+            compute_chunk(ch, ring[u], kUnmasked);
+            ++ch;
+            more = ch < ie;
+          }
         }
       }
+    } else {
+      load_edge(cb, head);
+      load_edge(ce - 1, tail);
+      if (e_head) compute_chunk(cb, head, kMasked);
+    }
+    if (e_tail) compute_chunk(ce - 1, tail, kMasked);
+  }
+
+  // ---- fused append: store the newest K/V row at its slot ---------------------------------
+  if (fused && any && ce == first_chunk + n_chunks && cb < ce && lane < 32) {
+    const int64_t slot = p.slot_mapping[r];
+    if (slot >= 0) {
+      const int64_t blk = slot / p.block_size;
+      const int64_t dst = blk * p.kv_sb + (slot - blk * p.block_size) * p.kv_sr + head_off + (lane & 15) * 16;
+      if (lane < 16)
+        *reinterpret_cast<uint4 *>(const_cast<char *>(p.k) + dst) = *reinterpret_cast<const uint4 *>(newk + lane * 16);
+      else
+        *reinterpret_cast<uint4 *>(const_cast<char *>(p.v) + dst) = *reinterpret_cast<const uint4 *>(newv + (lane & 15) * 16);
     }
   }
 
@@ -323,23 +385,20 @@ namespace sb_host {
 // `rows`, `n_split` give grid x and z; the kv heads are spread over wavefronts and grid y.
 void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
                                   hipStream_t st, const sb::DecodeParams &p) {
-  const int waves = Hkv < 8 ? Hkv : 8;
+  // up to 4 wavefronts (kv heads) per workgroup: one per SIMD, each with the whole register file
+  const int waves = Hkv < 4 ? Hkv : 4;
   const dim3 grid(rows, (unsigned)((Hkv + waves - 1) / waves), n_split), block(64 * waves);
-  // up to 4 wavefronts per workgroup: one per SIMD with the whole register file, deep pipeline;
-  // more: two per SIMD, pipeline one chunk deep
-  if (depth <= 0) depth = waves <= 4 ? 3 : 1;
-  if (waves > 4) depth = 1;
-#define SB_LAUNCH(E, D, T) hipLaunchKernelGGL((swa_decode_split_mfma_kernel<E, D, T>), grid, block, 0, st, p, G, Hkv)
+  // measured on the 7B decode shape: one chunk of prefetch is as fast as two or three
+  if (depth <= 0) depth = 1;
+#define SB_LAUNCH(E, D) hipLaunchKernelGGL((swa_decode_split_mfma_kernel<E, D, 256>), grid, block, 0, st, p, G, Hkv)
   if (dtype == SB_BF16) {
-    if (waves > 4) SB_LAUNCH(sb::BF16, 1, 512);
-    else if (depth == 1) SB_LAUNCH(sb::BF16, 1, 256);
-    else if (depth == 2) SB_LAUNCH(sb::BF16, 2, 256);
-    else SB_LAUNCH(sb::BF16, 3, 256);
+    if (depth == 1) SB_LAUNCH(sb::BF16, 1);
+    else if (depth == 2) SB_LAUNCH(sb::BF16, 2);
+    else SB_LAUNCH(sb::BF16, 3);
   } else {
-    if (waves > 4) SB_LAUNCH(sb::F16, 1, 512);
-    else if (depth == 1) SB_LAUNCH(sb::F16, 1, 256);
-    else if (depth == 2) SB_LAUNCH(sb::F16, 2, 256);
-    else SB_LAUNCH(sb::F16, 3, 256);
+    if (depth == 1) SB_LAUNCH(sb::F16, 1);
+    else if (depth == 2) SB_LAUNCH(sb::F16, 2);
+    else SB_LAUNCH(sb::F16, 3);
   }
 #undef SB_LAUNCH
 }

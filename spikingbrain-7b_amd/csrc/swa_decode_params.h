@@ -22,6 +22,11 @@ struct DecodeParams {
   int64_t q_sr, q_sh, o_sr, o_sh;  // elements
   int64_t kv_sb, kv_sr, kv_sh;     // bytes
   int64_t bt_stride;
+  // fused append (matrix-core kernel only): this step's key/value rows and their cache slots
+  const char *new_k;
+  const char *new_v;
+  const int64_t *slot_mapping;
+  int64_t nk_st, nk_sh, nv_st, nv_sh;  // bytes
 };
 
 }  // namespace sb

@@ -411,9 +411,17 @@ class MetaAttentionImpl:
             key = key.view(-1, self.num_kv_heads, self.head_size)
             value = value.view(-1, self.num_kv_heads, self.head_size)
 
+        # A pure decode step (one new token per sequence, the hot loop) appends and attends in ONE
+        # launch: the attention kernel takes the newest K/V row from `key`/`value` and stores it at
+        # its slot. Every other step appends first, exactly as the reference does (:790-799).
+        fuse_append = (kv_cache.numel() > 0 and key is not None and value is not None
+                       and attn_metadata.num_prefill_tokens == 0 and attn_metadata.num_decode_tokens > 0
+                       and (attn_metadata.max_decode_query_len or 1) == 1
+                       and query.dtype in (torch.bfloat16, torch.float16)
+                       and attn_metadata.slot_mapping is not None)
         if kv_cache.numel() > 0:
             key_cache, value_cache = kv_cache[0], kv_cache[1]
-            if key is not None and value is not None:
+            if key is not None and value is not None and not fuse_append:
                 # all new K/V of the step (prefill and decode tokens) go in with one launch (:790-799)
                 ops.kv_append(key, value, key_cache, value_cache, attn_metadata.slot_mapping.flatten())
 
@@ -445,13 +453,18 @@ class MetaAttentionImpl:
                                    decode_meta.seq_lens_tensor, decode_meta.block_tables,
                                    decode_meta.max_decode_seq_len, output[num_prefill_query_tokens:], window_left)
             else:
-                # one query token per sequence; K/V already appended above (:954-981)
+                # one query token per sequence (:954-981); K/V were appended above, or are appended
+                # by this very launch when the step is a pure decode step
                 n = decode_query.shape[0]
+                fused = {}
+                if fuse_append:
+                    fused = dict(new_key=key[:n], new_value=value[:n],
+                                 new_slot_mapping=decode_meta.slot_mapping.flatten()[:n].contiguous())
                 ops.swa_decode_attention(
                     decode_query, key_cache, value_cache, decode_meta.seq_lens_tensor[:n],
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
                     out=output[num_prefill_query_tokens:],
-                    max_seq_len=decode_meta.max_decode_seq_len or None)
+                    max_seq_len=decode_meta.max_decode_seq_len or None, **fused)
         return output
 
     # -- multi-query forms: every query token becomes one row of the single-query kernel ----

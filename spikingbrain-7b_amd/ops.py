@@ -93,8 +93,15 @@ def swa_decode_attention(
     phases: int = 0,
     force_valu: bool = False,
     pipeline_depth: int = 0,
+    new_key: Optional[torch.Tensor] = None,
+    new_value: Optional[torch.Tensor] = None,
+    new_slot_mapping: Optional[torch.Tensor] = None,
 ):
     """Single-query window attention for each row of q [R, Hq, D].
+
+    new_key/new_value [R, Hkv, D] + new_slot_mapping [R] int64 (all three or none): the newest key
+    of each row (index seq_lens[r]-1) is taken from these tensors and stored into the paged cache
+    at its slot by the same launch (append + attention fused; paged mode, one row per sequence).
 
     paged mode (block_table [S, max_blocks] int32): key_cache/value_cache are
     [num_blocks, block_size, Hkv, D] and strides are taken from them.
@@ -147,6 +154,23 @@ def swa_decode_attention(
             raise ValueError("out must match q in shape and dtype")
         _inner_contiguous(out, "out")
     lse = torch.empty((R, Hq), dtype=torch.float32, device=dev) if return_lse else None
+    fused = {}
+    if new_key is not None or new_value is not None or new_slot_mapping is not None:
+        if new_key is None or new_value is None or new_slot_mapping is None:
+            raise ValueError("new_key, new_value and new_slot_mapping go together")
+        N.require_gpu(q, new_key, new_value, new_slot_mapping)
+        if block_table is None or row_seq is not None:
+            raise ValueError("fused append needs paged mode and one query row per sequence")
+        if new_key.shape != (R, Hkv, D) or new_value.shape != (R, Hkv, D) or new_key.dtype != q.dtype \
+                or new_value.dtype != q.dtype:
+            raise ValueError(f"new_key/new_value must be [{R}, {Hkv}, {D}] of the cache dtype")
+        _inner_contiguous(new_key, "new_key")
+        _inner_contiguous(new_value, "new_value")
+        if new_slot_mapping.dtype != torch.int64 or new_slot_mapping.numel() < R or not new_slot_mapping.is_contiguous():
+            raise ValueError("new_slot_mapping must be a contiguous int64 vector with one entry per row")
+        fused = dict(new_key=N.ptr(new_key), new_value=N.ptr(new_value), new_slot_mapping=N.ptr(new_slot_mapping),
+                     new_key_stride_row=new_key.stride(0), new_key_stride_head=new_key.stride(1),
+                     new_value_stride_row=new_value.stride(0), new_value_stride_head=new_value.stride(1))
     if max_seq_len is None:
         max_seq_len = bound
     if window_left >= 0:
@@ -168,7 +192,7 @@ def swa_decode_attention(
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
         kv_stride_block=kv_strides[0], kv_stride_row=kv_strides[1], kv_stride_head=kv_strides[2],
-        block_table_stride=bt_stride, stream=N.stream_ptr(dev))
+        block_table_stride=bt_stride, stream=N.stream_ptr(dev), **fused)
     N.check(L.sb_swa_decode(C.byref(a)), "swa_decode")
     return (out, lse) if return_lse else out
 
@@ -235,6 +259,16 @@ def copy_blocks(cache_half: torch.Tensor, pairs: torch.Tensor) -> None:
     N.check(N.lib().sb_copy_blocks(N.ptr(cache_half), N.ptr(pairs), pairs.shape[0],
                                    cache_half[0].numel() * esz, cache_half.stride(0) * esz,
                                    N.stream_ptr(dev)), "copy_blocks")
+
+
+def stream_copy(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """Plain streaming device copy of contiguous tensors of equal byte size (a multiple of 16 KiB):
+    the bandwidth yardstick of bench.py and the calibration launch for the HBM byte counters."""
+    dev = N.require_gpu(dst, src)
+    nbytes = src.numel() * src.element_size()
+    if not (dst.is_contiguous() and src.is_contiguous()) or dst.numel() * dst.element_size() != nbytes:
+        raise ValueError("stream_copy needs contiguous tensors of equal byte size")
+    N.check(N.lib().sb_stream_copy(N.ptr(dst), N.ptr(src), nbytes, N.stream_ptr(dev)), "stream_copy")
 
 
 def window_shift(src: Optional[torch.Tensor], dst: torch.Tensor, fresh: Optional[torch.Tensor], *, keep_rows: int,

@@ -195,6 +195,41 @@ def test_config2_full_size_properties(sb, dev):
         assert np.abs(base[b:b + 1].float().cpu().numpy() - ref).max() <= 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("wl,n_split", [(40, 1), (40, 3), (-1, 2), (0, 1)])
+def test_fused_append_equals_append_then_attend(sb, dev, dtype, wl, n_split):
+    """One launch that appends the newest K/V row and attends == kv_append followed by attention:
+    identical cache bytes and identical output bits; padded rows (slot -1) store nothing.
+    (fp32 takes the vector-ALU kernel, where the same call runs the two launches internally.)"""
+    D, bs, Hq, Hkv = 128, 16, 28, 4
+    lens = [1, 16, 17, 33, 64, 100, 129]                      # includes a new token that opens a block
+    kv, tables = paged_problem(lens, bs, Hkv, D, dtype, seed=11)
+    g = torch.Generator().manual_seed(8)
+    R = len(lens)
+    q = torch.randn(R, Hq, D, generator=g).to(dtype).to(dev)
+    k_new = torch.randn(R, Hkv, D, generator=g).to(dtype).to(dev)
+    v_new = torch.randn(R, Hkv, D, generator=g).to(dtype).to(dev)
+    pos = torch.tensor(lens) - 1
+    slots = (tables[torch.arange(R), (pos // bs)].long() * bs + pos % bs)
+    slots[3] = -1                                              # a padded lane
+    slots = slots.to(dev)
+    sl = torch.tensor(lens, dtype=torch.int32, device=dev)
+    a = kv.clone().to(dev)
+    sb.ops.kv_append(k_new, v_new, a[0], a[1], slots)
+    ref = sb.ops.swa_decode_attention(q, a[0], a[1], sl, block_table=tables.to(dev), window_left=wl, n_split=n_split)
+    b = kv.clone().to(dev)
+    out = sb.ops.swa_decode_attention(q, b[0], b[1], sl, block_table=tables.to(dev), window_left=wl, n_split=n_split,
+                                      new_key=k_new, new_value=v_new, new_slot_mapping=slots)
+    live = [r for r in range(R) if r != 3]                     # the output of a padded lane is unspecified
+    assert torch.equal(out[live], ref[live])
+    assert torch.equal(a, b)                                   # same cache bytes, padded lane stored nothing
+    with pytest.raises(ValueError, match="go together"):
+        sb.ops.swa_decode_attention(q, b[0], b[1], sl, block_table=tables.to(dev), new_key=k_new)
+    with pytest.raises(ValueError, match="paged mode"):
+        sb.ops.swa_decode_attention(q, b[0], b[1], sl, block_table=tables.to(dev), row_seq=sl, new_key=k_new,
+                                    new_value=v_new, new_slot_mapping=slots)
+
+
 def test_argument_errors(sb, dev):
     q = torch.zeros(2, 28, 128, device=dev, dtype=torch.bfloat16)
     kv = torch.zeros(2, 4, 16, 4, 128, device=dev, dtype=torch.bfloat16)
