@@ -29,6 +29,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the matrix-core split kernel at the default workload, from rocprofv3 --pmc
+# FETCH_SIZE (253 377 KiB, scaled x2.000 by the same counter's reading of a 1 GiB stream copy) plus
+# WRITE_SIZE (3 768 KiB, scale x1.000): profiles/swa_decode_split_mfma_config2.md. Counters cannot be
+# read from inside this script, so the figure is the recorded one and is only attached when the run
+# is the default workload the profile covers.
+MEASURED_SPLIT_TRAFFIC_BYTES = (253377 * 2 + 3768) * 1024
 HQ, HKV, D, BS, WL = 28, 4, 128, 16, 4096
 E = 2  # bf16
 
@@ -110,6 +116,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--n-split", type=int, default=0)
     ap.add_argument("--unfused", action="store_true", help="append with a separate kv_append launch")
+    ap.add_argument("--force-valu", action="store_true",
+                    help="run the vector-ALU split kernel instead of the matrix-core one (for comparison profiles)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3)")
     args = ap.parse_args()
@@ -132,7 +140,7 @@ def main():
     def attend(c, phases, **kw):
         sb.ops.swa_decode_attention(prob["q"], c[0], c[1], prob["seqlens"], block_table=prob["tables"],
                                     window_left=WL, out=prob["out"], max_seq_len=prob["max_seq_len"],
-                                    n_split=args.n_split, phases=phases, **kw)
+                                    n_split=args.n_split, phases=phases, force_valu=args.force_valu, **kw)
 
     def step(i, events=None):
         """One layer-step as MetaAttentionImpl.forward runs a pure decode batch: the split kernel
@@ -171,6 +179,7 @@ def main():
     k_ms = statistics.mean(a.elapsed_time(b) for a, b in evs)
     achieved = prob["bytes_split_kernel"] / (k_ms * 1e-3) / 1e9
 
+    default_workload = not (args.force_valu or args.unfused or args.n_split)
     n_split = args.n_split or sb._native.lib().sb_swa_decode_auto_split(prob["B"], HKV, prob["max_seq_len"], WL)
     line = {
         "metric": "SWA decode-attn+append GB/s (% of HBM peak) and decode tok/s, 7B shapes, 1 GPU",
@@ -183,9 +192,9 @@ def main():
                    "kv_cache_copies_rotated": n_copies, "bytes_per_step": prob["bytes_step"]},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "decode_tok_per_s_layer_step": round(prob["B"] / (wall / args.steps), 1),
-        "roofline": {"bound": "hbm", "kernel": "swa_decode_split_mfma_kernel<BF16>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": "swa_decode_split_kernel<BF16,7> (vector ALU)" if args.force_valu else "swa_decode_split_mfma_kernel<BF16>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "kernel_ms": round(k_ms, 4), "bytes_per_launch": prob["bytes_split_kernel"]},
+                     "traffic": MEASURED_SPLIT_TRAFFIC_BYTES if default_workload else None, "kernel_ms": round(k_ms, 4), "bytes_per_launch": prob["bytes_split_kernel"]},
     }
 
     # plain streaming copy of 1 GiB in the same run: what this box's HBM gives a copy kernel
