@@ -227,6 +227,50 @@ typedef struct sb_window_shift_args {
 int sb_window_shift(const sb_window_shift_args *args);
 
 /* ------------------------------------------------------------------------------------
+ * Causal sliding-window attention over many query tokens per sequence (prompt prefill,
+ * chunked prefill over the paged cache, multi-token decode); bf16 / fp16, head_size 128,
+ * GQA group size 1, 2, 4 or 7.
+ * Replaces flash_attn_varlen_func as called from
+ *   vllm_hymeta/attention/fa_kernel_metatoken.py:235-253 (via meta_attention.py:827-871,
+ *   window_size = (window_left, 0), causal, block_table optional) and
+ *   hf_7B_model/window_attention.py:186-204.
+ * Query j of sequence s (row cu_seqlens_q[s] + j of q/out) sits at key position
+ *   pos = seq_lens_k[s] - (cu_seqlens_q[s+1] - cu_seqlens_q[s]) + j
+ * and attends keys i with max(0, pos - window_left) <= i <= pos (window_left < 0: all i <= pos).
+ * Keys of sequence s are addressed
+ *   block_table != NULL: key i lives in block block_table[s*block_table_stride + i/block_size],
+ *                        row i % block_size  (k, v = paged caches [blocks, block_size, Hkv, D]);
+ *   block_table == NULL: row kv_start[s] + i of k / v  ([rows, Hkv, D]; kv_start NULL = 0).
+ * The host supplies the tiling of the query axis: tile t covers queries
+ *   tile_q0[t] .. tile_q0[t]+63 of sequence tile_seq[t] (clipped to the sequence's length);
+ * every query must be covered by exactly one tile.
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_swa_prefill_args {
+  const void *q;   /* [total_q, Hq, D] */
+  const void *k;
+  const void *v;
+  void *out;       /* [total_q, Hq, D] */
+  const int32_t *block_table; /* [S, block_table_stride] or NULL */
+  const int64_t *kv_start;    /* [S] or NULL (dense addressing only) */
+  const int32_t *cu_seqlens_q; /* [S+1] */
+  const int32_t *seq_lens_k;   /* [S] */
+  const int32_t *tile_seq;     /* [num_tiles] */
+  const int32_t *tile_q0;      /* [num_tiles] */
+  int64_t num_tiles;
+  int32_t num_q_heads, num_kv_heads, head_size, block_size;
+  int32_t window_left;
+  int32_t dtype;
+  float scale;
+  int64_t q_stride_row, q_stride_head;     /* elements */
+  int64_t out_stride_row, out_stride_head;
+  int64_t kv_stride_block, kv_stride_row, kv_stride_head; /* elements; block stride unused when dense */
+  int64_t block_table_stride;
+  void *stream;
+} sb_swa_prefill_args;
+
+int sb_swa_prefill(const sb_swa_prefill_args *args);
+
+/* ------------------------------------------------------------------------------------
  * Plain device-to-device streaming copy (non-temporal 16-byte lanes), `bytes` a multiple of
  * 16384. No counterpart in the reference: it is the measured bandwidth yardstick printed by
  * bench.py next to the kernels, and the launch of known size that the HBM byte counters

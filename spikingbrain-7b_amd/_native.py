@@ -80,6 +80,22 @@ class WindowShiftArgs(C.Structure):
     ]
 
 
+class SwaPrefillArgs(C.Structure):
+    _fields_ = [
+        ("q", vp), ("k", vp), ("v", vp), ("out", vp),
+        ("block_table", vp), ("kv_start", vp), ("cu_seqlens_q", vp), ("seq_lens_k", vp),
+        ("tile_seq", vp), ("tile_q0", vp),
+        ("num_tiles", i64),
+        ("num_q_heads", i32), ("num_kv_heads", i32), ("head_size", i32), ("block_size", i32),
+        ("window_left", i32), ("dtype", i32), ("scale", f32),
+        ("q_stride_row", i64), ("q_stride_head", i64),
+        ("out_stride_row", i64), ("out_stride_head", i64),
+        ("kv_stride_block", i64), ("kv_stride_row", i64), ("kv_stride_head", i64),
+        ("block_table_stride", i64),
+        ("stream", vp),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/sbcache.h declares
 EXPORTS = {
     "sb_abi_version": (C.c_int, []),
@@ -91,6 +107,7 @@ EXPORTS = {
     "sb_gla_recurrent": (C.c_int, [C.POINTER(GlaRecurrentArgs)]),
     "sb_copy_blocks": (C.c_int, [vp, vp, i64, i64, i64, vp]),
     "sb_window_shift": (C.c_int, [C.POINTER(WindowShiftArgs)]),
+    "sb_swa_prefill": (C.c_int, [C.POINTER(SwaPrefillArgs)]),
     "sb_stream_copy": (C.c_int, [vp, vp, i64, vp]),
 }
 

@@ -34,58 +34,14 @@
 #include <type_traits>
 
 #include "common.h"
+#include "mfma_util.h"
 #include "swa_decode_params.h"
 
 namespace {
 
 using namespace sb;
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-
-template <typename E>
-struct Mma;
-template <>
-struct Mma<BF16> {
-  __device__ static __forceinline__ f32x4_t run(const uint4 &a, const uint4 &b, f32x4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-  }
-  __device__ static __forceinline__ uint32_t pack(float lo, float hi) {
-    bf16x2_t v;
-    v[0] = (__bf16)lo;
-    v[1] = (__bf16)hi;
-    return __builtin_bit_cast(uint32_t, v);
-  }
-};
-template <>
-struct Mma<F16> {
-  __device__ static __forceinline__ f32x4_t run(const uint4 &a, const uint4 &b, f32x4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
-                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-  }
-  __device__ static __forceinline__ uint32_t pack(float lo, float hi) { return pack_f16(lo, hi); }
-};
-
-constexpr float kNegInf = -__builtin_inff();
-
-__device__ __forceinline__ uint32_t perm_lo(uint32_t hi_src, uint32_t lo_src) {
-  return __builtin_amdgcn_perm(hi_src, lo_src, 0x05040100u);  // (hi_src.lo16 << 16) | lo_src.lo16
-}
-__device__ __forceinline__ uint32_t perm_hi(uint32_t hi_src, uint32_t lo_src) {
-  return __builtin_amdgcn_perm(hi_src, lo_src, 0x07060302u);  // (hi_src.hi16 << 16) | lo_src.hi16
-}
-__device__ __forceinline__ uint32_t word(const uint4 &v, int i) {
-  return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
-}
-
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-// K/V bytes are used exactly once per launch: stream them past the caches.
-__device__ __forceinline__ uint4 load_stream16(const char *p) {
-  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
-  return make_uint4(v.x, v.y, v.z, v.w);
-}
+constexpr float kNegInf = kNegInfF;
 
 struct Chunk {
   uint4 k0[4], k1[4];  // K operands of tile 0 / tile 1, one per 32-dim step

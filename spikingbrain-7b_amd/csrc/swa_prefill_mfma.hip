@@ -1,0 +1,352 @@
+// Causal sliding-window attention for many query tokens per sequence (prefill, chunked prefill,
+// multi-token decode), bf16/fp16, on the matrix cores. Keys/values come either from the step's own
+// key/value tensors (plain prompt) or from the paged cache through the block table (chunked prefill,
+// prefix reuse). Replaces the varlen flash-attention call of
+// vllm_hymeta/attention/fa_kernel_metatoken.py:235-253 (window_size=(window_left, 0), causal aligned to
+// the end of the key sequence).
+//
+// Work decomposition
+//   grid = (query tiles of 64 tokens, kv heads); 4 wavefronts per workgroup, wavefront w owns tokens
+//   16w..16w+15 of the tile for NH <= 4 query heads of the kv head (16*NH score rows, no padding); a
+//   GQA group wider than 4 heads is covered by several launches (7 = 4 + 3).
+//   The workgroup walks the union of its tokens' windows in chunks of 32 keys. Each chunk of K and V
+//   (32 rows x 256 B each) is fetched from global memory ONCE per workgroup (wavefront w fetches rows
+//   8w..8w+7 with whole-row 16-byte lanes) into a double-buffered LDS stage whose rows are padded to
+//   272 B, which makes both operand read patterns bank-conflict free; all four wavefronts then read
+//   their MFMA operands from LDS. Global loads of chunk n+1 are in flight while chunk n is computed.
+//   Per chunk and head: S^T = K Q^T (8 MFMA 16x16x32, tokens on the N axis), softmax numerators per
+//   lane for token lane%16 in log2 units, O^T += V^T P^T (8 MFMA). P stays in the lane that produced
+//   it; V^T operands come from an in-register 8x8 transpose shared by the heads.
+//
+// Softmax reference point
+//   The numerators are exp2(s - m_ref) with a per-row reference m_ref that is only raised when some
+//   row of the wavefront scores more than kRaise (log2 units) above it, so they stay below 2^kRaise
+//   (exact in fp32 sums, inside fp16 range). Raising m_ref rescales the output accumulators; that code
+//   sits OUTSIDE the chunk loop (the loop is left and re-entered), because the accumulators live in the
+//   accumulation registers and any branch inside the loop that touches them makes the compiler carry
+//   all of them in vector registers and copy them to and fro on every chunk.
+#include "common.h"
+#include "mfma_util.h"
+
+namespace {
+
+using namespace sb;
+
+struct PrefillParams {
+  const char *q;
+  const char *k;
+  const char *v;
+  char *out;
+  const int32_t *block_table;
+  const int64_t *kv_start;
+  const int32_t *cu_q;        // [S+1] first q/out row of each sequence
+  const int32_t *seq_lens_k;  // [S] keys of each sequence (context + new tokens)
+  const int32_t *tile_seq;    // [tiles] sequence of each 64-token query tile
+  const int32_t *tile_q0;     // [tiles] first query (index inside its sequence) of the tile
+  int G, head_begin;          // query heads per kv head; first of them handled by this launch
+  int block_size, window_left;
+  float scale_log2;
+  int64_t q_sr, q_sh, o_sr, o_sh;  // elements
+  int64_t kv_sb, kv_sr, kv_sh;     // bytes
+  int64_t bt_stride;
+};
+
+constexpr int kRowPad = 272;          // LDS row stride: 256 B of data + 16 B
+constexpr int kStage = 32 * kRowPad;  // one K or V chunk
+constexpr float kNegInf = kNegInfF;
+constexpr float kRaise = 8.f;
+
+template <typename E, int NH>
+__global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams p) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * 2 * kStage];  // [buffer][K|V]
+
+  const int tile = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+
+  const int seq = p.tile_seq[tile];
+  const int q0 = p.tile_q0[tile];
+  const int qrow0 = p.cu_q[seq];
+  const int Lq = p.cu_q[seq + 1] - qrow0;
+  const int Lk = p.seq_lens_k[seq];
+  const int shift = Lk - Lq;  // query j sits at key index shift + j
+  const int wl = p.window_left;
+
+  // keys any token of this workgroup can see: [wg_lo, wg_hi)
+  const int j_last = min(q0 + 63, Lq - 1);
+  const int wg_lo = wl >= 0 ? max(0, shift + q0 - wl) : 0;
+  const int wg_hi = shift + j_last + 1;
+  const int first_tile = wg_lo >> 4, last_tile = (wg_hi - 1) >> 4;
+  const int ch_begin = wg_lo >> 5, ch_end = ((wg_hi - 1) >> 5) + 1;
+
+  // this wavefront's 16 tokens (rows past the end of the sequence repeat its last token; never stored)
+  const int jw0 = min(q0 + 16 * wave, Lq - 1);
+  const int jw_last = min(q0 + 16 * wave + 15, Lq - 1);
+  const int j_mine = min(q0 + 16 * wave + c, Lq - 1);
+  const int my_pos = shift + j_mine;
+  const int my_lo = wl >= 0 ? my_pos - wl : -1;
+  const int head0 = kvh * p.G + p.head_begin;
+
+  // Q^T operands: token lane%16, head h, dims of 16-byte piece 4s+g
+  uint4 qb[NH][4];
+#pragma unroll
+  for (int h = 0; h < NH; ++h)
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      qb[h][s] = *reinterpret_cast<const uint4 *>(
+          p.q + ((int64_t)(qrow0 + j_mine) * p.q_sr + (int64_t)(head0 + h) * p.q_sh + (4 * s + g) * 8) * 2);
+
+  f32x4_t acc[NH][8];
+  float m[NH], l[NH];  // m: reference point of the numerators (log2 units), l: this lane's share of the sum
+#pragma unroll
+  for (int h = 0; h < NH; ++h) {
+    m[h] = kNegInf;
+    l[h] = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) acc[h][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const bool paged = p.block_table != nullptr;
+  const int64_t dense_row0 = (!paged && p.kv_start) ? p.kv_start[seq] : 0;
+  const int64_t head_off = (int64_t)kvh * p.kv_sh;
+  auto tile_base = [&](int t) -> int64_t {  // t inside [first_tile, last_tile], wave-uniform
+    const int i0 = t << 4;
+    if (paged) {
+      const int bi = i0 / p.block_size;
+      const int64_t blk = p.block_table[(int64_t)seq * p.bt_stride + bi];
+      return blk * p.kv_sb + (int64_t)(i0 - bi * p.block_size) * p.kv_sr + head_off;
+    }
+    return (dense_row0 + i0) * p.kv_sr + head_off;
+  };
+
+  // ---- global -> registers: wavefront w fetches rows 8w..8w+7 of the chunk (K and V) ----------
+  // rows outside [wg_lo, wg_hi) are clamped onto the nearest visible key (masked for every token)
+  const int lrow = (wave & 1) * 8 + (lane >> 4);  // row inside the 16-key tile, +4 for the second load
+  uint4 stage_k[2], stage_v[2];
+  auto fetch = [&](int ch) {
+    const int t = min(max(2 * ch + (wave >> 1), first_tile), last_tile);
+    const int64_t base = tile_base(t);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int row = min(max((t << 4) + lrow + 4 * u, wg_lo), wg_hi - 1) - (t << 4);
+      const int64_t off = base + (int64_t)row * p.kv_sr + c * 16;
+      stage_k[u] = load_stream16(p.k + off);
+      stage_v[u] = load_stream16(p.v + off);
+    }
+  };
+  // registers -> LDS stage `buf`
+  auto stash = [&](int buf) {
+    char *sk = smem + buf * 2 * kStage, *sv = sk + kStage;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int kk = wave * 8 + (lane >> 4) + 4 * u;
+      *reinterpret_cast<uint4 *>(sk + kk * kRowPad + c * 16) = stage_k[u];
+      *reinterpret_cast<uint4 *>(sv + kk * kRowPad + c * 16) = stage_v[u];
+    }
+  };
+
+  float sc[NH][8];  // scores of the chunk in flight (raw dot products; -inf where masked)
+  float mx[NH];     // their row maxima, in log2 units
+
+  // scores of chunk `ch` for every head; true when some row needs a higher reference point
+  auto scores = [&](int ch, int buf) -> bool {
+    const char *sk = smem + buf * 2 * kStage;
+    uint4 k0[4], k1[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      k0[s] = *reinterpret_cast<const uint4 *>(sk + c * kRowPad + (4 * s + g) * 16);
+      k1[s] = *reinterpret_cast<const uint4 *>(sk + (16 + c) * kRowPad + (4 * s + g) * 16);
+    }
+    const int c0 = ch << 5;
+    // wholly visible to all 16 tokens: above every token's lower bound, at or below the first token
+    const bool full = (wl < 0 || c0 >= shift + jw_last - wl) && (c0 + 31 <= shift + jw0);
+    bool raise = false;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        s0 = Mma<E>::run(k0[s], qb[h][s], s0);
+        s1 = Mma<E>::run(k1[s], qb[h][s], s1);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        sc[h][j] = s0[j];
+        sc[h][4 + j] = s1[j];
+      }
+      if (!full) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+          if (i > my_pos || i < my_lo) sc[h][j] = kNegInf;
+        }
+      }
+      float t = fmaxf(fmaxf(fmaxf(sc[h][0], sc[h][1]), fmaxf(sc[h][2], sc[h][3])),
+                      fmaxf(fmaxf(sc[h][4], sc[h][5]), fmaxf(sc[h][6], sc[h][7])));
+      t = fmaxf(t, __shfl_xor(t, 16));
+      t = fmaxf(t, __shfl_xor(t, 32));
+      mx[h] = t * p.scale_log2;
+      raise |= mx[h] > m[h] + kRaise;  // also true for the first finite score of a row (m = -inf)
+    }
+    return __builtin_amdgcn_ballot_w64(raise) != 0;
+  };
+
+  // numerators against the current reference points, then O^T += V^T P^T
+  auto accumulate = [&](int buf) {
+    const char *sv = smem + buf * 2 * kStage + kStage;
+    uint4 pb[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      const float m_safe = (m[h] == kNegInf) ? 0.f : m[h];
+      float psum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        sc[h][j] = fast_exp2(fmaf(sc[h][j], p.scale_log2, -m_safe));
+        psum += sc[h][j];
+      }
+      l[h] += psum;
+      pb[h] = make_uint4(Mma<E>::pack(sc[h][0], sc[h][1]), Mma<E>::pack(sc[h][2], sc[h][3]),
+                         Mma<E>::pack(sc[h][4], sc[h][5]), Mma<E>::pack(sc[h][6], sc[h][7]));
+    }
+    uint4 v[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = *reinterpret_cast<const uint4 *>(sv + (4 * g + j) * kRowPad + c * 16);
+      v[4 + j] = *reinterpret_cast<const uint4 *>(sv + (16 + 4 * g + j) * kRowPad + c * 16);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) {
+      const uint4 vt = v_transposed(v, mt);  // built once, used by every head
+#pragma unroll
+      for (int h = 0; h < NH; ++h) acc[h][mt] = Mma<E>::run(vt, pb[h], acc[h][mt]);
+    }
+  };
+
+  // ---- chunk loop: one barrier per chunk, every wavefront visits every chunk -------------------
+  // (chunks outside a wavefront's own band come out fully masked and add zero)
+  fetch(ch_begin);
+  stash(0);
+  __syncthreads();
+  int ch = ch_begin;
+  for (;;) {
+    bool raise = false;
+    for (; ch < ch_end; ++ch) {
+      const int buf = (ch - ch_begin) & 1;
+      const bool more = ch + 1 < ch_end;
+      if (more) fetch(ch + 1);  // global loads fly while this chunk is computed
+      raise = scores(ch, buf);
+      if (raise) break;
+      accumulate(buf);
+      if (more) stash(buf ^ 1);
+      __syncthreads();
+    }
+    if (!raise) break;
+    // rare: lift the reference points to the running maxima and rescale, then finish this chunk
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      const float m_new = fmaxf(m[h], mx[h]);
+      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+      const float alpha = fast_exp2(m[h] - m_safe);
+      m[h] = m_new;
+      l[h] *= alpha;
+#pragma unroll
+      for (int mt = 0; mt < 8; ++mt) acc[h][mt] *= alpha;
+    }
+    {
+      const int buf = (ch - ch_begin) & 1;
+      const bool more = ch + 1 < ch_end;
+      accumulate(buf);
+      if (more) stash(buf ^ 1);
+      __syncthreads();
+      ++ch;
+    }
+  }
+
+  // ---- epilogue: lane (g, c) owns token c, dims 32g + 8i + mt of each head ---------------------
+  if (q0 + 16 * wave + c < Lq) {
+    const int64_t orow = (int64_t)(qrow0 + q0 + 16 * wave + c) * p.o_sr;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      float lt = l[h];
+      lt += __shfl_xor(lt, 16);
+      lt += __shfl_xor(lt, 32);
+      const float inv = lt > 0.f ? 1.f / lt : 0.f;
+      char *dst = p.out + (orow + (int64_t)(head0 + h) * p.o_sh + 32 * g) * 2;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint4 o;
+        o.x = E::pack(acc[h][0][i] * inv, acc[h][1][i] * inv);
+        o.y = E::pack(acc[h][2][i] * inv, acc[h][3][i] * inv);
+        o.z = E::pack(acc[h][4][i] * inv, acc[h][5][i] * inv);
+        o.w = E::pack(acc[h][6][i] * inv, acc[h][7][i] * inv);
+        *reinterpret_cast<uint4 *>(dst + 16 * i) = o;
+      }
+    }
+  }
+}
+
+template <typename E>
+void launch_prefill(int nh, dim3 grid, hipStream_t st, const PrefillParams &p) {
+  switch (nh) {
+    case 1: hipLaunchKernelGGL((swa_prefill_kernel<E, 1>), grid, dim3(256), 0, st, p); break;
+    case 2: hipLaunchKernelGGL((swa_prefill_kernel<E, 2>), grid, dim3(256), 0, st, p); break;
+    case 3: hipLaunchKernelGGL((swa_prefill_kernel<E, 3>), grid, dim3(256), 0, st, p); break;
+    default: hipLaunchKernelGGL((swa_prefill_kernel<E, 4>), grid, dim3(256), 0, st, p); break;
+  }
+}
+
+}  // namespace
+
+extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
+  using namespace sb_host;
+  if (!a) return fail(SB_ERR_INVALID, "sb_swa_prefill: null args");
+  if (a->num_tiles < 0) return fail(SB_ERR_INVALID, "sb_swa_prefill: negative num_tiles");
+  if (a->num_tiles == 0) return SB_OK;
+  if (!a->q || !a->k || !a->v || !a->out || !a->cu_seqlens_q || !a->seq_lens_k || !a->tile_seq || !a->tile_q0)
+    return fail(SB_ERR_INVALID, "sb_swa_prefill: null tensor pointer");
+  if (a->head_size != 128)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: head_size %d (only 128 is built)", a->head_size);
+  if (a->dtype != SB_BF16 && a->dtype != SB_F16)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: dtype must be bf16 or fp16");
+  if (a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_q_heads % a->num_kv_heads != 0)
+    return fail(SB_ERR_INVALID, "sb_swa_prefill: num_q_heads must be a positive multiple of num_kv_heads");
+  if (!(a->scale > 0.f)) return fail(SB_ERR_INVALID, "sb_swa_prefill: scale must be positive");
+  if (a->block_table && (a->block_size < 16 || a->block_size % 16 != 0))
+    return fail(SB_ERR_INVALID, "sb_swa_prefill: block_size %d must be a multiple of 16", a->block_size);
+  if (a->num_tiles > 0x7fffffffLL || a->num_kv_heads > 65535)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: grid too large");
+  const int64_t es[] = {a->q_stride_row, a->q_stride_head, a->out_stride_row, a->out_stride_head,
+                        a->kv_stride_block, a->kv_stride_row, a->kv_stride_head};
+  for (int64_t s : es)
+    if ((s * 2) % 16 != 0)
+      return fail(SB_ERR_INVALID, "sb_swa_prefill: stride %lld elements is not 16-byte aligned", (long long)s);
+  if ((reinterpret_cast<uintptr_t>(a->q) | reinterpret_cast<uintptr_t>(a->k) | reinterpret_cast<uintptr_t>(a->v) |
+       reinterpret_cast<uintptr_t>(a->out)) & 15u)
+    return fail(SB_ERR_INVALID, "sb_swa_prefill: q/k/v/out base not 16-byte aligned");
+
+  PrefillParams p;
+  p.q = (const char *)a->q; p.k = (const char *)a->k; p.v = (const char *)a->v; p.out = (char *)a->out;
+  p.block_table = a->block_table; p.kv_start = a->kv_start;
+  p.cu_q = a->cu_seqlens_q; p.seq_lens_k = a->seq_lens_k; p.tile_seq = a->tile_seq; p.tile_q0 = a->tile_q0;
+  p.G = a->num_q_heads / a->num_kv_heads; p.head_begin = 0;
+  p.block_size = a->block_size > 0 ? a->block_size : 16; p.window_left = a->window_left;
+  p.scale_log2 = a->scale * sb::kLog2e;
+  p.q_sr = a->q_stride_row; p.q_sh = a->q_stride_head; p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
+  p.kv_sb = a->kv_stride_block * 2; p.kv_sr = a->kv_stride_row * 2; p.kv_sh = a->kv_stride_head * 2;
+  p.bt_stride = a->block_table_stride;
+
+  const dim3 grid((unsigned)a->num_tiles, (unsigned)a->num_kv_heads);
+  for (int h0 = 0; h0 < p.G; h0 += 4) {  // a GQA group is covered 4 heads at a time
+    p.head_begin = h0;
+    const int nh = p.G - h0 < 4 ? p.G - h0 : 4;
+    if (a->dtype == SB_BF16) launch_prefill<BF16>(nh, grid, (hipStream_t)a->stream, p);
+    else launch_prefill<F16>(nh, grid, (hipStream_t)a->stream, p);
+    const int rc = check_launch("swa_prefill_kernel");
+    if (rc != SB_OK) return rc;
+  }
+  return SB_OK;
+}

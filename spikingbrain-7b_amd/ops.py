@@ -197,6 +197,127 @@ def swa_decode_attention(
     return (out, lse) if return_lse else out
 
 
+PREFILL_TILE = 64  # query tokens per workgroup of the prefill kernel
+
+
+class PrefillPlan:
+    """Device-side description of one prefill launch: per-sequence query offsets and key counts, and
+    the cover of the query axis by 64-token tiles. Built on the host from the step's length lists
+    (which the scheduler already has as Python ints), uploaded with one copy."""
+
+    __slots__ = ("cu_seqlens_q", "seq_lens_k", "tile_seq", "tile_q0", "num_tiles", "total_q", "num_seqs", "max_k",
+                 "total_k")
+
+    def __init__(self, query_lens, seq_lens_k, device):
+        query_lens = [int(x) for x in query_lens]
+        seq_lens_k = query_lens if seq_lens_k is None else [int(x) for x in seq_lens_k]
+        if len(seq_lens_k) != len(query_lens):
+            raise ValueError("query_lens and seq_lens_k must have one entry per sequence")
+        cu, tile_seq, tile_q0 = [0], [], []
+        for s, (lq, lk) in enumerate(zip(query_lens, seq_lens_k)):
+            if lq < 0 or lk < lq:
+                raise ValueError(f"sequence {s}: {lq} queries need at least as many keys, got {lk}")
+            cu.append(cu[-1] + lq)
+            for q0 in range(0, lq, PREFILL_TILE):
+                tile_seq.append(s)
+                tile_q0.append(q0)
+        S, T = len(query_lens), len(tile_seq)
+        packed = torch.tensor(cu + seq_lens_k + tile_seq + tile_q0, dtype=torch.int32).to(device, non_blocking=False)
+        self.cu_seqlens_q = packed[:S + 1]
+        self.seq_lens_k = packed[S + 1:2 * S + 1]
+        self.tile_seq = packed[2 * S + 1:2 * S + 1 + T]
+        self.tile_q0 = packed[2 * S + 1 + T:]
+        self.num_tiles, self.total_q, self.num_seqs = T, cu[-1], S
+        self.max_k, self.total_k = max(seq_lens_k, default=0), sum(seq_lens_k)
+
+
+def swa_prefill_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    *,
+    query_lens=None,
+    seq_lens_k=None,
+    plan: Optional[PrefillPlan] = None,
+    block_table: Optional[torch.Tensor] = None,
+    kv_start: Optional[torch.Tensor] = None,
+    num_kv_heads: Optional[int] = None,
+    window_left: int = -1,
+    scale: Optional[float] = None,
+    out: Optional[torch.Tensor] = None,
+):
+    """Causal sliding-window attention for q [total_q, Hq, D] packed sequence after sequence.
+
+    query_lens / seq_lens_k: per-sequence host ints (keys default to the queries: plain prompt), or a
+    prebuilt `plan`. Query j of a sequence sits at key position seq_len_k - query_len + j.
+    paged (block_table [S, max_blocks] int32): k/v are the caches [num_blocks, block_size, Hkv, D].
+    dense (block_table None): k/v are [rows, Hkv, D]; keys of sequence s start at row kv_start[s]
+    (int64 device vector; default: the same packing as q, which needs seq_lens_k == query_lens)."""
+    dev = N.require_gpu(q, k, v, block_table, kv_start, out)
+    if q.dim() != 3:
+        raise ValueError(f"q must be [total_q, num_heads, head_size], got {tuple(q.shape)}")
+    Tq, Hq, D = q.shape
+    _inner_contiguous(q, "q")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k and v must share one dtype")
+    if plan is None:
+        if query_lens is None:
+            raise ValueError("give query_lens (and seq_lens_k) or a prebuilt plan")
+        plan = PrefillPlan(query_lens, seq_lens_k, dev)
+    if plan.total_q != Tq:
+        raise ValueError(f"query_lens sum to {plan.total_q}, q has {Tq} rows")
+    if k.shape != v.shape or k.stride() != v.stride():
+        raise ValueError("k and v must have identical shapes and strides")
+    _inner_contiguous(k, "k")
+    if block_table is not None:
+        if k.dim() != 4:
+            raise ValueError("paged caches must be [num_blocks, block_size, num_kv_heads, head_size]")
+        nb, bs, Hkv, Dc = k.shape
+        strides = (k.stride(0), k.stride(1), k.stride(2))
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1 \
+                or block_table.shape[0] < plan.num_seqs:
+            raise ValueError("block_table must be a 2-D int32 tensor with contiguous rows, one per sequence")
+        if block_table.shape[1] * bs < plan.max_k:
+            raise ValueError(f"block_table rows hold {block_table.shape[1] * bs} keys, a sequence has {plan.max_k}")
+        bt_stride = block_table.stride(0)
+    else:
+        if k.dim() != 3:
+            raise ValueError("dense k/v must be [rows, num_kv_heads, head_size]")
+        Hkv, Dc, bs, bt_stride = k.shape[1], k.shape[2], 16, 0
+        strides = (0, k.stride(0), k.stride(1))
+        if kv_start is None:
+            kv_start = plan.cu_seqlens_q.to(torch.int64)
+        if kv_start.dtype != torch.int64 or not kv_start.is_contiguous() or kv_start.numel() < plan.num_seqs:
+            raise ValueError("kv_start must be a contiguous int64 vector with one entry per sequence")
+    if num_kv_heads is not None and num_kv_heads != Hkv:
+        raise ValueError(f"num_kv_heads {num_kv_heads} does not match k's {Hkv}")
+    if Dc != D:
+        raise ValueError(f"head_size mismatch: q {D}, k {Dc}")
+    if scale is None:
+        scale = D ** -0.5
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        if out.shape != q.shape or out.dtype != q.dtype:
+            raise ValueError("out must match q in shape and dtype")
+        _inner_contiguous(out, "out")
+    if plan.num_tiles == 0:
+        return out
+    a = N.SwaPrefillArgs(
+        q=N.ptr(q), k=N.ptr(k), v=N.ptr(v), out=N.ptr(out),
+        block_table=N.ptr(block_table), kv_start=N.ptr(kv_start) if block_table is None else None,
+        cu_seqlens_q=N.ptr(plan.cu_seqlens_q), seq_lens_k=N.ptr(plan.seq_lens_k),
+        tile_seq=N.ptr(plan.tile_seq), tile_q0=N.ptr(plan.tile_q0), num_tiles=plan.num_tiles,
+        num_q_heads=Hq, num_kv_heads=Hkv, head_size=D, block_size=bs, window_left=int(window_left),
+        dtype=N.dtype_code(q.dtype), scale=float(scale),
+        q_stride_row=q.stride(0), q_stride_head=q.stride(1),
+        out_stride_row=out.stride(0), out_stride_head=out.stride(1),
+        kv_stride_block=strides[0], kv_stride_row=strides[1], kv_stride_head=strides[2],
+        block_table_stride=bt_stride, stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_swa_prefill(C.byref(a)), "swa_prefill")
+    return out
+
+
 def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
                   slot_idx: Optional[torch.Tensor] = None, scale: Optional[float] = None,
                   out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -1,0 +1,140 @@
+"""Many-query causal sliding-window attention (prefill kernel) vs the float64 oracle.
+Tolerance (BASELINE): max-abs 2e-2 for bf16 (5e-3 for fp16) against fp64 mathematics on the same
+bf16/fp16 inputs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as A
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3}
+
+
+def dense_problem(query_lens, ctx_lens, Hq, Hkv, D, dtype, seed, spread=1.0):
+    g = torch.Generator().manual_seed(seed)
+    Tq = sum(query_lens)
+    lens_k = [a + b for a, b in zip(query_lens, ctx_lens)]
+    Tk = sum(lens_k)
+    q = (torch.randn(Tq, Hq, D, generator=g) * spread).to(dtype)
+    k = (torch.randn(Tk, Hkv, D, generator=g) * spread).to(dtype)
+    v = torch.randn(Tk, Hkv, D, generator=g).to(dtype)
+    cu_q = np.concatenate([[0], np.cumsum(query_lens)])
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)])
+    return q, k, v, lens_k, cu_q, cu_k
+
+
+def check(out, q, k, v, cu_q, cu_k, scale, wl, tol):
+    ref = A.varlen_window_attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), cu_q, cu_k, scale, wl)
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    err = np.abs(got - ref).max()
+    assert err <= tol, f"max abs err {err}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Hq,Hkv", [(28, 4), (8, 8), (8, 2), (6, 2), (5, 1)])
+@pytest.mark.parametrize("wl", [-1, 0, 1, 31, 64, 100])
+def test_prompt_prefill_vs_oracle(sb, dev, dtype, Hq, Hkv, wl):
+    """Plain prompts (keys = the step's own tokens): ragged lengths around the 16/32/64 boundaries."""
+    D = 128
+    query_lens = [1, 15, 16, 17, 33, 64, 65, 127, 130]
+    q, k, v, lens_k, cu_q, cu_k = dense_problem(query_lens, [0] * len(query_lens), Hq, Hkv, D, dtype, seed=Hq + wl)
+    scale = D ** -0.5
+    out = sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), query_lens=query_lens, window_left=wl,
+                                       scale=scale)
+    check(out, q, k, v, cu_q, cu_k, scale, wl, TOL[dtype])
+
+
+@pytest.mark.parametrize("wl", [-1, 50, 256])
+def test_dense_context_offsets(sb, dev, wl):
+    """Queries at the end of longer key sequences (multi-token decode over a dense cache)."""
+    D, Hq, Hkv = 128, 28, 4
+    query_lens = [3, 64, 20, 1, 70]
+    ctx = [200, 5, 0, 77, 300]
+    q, k, v, lens_k, cu_q, cu_k = dense_problem(query_lens, ctx, Hq, Hkv, D, torch.bfloat16, seed=wl + 3)
+    out = sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), query_lens=query_lens, seq_lens_k=lens_k,
+                                       kv_start=torch.tensor(cu_k[:-1], dtype=torch.int64, device=dev),
+                                       window_left=wl, scale=D ** -0.5)
+    check(out, q, k, v, cu_q, cu_k, D ** -0.5, wl, 2e-2)
+
+
+@pytest.mark.parametrize("bs", [16, 32, 256])
+@pytest.mark.parametrize("wl", [-1, 40, 300])
+def test_paged_chunked_prefill_vs_oracle(sb, dev, bs, wl):
+    """Chunked prefill: keys (context + the chunk) live in the paged cache in a shuffled block order."""
+    D, Hq, Hkv = 128, 28, 4
+    query_lens = [64, 10, 130, 1]
+    ctx = [100, 0, 515, 33]
+    dtype = torch.bfloat16
+    q, k, v, lens_k, cu_q, cu_k = dense_problem(query_lens, ctx, Hq, Hkv, D, dtype, seed=bs + wl)
+    g = torch.Generator().manual_seed(9)
+    need = [(n + bs - 1) // bs for n in lens_k]
+    nb = sum(need) + 3
+    perm = torch.randperm(nb, generator=g)
+    kc = torch.randn(nb, bs, Hkv, D, generator=g).to(dtype)   # stale rows hold finite garbage
+    vc = torch.randn(nb, bs, Hkv, D, generator=g).to(dtype)
+    tables = torch.zeros(len(lens_k), max(need), dtype=torch.int32)
+    p = 0
+    for s, n in enumerate(need):
+        tables[s, :n] = perm[p:p + n]; p += n
+        for i in range(lens_k[s]):
+            blk = int(tables[s, i // bs])
+            kc[blk, i % bs] = k[cu_k[s] + i]
+            vc[blk, i % bs] = v[cu_k[s] + i]
+    out = sb.ops.swa_prefill_attention(q.to(dev), kc.to(dev), vc.to(dev), query_lens=query_lens, seq_lens_k=lens_k,
+                                       block_table=tables.to(dev), window_left=wl, scale=D ** -0.5)
+    check(out, q, k, v, cu_q, cu_k, D ** -0.5, wl, 2e-2)
+
+
+def test_growing_scores_raise_the_reference(sb, dev):
+    """Keys whose scores keep growing along the sequence force the softmax reference point up many
+    times (the rescale path outside the chunk loop), including jumps far above the raise threshold."""
+    D, Hq, Hkv = 128, 8, 2
+    L = 300
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(L, Hq, D, generator=g).abs()
+    k = torch.randn(L, Hkv, D, generator=g).abs() * torch.linspace(0.05, 3.0, L)[:, None, None]
+    k[150:] *= 2.0
+    v = torch.randn(L, Hkv, D, generator=g)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    cu = np.array([0, L])
+    for wl in (-1, 100):
+        out = sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), query_lens=[L], window_left=wl,
+                                           scale=D ** -0.5)
+        check(out, q, k, v, cu, cu, D ** -0.5, wl, 2e-2)
+
+
+def test_matches_decode_kernel_row_by_row(sb, dev):
+    """The many-query kernel and the single-query kernel agree on the same paged cache."""
+    D, Hq, Hkv, bs, wl = 128, 28, 4, 16, 90
+    L = 200
+    g = torch.Generator().manual_seed(11)
+    nb = (L + bs - 1) // bs
+    kc = torch.randn(nb, bs, Hkv, D, generator=g).bfloat16().to(dev)
+    vc = torch.randn(nb, bs, Hkv, D, generator=g).bfloat16().to(dev)
+    q = torch.randn(L, Hq, D, generator=g).bfloat16().to(dev)
+    table = torch.arange(nb, dtype=torch.int32, device=dev)[None]
+    pre = sb.ops.swa_prefill_attention(q, kc, vc, query_lens=[L], block_table=table, window_left=wl)
+    dec = sb.ops.swa_decode_attention(q, kc, vc, torch.arange(1, L + 1, dtype=torch.int32, device=dev),
+                                      block_table=table, row_seq=torch.zeros(L, dtype=torch.int32, device=dev),
+                                      window_left=wl)
+    assert (pre.float() - dec.float()).abs().max().item() <= 2e-2
+
+
+def test_prefill_argument_errors(sb, dev):
+    q = torch.zeros(4, 8, 128, dtype=torch.bfloat16, device=dev)
+    kv = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ValueError):
+        sb.ops.swa_prefill_attention(q, kv, kv, query_lens=[3])            # lengths do not cover q
+    with pytest.raises(ValueError):
+        sb.ops.swa_prefill_attention(q, kv, kv, query_lens=[4], seq_lens_k=[2])   # fewer keys than queries
+    with pytest.raises(NotImplementedError):
+        sb.ops.swa_prefill_attention(q.float(), kv.float(), kv.float(), query_lens=[4])
+    q64 = torch.zeros(4, 8, 64, dtype=torch.bfloat16, device=dev)
+    kv64 = torch.zeros(4, 2, 64, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(NotImplementedError):
+        sb.ops.swa_prefill_attention(q64, kv64, kv64, query_lens=[4])
+    out = sb.ops.swa_prefill_attention(q[:0], kv, kv, query_lens=[])       # empty step
+    assert out.shape == (0, 8, 128)
