@@ -236,7 +236,8 @@ int sb_window_shift(const sb_window_shift_args *args);
  *   hf_7B_model/window_attention.py:186-204.
  * Query j of sequence s (row cu_seqlens_q[s] + j of q/out) sits at key position
  *   pos = seq_lens_k[s] - (cu_seqlens_q[s+1] - cu_seqlens_q[s]) + j
- * and attends keys i with max(0, pos - window_left) <= i <= pos (window_left < 0: all i <= pos).
+ * and attends keys i with max(0, pos - window_left) <= i <= pos (window_left < 0: all i <= pos),
+ * further restricted to i >= key_lo[s] when key_lo is given; a query with no visible key gets zeros.
  * Keys of sequence s are addressed
  *   block_table != NULL: key i lives in block block_table[s*block_table_stride + i/block_size],
  *                        row i % block_size  (k, v = paged caches [blocks, block_size, Hkv, D]);
@@ -252,6 +253,7 @@ typedef struct sb_swa_prefill_args {
   void *out;       /* [total_q, Hq, D] */
   const int32_t *block_table; /* [S, block_table_stride] or NULL */
   const int64_t *kv_start;    /* [S] or NULL (dense addressing only) */
+  const int32_t *key_lo;      /* [S] or NULL: keys below this index are invisible (left padding) */
   const int32_t *cu_seqlens_q; /* [S+1] */
   const int32_t *seq_lens_k;   /* [S] */
   const int32_t *tile_seq;     /* [num_tiles] */

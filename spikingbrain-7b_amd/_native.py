@@ -83,7 +83,7 @@ class WindowShiftArgs(C.Structure):
 class SwaPrefillArgs(C.Structure):
     _fields_ = [
         ("q", vp), ("k", vp), ("v", vp), ("out", vp),
-        ("block_table", vp), ("kv_start", vp), ("cu_seqlens_q", vp), ("seq_lens_k", vp),
+        ("block_table", vp), ("kv_start", vp), ("key_lo", vp), ("cu_seqlens_q", vp), ("seq_lens_k", vp),
         ("tile_seq", vp), ("tile_q0", vp),
         ("num_tiles", i64),
         ("num_q_heads", i32), ("num_kv_heads", i32), ("head_size", i32), ("block_size", i32),

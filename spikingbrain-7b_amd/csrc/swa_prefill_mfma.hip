@@ -39,6 +39,7 @@ struct PrefillParams {
   char *out;
   const int32_t *block_table;
   const int64_t *kv_start;
+  const int32_t *key_lo;      // [S] first visible key of each sequence, or null
   const int32_t *cu_q;        // [S+1] first q/out row of each sequence
   const int32_t *seq_lens_k;  // [S] keys of each sequence (context + new tokens)
   const int32_t *tile_seq;    // [tiles] sequence of each 64-token query tile
@@ -78,8 +79,10 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
 
   // keys any token of this workgroup can see: [wg_lo, wg_hi)
   const int j_last = min(q0 + 63, Lq - 1);
-  const int wg_lo = wl >= 0 ? max(0, shift + q0 - wl) : 0;
   const int wg_hi = shift + j_last + 1;
+  const int klo = p.key_lo ? max(p.key_lo[seq], 0) : 0;
+  // (kept inside the sequence even when padding hides every key: such rows end up fully masked)
+  const int wg_lo = min(max(wl >= 0 ? shift + q0 - wl : 0, klo), wg_hi - 1);
   const int first_tile = wg_lo >> 4, last_tile = (wg_hi - 1) >> 4;
   const int ch_begin = wg_lo >> 5, ch_end = ((wg_hi - 1) >> 5) + 1;
 
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
   const int jw_last = min(q0 + 16 * wave + 15, Lq - 1);
   const int j_mine = min(q0 + 16 * wave + c, Lq - 1);
   const int my_pos = shift + j_mine;
-  const int my_lo = wl >= 0 ? my_pos - wl : -1;
+  const int my_lo = max(wl >= 0 ? my_pos - wl : 0, klo);
   const int head0 = kvh * p.G + p.head_begin;
 
   // Q^T operands: token lane%16, head h, dims of 16-byte piece 4s+g
@@ -163,7 +166,7 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
     }
     const int c0 = ch << 5;
     // wholly visible to all 16 tokens: above every token's lower bound, at or below the first token
-    const bool full = (wl < 0 || c0 >= shift + jw_last - wl) && (c0 + 31 <= shift + jw0);
+    const bool full = (wl < 0 || c0 >= shift + jw_last - wl) && c0 >= klo && (c0 + 31 <= shift + jw0);
     bool raise = false;
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
@@ -330,7 +333,7 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
 
   PrefillParams p;
   p.q = (const char *)a->q; p.k = (const char *)a->k; p.v = (const char *)a->v; p.out = (char *)a->out;
-  p.block_table = a->block_table; p.kv_start = a->kv_start;
+  p.block_table = a->block_table; p.kv_start = a->kv_start; p.key_lo = a->key_lo;
   p.cu_q = a->cu_seqlens_q; p.seq_lens_k = a->seq_lens_k; p.tile_seq = a->tile_seq; p.tile_q0 = a->tile_q0;
   p.G = a->num_q_heads / a->num_kv_heads; p.head_begin = 0;
   p.block_size = a->block_size > 0 ? a->block_size : 16; p.window_left = a->window_left;

@@ -124,6 +124,24 @@ class MetaAttentionMetadata:
     num_encoder_tokens: Optional[int] = None
     cross_slot_mapping: Optional[torch.Tensor] = None
     cross_block_tables: Optional[torch.Tensor] = None
+    # Not in the reference's metadata: host copies of the per-sequence query and key counts (the
+    # builder has them as Python ints anyway). With them the many-query kernel lays out its 64-token
+    # tiles without reading a device tensor back; without them every query token runs as one row of
+    # the single-query kernel.
+    query_lens: Optional[List[int]] = None
+    host_seq_lens: Optional[List[int]] = None
+    _prefill_plan: Any = None
+
+    def prefill_plan(self, device) -> Any:
+        """Tile layout of this (sub)step for ops.swa_prefill_attention, built once and shared by
+        every layer; None when the host lengths are not known."""
+        lens_k = self.seq_lens if self.seq_lens is not None else self.host_seq_lens
+        if self.query_lens is None or lens_k is None:
+            return None
+        if self._prefill_plan is None:
+            n = len(self.query_lens)
+            self._prefill_plan = ops.PrefillPlan(self.query_lens, list(lens_k[:n]), device)
+        return self._prefill_plan
 
     @property
     def is_all_encoder_attn_metadata_set(self) -> bool:
@@ -161,7 +179,8 @@ class MetaAttentionMetadata:
             use_cuda_graph=False,
             encoder_seq_lens=self.encoder_seq_lens, encoder_seq_lens_tensor=self.encoder_seq_lens_tensor,
             encoder_seq_start_loc=self.encoder_seq_start_loc, max_encoder_seq_len=self.max_encoder_seq_len,
-            cross_slot_mapping=self.cross_slot_mapping, cross_block_tables=self.cross_block_tables)
+            cross_slot_mapping=self.cross_slot_mapping, cross_block_tables=self.cross_block_tables,
+            query_lens=head(self.query_lens, n), host_seq_lens=head(self.seq_lens, n))
         return self._cached_prefill_metadata
 
     @property
@@ -191,7 +210,9 @@ class MetaAttentionMetadata:
             use_cuda_graph=self.use_cuda_graph,
             encoder_seq_lens=self.encoder_seq_lens, encoder_seq_lens_tensor=self.encoder_seq_lens_tensor,
             encoder_seq_start_loc=self.encoder_seq_start_loc, max_encoder_seq_len=self.max_encoder_seq_len,
-            cross_slot_mapping=self.cross_slot_mapping, cross_block_tables=self.cross_block_tables)
+            cross_slot_mapping=self.cross_slot_mapping, cross_block_tables=self.cross_block_tables,
+            query_lens=tail(self.query_lens, n),
+            host_seq_lens=tail(self.seq_lens if self.seq_lens is not None else self.host_seq_lens, n))
         return self._cached_decode_metadata
 
 
@@ -314,6 +335,7 @@ class MetaAttentionMetadataBuilder:
             context_lens_tensor=h2d(self.context_lens, torch.int),
             block_tables=block_tables,
             use_cuda_graph=use_captured_graph,
+            query_lens=list(query_lens),
         )
 
 
@@ -443,7 +465,8 @@ class MetaAttentionImpl:
                 assert prefill_meta.query_start_loc is not None
                 self._varlen_paged(query, key_cache, value_cache, prefill_meta.query_start_loc,
                                    prefill_meta.seq_lens_tensor, prefill_meta.block_tables,
-                                   max(prefill_meta.seq_lens), output[:num_prefill_query_tokens], window_left)
+                                   max(prefill_meta.seq_lens), output[:num_prefill_query_tokens], window_left,
+                                   meta=prefill_meta)
         if decode_meta := attn_metadata.decode_metadata:
             assert decode_meta.max_decode_query_len is not None
             if decode_meta.max_decode_query_len > 1:
@@ -451,7 +474,8 @@ class MetaAttentionImpl:
                 assert decode_meta.query_start_loc is not None
                 self._varlen_paged(decode_query, key_cache, value_cache, decode_meta.query_start_loc,
                                    decode_meta.seq_lens_tensor, decode_meta.block_tables,
-                                   decode_meta.max_decode_seq_len, output[num_prefill_query_tokens:], window_left)
+                                   decode_meta.max_decode_seq_len, output[num_prefill_query_tokens:], window_left,
+                                   meta=decode_meta)
             else:
                 # one query token per sequence (:954-981); K/V were appended above, or are appended
                 # by this very launch when the step is a pure decode step
@@ -478,15 +502,31 @@ class MetaAttentionImpl:
         j = torch.arange(num_tokens, device=qsl.device) - qsl[row_seq]
         return row_seq, j, lens
 
+    @staticmethod
+    def _plan_for(meta, q):
+        """Tile plan for the many-query matrix-core kernel, or None when it cannot take the step
+        (fp32, host lengths unknown, rows padded beyond the sequences' tokens)."""
+        if q.dtype not in (torch.bfloat16, torch.float16):
+            return None
+        plan = meta.prefill_plan(q.device)
+        if plan is None or plan.total_q != q.shape[0]:
+            return None
+        return plan
+
     def _varlen_inflight(self, q, k, v, meta, out, window_left):
         T = q.shape[0]
         if T == 0:
             return
-        row_seq, j, _ = self._rows(meta.query_start_loc, T)
-        seq_lens_row = (j + 1).to(torch.int32)
         if k.stride() != v.stride():
             v = v.contiguous()
             k = k.contiguous()
+        plan = self._plan_for(meta, q)
+        if plan is not None and plan.total_k <= k.shape[0]:
+            ops.swa_prefill_attention(q, k, v, plan=plan, window_left=window_left, scale=self.scale, out=out,
+                                      kv_start=meta.seq_start_loc.to(torch.int64)[:-1].contiguous())
+            return
+        row_seq, j, _ = self._rows(meta.query_start_loc, T)
+        seq_lens_row = (j + 1).to(torch.int32)
         ops.swa_decode_attention(
             q, k, v, seq_lens_row, kv_start=meta.seq_start_loc.to(torch.int64)[:-1].contiguous(),
             row_seq=row_seq.to(torch.int32), kv_strides=(0, k.stride(0), k.stride(1)),
@@ -494,9 +534,14 @@ class MetaAttentionImpl:
             max_seq_len=meta.max_prefill_seq_len or None)
 
     def _varlen_paged(self, q, key_cache, value_cache, query_start_loc, seq_lens_tensor, block_tables,
-                      max_seq_len, out, window_left):
+                      max_seq_len, out, window_left, meta=None):
         T = q.shape[0]
         if T == 0:
+            return
+        plan = self._plan_for(meta, q) if meta is not None else None
+        if plan is not None and block_tables.shape[1] * key_cache.shape[1] >= plan.max_k:
+            ops.swa_prefill_attention(q, key_cache, value_cache, plan=plan, block_table=block_tables,
+                                      window_left=window_left, scale=self.scale, out=out)
             return
         row_seq, j, lens = self._rows(query_start_loc, T)
         # query j of a run of n queries in a sequence of L keys sits at key index L - n + j

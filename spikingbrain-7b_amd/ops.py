@@ -241,6 +241,8 @@ def swa_prefill_attention(
     plan: Optional[PrefillPlan] = None,
     block_table: Optional[torch.Tensor] = None,
     kv_start: Optional[torch.Tensor] = None,
+    key_lo: Optional[torch.Tensor] = None,
+    kv_strides: Optional[Tuple[int, int]] = None,
     num_kv_heads: Optional[int] = None,
     window_left: int = -1,
     scale: Optional[float] = None,
@@ -252,8 +254,12 @@ def swa_prefill_attention(
     prebuilt `plan`. Query j of a sequence sits at key position seq_len_k - query_len + j.
     paged (block_table [S, max_blocks] int32): k/v are the caches [num_blocks, block_size, Hkv, D].
     dense (block_table None): k/v are [rows, Hkv, D]; keys of sequence s start at row kv_start[s]
-    (int64 device vector; default: the same packing as q, which needs seq_lens_k == query_lens)."""
-    dev = N.require_gpu(q, k, v, block_table, kv_start, out)
+    (int64 device vector; default: the same packing as q, which needs seq_lens_k == query_lens).
+    With kv_strides = (row, head) in elements (and num_kv_heads), k/v may be any tensors whose
+    element offset for (sequence s, key i, head h) is (kv_start[s] + i)*row + h*head.
+    key_lo [S] int32: keys below key_lo[s] are invisible (left padding); a query that sees no key
+    gets zeros."""
+    dev = N.require_gpu(q, k, v, block_table, kv_start, key_lo, out)
     if q.dim() != 3:
         raise ValueError(f"q must be [total_q, num_heads, head_size], got {tuple(q.shape)}")
     Tq, Hq, D = q.shape
@@ -281,22 +287,34 @@ def swa_prefill_attention(
             raise ValueError(f"block_table rows hold {block_table.shape[1] * bs} keys, a sequence has {plan.max_k}")
         bt_stride = block_table.stride(0)
     else:
-        if k.dim() != 3:
-            raise ValueError("dense k/v must be [rows, num_kv_heads, head_size]")
-        Hkv, Dc, bs, bt_stride = k.shape[1], k.shape[2], 16, 0
-        strides = (0, k.stride(0), k.stride(1))
-        if kv_start is None:
-            kv_start = plan.cu_seqlens_q.to(torch.int64)
+        bs, bt_stride = 16, 0
+        if kv_strides is not None:
+            if num_kv_heads is None or kv_start is None:
+                raise ValueError("kv_strides needs num_kv_heads and kv_start")
+            Hkv, Dc = num_kv_heads, k.shape[-1]
+            strides = (0, int(kv_strides[0]), int(kv_strides[1]))
+        else:
+            if k.dim() != 3:
+                raise ValueError("dense k/v must be [rows, num_kv_heads, head_size]")
+            Hkv, Dc = k.shape[1], k.shape[2]
+            strides = (0, k.stride(0), k.stride(1))
+            if kv_start is None:
+                if plan.total_k > k.shape[0]:
+                    raise ValueError(f"k has {k.shape[0]} rows, the sequences hold {plan.total_k} keys")
+                kv_start = plan.cu_seqlens_q.to(torch.int64)
         if kv_start.dtype != torch.int64 or not kv_start.is_contiguous() or kv_start.numel() < plan.num_seqs:
             raise ValueError("kv_start must be a contiguous int64 vector with one entry per sequence")
     if num_kv_heads is not None and num_kv_heads != Hkv:
         raise ValueError(f"num_kv_heads {num_kv_heads} does not match k's {Hkv}")
     if Dc != D:
         raise ValueError(f"head_size mismatch: q {D}, k {Dc}")
+    if key_lo is not None and (key_lo.dtype != torch.int32 or not key_lo.is_contiguous()
+                               or key_lo.numel() < plan.num_seqs):
+        raise ValueError("key_lo must be a contiguous int32 vector with one entry per sequence")
     if scale is None:
         scale = D ** -0.5
     if out is None:
-        out = torch.empty_like(q)
+        out = torch.empty((Tq, Hq, D), dtype=q.dtype, device=dev)
     else:
         if out.shape != q.shape or out.dtype != q.dtype:
             raise ValueError("out must match q in shape and dtype")
@@ -306,7 +324,7 @@ def swa_prefill_attention(
     a = N.SwaPrefillArgs(
         q=N.ptr(q), k=N.ptr(k), v=N.ptr(v), out=N.ptr(out),
         block_table=N.ptr(block_table), kv_start=N.ptr(kv_start) if block_table is None else None,
-        cu_seqlens_q=N.ptr(plan.cu_seqlens_q), seq_lens_k=N.ptr(plan.seq_lens_k),
+        key_lo=N.ptr(key_lo), cu_seqlens_q=N.ptr(plan.cu_seqlens_q), seq_lens_k=N.ptr(plan.seq_lens_k),
         tile_seq=N.ptr(plan.tile_seq), tile_q0=N.ptr(plan.tile_q0), num_tiles=plan.num_tiles,
         num_q_heads=Hq, num_kv_heads=Hkv, head_size=D, block_size=bs, window_left=int(window_left),
         dtype=N.dtype_code(q.dtype), scale=float(scale),

@@ -17,6 +17,25 @@ from . import ops
 from .hf_cache import Cache
 
 
+# query runs at least this long use the many-query kernel; shorter ones (speculative / multi-token
+# decode) run as rows of the single-query kernel, which wastes no tile rows on them
+PREFILL_MIN_QUERIES = 16
+
+_plans: dict = {}
+
+
+def _uniform_plan(B: int, Q: int, K: int, dev: torch.device):
+    """Tile plan for B sequences of Q queries over K keys each (every layer of a forward pass asks
+    for the same one)."""
+    key = (B, Q, K, dev)
+    plan = _plans.get(key)
+    if plan is None:
+        if len(_plans) >= 64:
+            _plans.clear()
+        plan = _plans[key] = ops.PrefillPlan([Q] * B, [K] * B, dev)
+    return plan
+
+
 def _kv_start_rows(k: torch.Tensor) -> Optional[torch.Tensor]:
     """Row offset of each batch entry, in units of k.stride(2); None if it is not a whole number."""
     B = k.shape[0]
@@ -76,6 +95,15 @@ def sliding_window_attention(
 
     q_rows = query_states.transpose(1, 2).reshape(B * Q, Hq, D)
     dev = q_rows.device
+    if Q >= PREFILL_MIN_QUERIES and q_rows.dtype in (torch.bfloat16, torch.float16) and D == 128:
+        # prompt-sized query runs go to the matrix-core kernel (64-token tiles)
+        pad = None
+        if attention_mask is not None:
+            pad = (K - (attention_mask[:, -K:] != 0).sum(dim=1)).to(torch.int32).contiguous()
+        out = ops.swa_prefill_attention(
+            q_rows, k, v, plan=_uniform_plan(B, Q, K, dev), kv_start=kv_start, key_lo=pad,
+            kv_strides=(k.stride(2), k.stride(1)), num_kv_heads=Hkv, window_left=window_left, scale=D ** -0.5)
+        return out.view(B, Q, Hq, D)
     j = torch.arange(Q, device=dev, dtype=torch.int32)
     seq_lens_row = (K - Q + 1 + j).repeat(B)                       # query j sits at key index K - Q + j
     row_seq = torch.arange(B, device=dev, dtype=torch.int32).repeat_interleave(Q)

@@ -123,6 +123,62 @@ def test_matches_decode_kernel_row_by_row(sb, dev):
     assert (pre.float() - dec.float()).abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("wl", [-1, 70])
+def test_key_lo_hides_left_padding(sb, dev, wl):
+    """Keys below key_lo are invisible; queries inside the padding get zeros."""
+    D, Hq, Hkv = 128, 8, 2
+    lens = [100, 64, 130]
+    pads = [0, 63, 77]
+    g = torch.Generator().manual_seed(21)
+    T = sum(lens)
+    q = torch.randn(T, Hq, D, generator=g).bfloat16()
+    k = torch.randn(T, Hkv, D, generator=g).bfloat16()
+    v = torch.randn(T, Hkv, D, generator=g).bfloat16()
+    out = sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), query_lens=lens, window_left=wl,
+                                       key_lo=torch.tensor(pads, dtype=torch.int32, device=dev)).float().cpu().numpy()
+    start = 0
+    for n, pad in zip(lens, pads):
+        sl = slice(start + pad, start + n)                      # the real tokens form their own sequence
+        ref = A.varlen_window_attention(q[sl].float().numpy(), k[sl].float().numpy(), v[sl].float().numpy(),
+                                        [0, n - pad], [0, n - pad], D ** -0.5, wl)
+        assert np.abs(out[sl] - ref).max() <= 2e-2
+        assert (out[start:start + pad] == 0).all()
+        start += n
+
+
+def test_hf_layer_prompt_bf16_left_padded(sb, dev):
+    """The HuggingFace-side layer slice routes bf16 prompts through the many-query kernel:
+    left-padded batch, window 512, then cached decode steps (single-query kernel)."""
+    from oracle.hf_cache import OracleCache
+    HQ, HKV, D, W = 28, 4, 128, 512
+    prompts = [300, 511, 700, 900]
+    L = max(prompts)
+    g = torch.Generator().manual_seed(0)
+    mask = np.zeros((4, L), np.int64)
+    for b, n in enumerate(prompts):
+        mask[b, L - n:] = 1
+    prod, orc = sb.Cache(), OracleCache()
+    for step in range(3):
+        n = L if step == 0 else 1
+        k = torch.randn(4, HKV, n, D, generator=g).bfloat16()
+        v = torch.randn(4, HKV, n, D, generator=g).bfloat16()
+        q = torch.randn(4, HQ, n, D, generator=g).bfloat16()
+        if step:
+            mask = np.concatenate([mask, np.ones((4, 1), np.int64)], axis=1)
+        has = orc.get_seq_length(0) > 0
+        kc, vc = orc.update(attn_state=(k.float().numpy(), v.float().numpy()), layer_idx=0, offset=n,
+                            cache_kwargs={"window_size": W})["attn_state"]
+        kk, vv = (kc, vc) if has else (k.float().numpy(), v.float().numpy())
+        ref = A.sdpa_window_attention(q.float().numpy(), kk, vv, W, mask)
+        got = sb.sliding_window_attention(q.to(dev), k.to(dev), v.to(dev), W, prod, 0,
+                                          attention_mask=torch.from_numpy(mask).to(dev), cache_window_size=W,
+                                          window_left=W - 1).permute(0, 2, 1, 3).float().cpu().numpy()
+        assert np.abs(got - ref).max() <= 2e-2
+        if step == 0:
+            for b, n_real in enumerate(prompts):
+                assert (got[b, :, :L - n_real] == 0).all()
+
+
 def test_prefill_argument_errors(sb, dev):
     q = torch.zeros(4, 8, 128, dtype=torch.bfloat16, device=dev)
     kv = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device=dev)
