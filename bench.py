@@ -109,6 +109,119 @@ def cpu_baseline(seconds_budget=12.0, sample_B=8):
                        f"{med * 1e3:.1f} ms/step")
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def bench_prefill(sb, dev, S=16, L=8192, iters=5):
+    """BASELINE config 4 through the backend: 16 prompts x 8192 new tokens, window_left 4096, one layer.
+    Times MetaAttentionImpl.forward (bulk KV append + causal sliding-window attention) for a plain
+    prompt run (keys in flight, only in-window tokens get slots) and for a chunked-prefill run (every
+    token stored, attention reads the paged cache); metadata is built once, outside the timed region."""
+    res = {}
+    g = torch.Generator(device=dev).manual_seed(0)
+    T = S * L
+    q = torch.randn(T, HQ, D, device=dev, dtype=torch.bfloat16, generator=g)
+    k = torch.randn(T, HKV, D, device=dev, dtype=torch.bfloat16, generator=g)
+    v = torch.randn(T, HKV, D, device=dev, dtype=torch.bfloat16, generator=g)
+    out = torch.empty_like(q)
+    visits = S * ((WL + 1) * (WL + 2) // 2 + (L - WL - 1) * (WL + 1))      # sum_i min(i + 1, window_left + 1)
+    flops = 4 * HQ * D * visits
+    impl = sb.MetaAttentionImpl(HQ, D, D ** -0.5, HKV, None, WL + 1, "auto")
+    for name, chunked in (("prompt_inflight_kv", False), ("chunked_paged_kv", True)):
+        nb = S * ((L if chunked else WL) // BS + 3) + 8
+        runner = sb.SwaCacheRunner(1, nb, BS, WL, HKV, D, torch.bfloat16, dev, max_seqs=S, max_chunk_tokens=L)
+        for s in range(S):
+            runner.add_seq(s)
+        t0 = time.perf_counter()
+        meta = runner.build_step([(s, L) for s in range(S)], [], chunked_prefill=chunked)
+        host_ms = (time.perf_counter() - t0) * 1e3
+        stored = int((meta.slot_mapping >= 0).sum())
+
+        def run():
+            impl.forward(None, q, k, v, None, None, None, runner.kv_caches[0], meta, output=out)
+
+        run()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        for a, b in evs:
+            a.record()
+            run()
+            b.record()
+        torch.cuda.synchronize()
+        ms = statistics.median(a.elapsed_time(b) for a, b in evs)
+        # the append alone
+        eva = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        for a, b in eva:
+            a.record()
+            sb.ops.kv_append(k, v, runner.kv_caches[0][0], runner.kv_caches[0][1], meta.slot_mapping)
+            b.record()
+        torch.cuda.synchronize()
+        ms_app = statistics.median(a.elapsed_time(b) for a, b in eva)
+        app_bytes = stored * 2 * HKV * D * E * 2 + T * 8
+        res[name] = {"ms_append_plus_attention": round(ms, 3), "ms_append": round(ms_app, 4),
+                     "tokens_stored": stored, "append_GBps": round(app_bytes / (ms_app * 1e-3) / 1e9, 1),
+                     "attention_TFLOPs": round(flops / ((ms - ms_app) * 1e-3) / 1e12, 1),
+                     "mfma_frac_of_bf16_peak": round(flops / ((ms - ms_app) * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "prefill_tok_per_s_layer": round(T / (ms * 1e-3)), "host_metadata_ms": round(host_ms, 1)}
+        del runner
+    res["workload"] = f"BASELINE config 4: {S} x {L} new tokens, window_left {WL}, block_size {BS}, one layer"
+    res["attention_flops"] = flops
+    return res
+
+
+def bench_hybrid(sb, dev, B=256, steps=128, warmup=4):
+    """BASELINE config 5: the cache work of 128 consecutive decode steps of the 28-layer stack
+    (14 GLA state layers + 14 paged SWA layers, one shared block table), B=256, every sequence at a
+    logical context of 512k tokens (window-saturated), real appends, eviction and block recycling."""
+    c = sb.HybridDecodeCache(B, randomize=True, device=dev)
+    c.start(512 * 1024)
+    g = torch.Generator(device=dev).manual_seed(1)
+    q = torch.randn(B, HQ, D, device=dev, dtype=torch.bfloat16, generator=g)
+    k = torch.randn(B, HKV, D, device=dev, dtype=torch.bfloat16, generator=g)
+    v = torch.randn(B, HKV, D, device=dev, dtype=torch.bfloat16, generator=g)
+    gq, gk, gv = (torch.randn(B, HQ, 1, D, device=dev, dtype=torch.bfloat16, generator=g) for _ in range(3))
+    gg = torch.nn.functional.logsigmoid(torch.randn(B, HQ, 1, D, device=dev, generator=g)) / 16
+    out = torch.empty(B, HQ, D, device=dev, dtype=torch.bfloat16)
+
+    def layers(meta):
+        for li in range(c.num_layers):
+            if li % 2 == 0:
+                c.gla_layer(li, gq, gk, gv, gg)
+            else:
+                c.swa_layer(li, q, k, v, meta, out)
+
+    host = []
+    for _ in range(warmup):
+        layers(c.step_metadata())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        th = time.perf_counter()
+        meta = c.step_metadata()
+        host.append(time.perf_counter() - th)
+        layers(meta)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    gpu = []
+    for _ in range(8):  # device time of one step with the host out of the way
+        meta = c.step_metadata()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        layers(meta)
+        b.record()
+        torch.cuda.synchronize()
+        gpu.append(a.elapsed_time(b))
+    by = c.bytes_per_step()
+    gpu_ms = statistics.median(gpu)
+    return {"workload": f"BASELINE config 5: 28-layer hybrid decode step, B={B}, logical context 512k, "
+                        f"{steps} consecutive steps", "ms_per_step": round(ms, 3),
+            "decode_tok_per_s": round(B / (ms * 1e-3)), "bytes_per_step": by,
+            "GBps": round(by / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "gpu_ms_per_step": round(gpu_ms, 3), "host_metadata_ms_per_step": round(statistics.mean(host) * 1e3, 3),
+            "host_overhead_share": round(max(0.0, ms - gpu_ms) / ms, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -119,7 +232,8 @@ def main():
     ap.add_argument("--force-valu", action="store_true",
                     help="run the vector-ALU split kernel instead of the matrix-core one (for comparison profiles)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3)")
+    ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
+                                                    "28-layer hybrid decode step (config 5)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1",
@@ -232,6 +346,12 @@ def main():
         line["gla_state_update"] = {"workload": "BASELINE config 3: B=64, H=28, fp32 state", "kernel_ms": round(ms3, 4),
                                     "GBps": round(bytes3 / (ms3 * 1e-3) / 1e9, 1),
                                     "frac_hbm_peak": round(bytes3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+        del states
+        line["prefill"] = bench_prefill(sb, dev)
+        torch.cuda.empty_cache()
+        line["hybrid_decode"] = bench_hybrid(sb, dev)
+        torch.cuda.empty_cache()
 
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()

@@ -9,9 +9,12 @@ and registered in `sys.modules` as `spikingbrain_7b_amd`.
   gla                                 GLA recurrent step + constant-size state cache
   block_manager.WindowBlockManager    window eviction / block recycling / slot mapping
   ops                                 tensor-level wrappers over the C ABI (include/sbcache.h)
+  decode_driver.HybridDecodeCache     the 28-layer stack's cache work per generated token
 """
-from . import _native, block_manager, gla, hf_cache, meta_attention, ops, runner, window_attention  # noqa: F401
+from . import (_native, block_manager, decode_driver, gla, hf_cache, meta_attention, ops, runner,  # noqa: F401
+               window_attention)
 from .block_manager import PAD_SLOT_ID, WindowBlockManager, compute_slot_mapping, compute_slot_mapping_start_idx  # noqa: F401
+from .decode_driver import HybridDecodeCache  # noqa: F401
 from .gla import GLACacheManager, GLACacheParams, fused_recurrent_gla, my_fused_recurrent_gla  # noqa: F401
 from .hf_cache import Cache  # noqa: F401
 from .meta_attention import (AttentionType, MetaAttentionBackend, MetaAttentionImpl,  # noqa: F401
@@ -23,5 +26,5 @@ __all__ = [
     "Cache", "sliding_window_attention", "MetaAttentionBackend", "MetaAttentionImpl", "MetaAttentionMetadata",
     "MetaAttentionMetadataBuilder", "AttentionType", "GLACacheManager", "GLACacheParams",
     "my_fused_recurrent_gla", "fused_recurrent_gla", "WindowBlockManager", "PAD_SLOT_ID",
-    "compute_slot_mapping", "compute_slot_mapping_start_idx", "ops", "SwaCacheRunner",
+    "compute_slot_mapping", "compute_slot_mapping_start_idx", "ops", "SwaCacheRunner", "HybridDecodeCache",
 ]

@@ -1,0 +1,107 @@
+"""Cache side of the hybrid stack's decode loop: what the reference's model forward does to the
+caches on every generated token, with the projections, norms and MLPs left to the caller.
+
+Layer order follows hf_7B_model/configuration_gla_swa.py:75 (even layers GLA, odd layers sliding
+window). Per step and sequence
+  * every GLA layer reads and rewrites its [H, D, D] fp32 state at the sequence's slot
+    (vllm_hymeta/model_for_7B/gla_attention.py:223-235 -> my_fused_recurrent_gla);
+  * every SWA layer appends the new K/V row at the step's slot and attends inside the window
+    (vllm_hymeta/attention/meta_attention.py:767-799, 920-981), all SWA layers sharing ONE block table
+    and slot mapping (each layer has its own KV tensor indexed by the same block ids);
+  * the block manager evicts the block that left the window and hands its id to the block the
+    sequence grows into (one recycle per sequence every block_size steps once the window is full).
+
+The step metadata comes from the block manager's vectorised host path (numpy over the batch; only
+sequences that cross a block boundary do per-sequence work) and three small uploads.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import numpy as np
+import torch
+
+from . import ops
+from .block_manager import WindowBlockManager
+from .meta_attention import MetaAttentionBackend, MetaAttentionImpl, MetaAttentionMetadata
+
+
+class HybridDecodeCache:
+    def __init__(self, batch: int, *, num_layers: int = 28, num_heads: int = 28, num_kv_heads: int = 4,
+                 head_size: int = 128, block_size: int = 16, window_left: int = 4096,
+                 dtype: torch.dtype = torch.bfloat16, device="cuda:0", num_blocks: Optional[int] = None,
+                 randomize: bool = False, seed: int = 0):
+        self.device = torch.device(device)
+        self.batch, self.num_layers = batch, num_layers
+        self.H, self.Hkv, self.D, self.bs, self.wl = num_heads, num_kv_heads, head_size, block_size, window_left
+        self.swa_layers = [i for i in range(num_layers) if i % 2 == 1]
+        self.gla_layers = [i for i in range(num_layers) if i % 2 == 0]
+        per_seq = (window_left + 1) // block_size + 2
+        self.num_blocks = num_blocks if num_blocks is not None else batch * per_seq + 8
+        self.manager = WindowBlockManager(self.num_blocks, block_size, window_left, batch)
+        shape = MetaAttentionBackend.get_kv_cache_shape(self.num_blocks, block_size, num_kv_heads, head_size)
+        g = torch.Generator(device=self.device).manual_seed(seed)
+
+        def alloc(shape, dt, std):
+            if randomize:
+                return torch.randn(shape, dtype=torch.float32, device=self.device, generator=g).mul_(std).to(dt) \
+                    if dt != torch.float32 else torch.randn(shape, dtype=dt, device=self.device, generator=g).mul_(std)
+            return torch.zeros(shape, dtype=dt, device=self.device)
+
+        self.kv_caches: List[torch.Tensor] = [alloc(shape, dtype, 1.0) for _ in self.swa_layers]
+        # [n_gla_layers, slots, H, D, D] fp32, as vllm_hymeta/model_for_7B/modeling_gla_swa.py:348-356
+        self.gla_state = alloc((len(self.gla_layers), batch, num_heads, head_size, head_size), torch.float32, 0.02)
+        self.slot_idx = torch.arange(batch, dtype=torch.int32, device=self.device)
+        self.impl = MetaAttentionImpl(num_heads, head_size, head_size ** -0.5, num_kv_heads, None, window_left + 1,
+                                      "auto")
+        self.seq_ids = list(range(batch))
+        for s in self.seq_ids:
+            self.manager.add_seq(s)
+        self._gla_out = torch.empty(batch, num_heads, 1, head_size, dtype=dtype, device=self.device)
+        self._layer = _Layer()
+
+    def start(self, context_len: int) -> None:
+        """Every sequence already holds `context_len` tokens: only the blocks inside the window get
+        ids (what a prompt run leaves behind); the cache contents are whatever the tensors hold."""
+        for s in self.seq_ids:
+            self.manager.append_tokens(s, context_len, True)
+
+    def step_metadata(self) -> MetaAttentionMetadata:
+        """Advance every sequence by one token (eviction + allocation) and build the decode-only
+        metadata the SWA layers of this step share."""
+        mgr = self.manager
+        slots = mgr.decode_step(self.seq_ids)
+        tables, seqlens, _ = mgr.kernel_view(self.seq_ids)
+        dev = self.device
+        packed = torch.from_numpy(np.concatenate([slots, seqlens.astype(np.int64)])).to(dev, non_blocking=True)
+        B = self.batch
+        return MetaAttentionMetadata(
+            num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B,
+            slot_mapping=packed[:B], seq_lens=None, seq_lens_tensor=packed[B:].to(torch.int32),
+            max_prefill_seq_len=0, max_decode_seq_len=int(seqlens.max()), context_lens_tensor=None,
+            block_tables=torch.from_numpy(tables).to(dev, non_blocking=True), use_cuda_graph=False,
+            max_query_len=1, max_decode_query_len=1)
+
+    def gla_layer(self, layer_idx: int, q, k, v, g, out=None) -> torch.Tensor:
+        """q, k, v, g [B, H, 1, D]; the layer's state is advanced in place. Returns o [B, H, 1, D]."""
+        out = self._gla_out if out is None else out
+        ops.gla_recurrent(q, k, v, g, self.gla_state[layer_idx // 2], self.slot_idx, self.D ** -0.5, out)
+        return out
+
+    def swa_layer(self, layer_idx: int, q, k, v, meta: MetaAttentionMetadata, out) -> torch.Tensor:
+        """q [B, Hq, D], k/v [B, Hkv, D]: append + window attention for one SWA layer."""
+        return self.impl.forward(self._layer, q, k, v, None, None, None, self.kv_caches[layer_idx // 2], meta, out)
+
+    def bytes_per_step(self) -> int:
+        """Algorithmic HBM bytes of one decode step over all layers (window-saturated sequences)."""
+        e = self.kv_caches[0].element_size()
+        n_keys = np.minimum(self.manager.n_tokens[:self.batch], self.wl + 1)
+        swa = int(n_keys.sum()) * self.Hkv * self.D * 2 * e + self.batch * (2 * self.H * self.D * e
+                                                                           + 4 * self.Hkv * self.D * e)
+        gla = self.batch * self.H * (2 * self.D * self.D * 4 + 3 * self.D * e + self.D * 4 + self.D * e)
+        return len(self.swa_layers) * swa + len(self.gla_layers) * gla
+
+
+class _Layer:
+    _k_scale_float = 1.0
+    _v_scale_float = 1.0

@@ -1,0 +1,66 @@
+"""The hybrid stack's per-token cache work (GLA state layers interleaved with paged sliding-window
+layers sharing one block table) stepped next to the oracle: numpy window-cache model, numpy paged
+caches, float64 GLA recurrence. Sequences start window-saturated at a long logical context, so
+every block_size steps each one evicts a block and recycles its id.
+Bit-exact: slot mapping, block tables, view lengths, every byte of every layer's KV tensor.
+Within tolerance: attention outputs 2e-2 (bf16); GLA outputs 2e-2 + half an ulp of bf16, states 1e-4 rel."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as A
+from oracle import gla as G
+from oracle import paged as P
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("ctx", [5, 1000])
+def test_hybrid_decode_steps_vs_oracle(sb, dev, ctx):
+    B, L, H, HKV, D, bs, wl = 3, 4, 8, 2, 128, 16, 40
+    drv = sb.HybridDecodeCache(B, num_layers=L, num_heads=H, num_kv_heads=HKV, head_size=D, block_size=bs,
+                               window_left=wl, device=dev, randomize=True, seed=3)
+    drv.start(ctx)
+    model = P.WindowCacheModel(drv.num_blocks, bs, wl)
+    for s in range(B):
+        model.add_seq(s)
+        model.append_tokens(s, ctx, True)
+    kc = [c[0].float().cpu().numpy() for c in drv.kv_caches]
+    vc = [c[1].float().cpu().numpy() for c in drv.kv_caches]
+    state = drv.gla_state.cpu().numpy().astype(np.float64)
+    g = torch.Generator().manual_seed(ctx)
+    for step in range(2 * bs + 3):
+        meta = drv.step_metadata()
+        slots = [model.append_tokens(s, 1, False)[0] for s in range(B)]
+        assert meta.slot_mapping.cpu().tolist() == slots
+        views = [model.view(s) for s in range(B)]
+        lens = [v[1] for v in views]
+        assert meta.seq_lens_tensor.cpu().tolist() == lens
+        width = max(len(v[0]) for v in views)
+        tables = np.zeros((B, width), np.int32)
+        for s, v in enumerate(views):
+            tables[s, :len(v[0])] = v[0]
+        assert np.array_equal(meta.block_tables.cpu().numpy(), tables)
+        for li in range(L):
+            if li % 2 == 0:
+                q, k, v = (torch.randn(B, H, 1, D, generator=g).bfloat16() for _ in range(3))
+                gate = torch.nn.functional.logsigmoid(torch.randn(B, H, 1, D, generator=g)) / 16
+                o = drv.gla_layer(li, q.to(dev), k.to(dev), v.to(dev), gate.to(dev)).float().cpu().numpy()[:, :, 0]
+                ref = G.gla_step(q.float().numpy()[:, :, 0], k.float().numpy()[:, :, 0], v.float().numpy()[:, :, 0],
+                                 gate.numpy()[:, :, 0], state[li // 2])
+                assert (np.abs(o - ref) <= 2e-2 + np.abs(ref) * 2.0 ** -8).all()
+                got_state = drv.gla_state[li // 2].cpu().numpy()
+                assert np.abs(got_state - state[li // 2]).max() <= 1e-4 * max(1.0, np.abs(state[li // 2]).max())
+            else:
+                q = torch.randn(B, H, D, generator=g).bfloat16()
+                k = torch.randn(B, HKV, D, generator=g).bfloat16()
+                v = torch.randn(B, HKV, D, generator=g).bfloat16()
+                out = torch.full((B, H, D), float("nan"), dtype=torch.bfloat16, device=dev)
+                drv.swa_layer(li, q.to(dev), k.to(dev), v.to(dev), meta, out)
+                j = li // 2
+                P.kv_append(k.float().numpy(), v.float().numpy(), kc[j], vc[j], slots)
+                ref = A.paged_decode_attention(q.float().numpy(), kc[j], vc[j], tables, lens, D ** -0.5, wl)
+                assert np.abs(out.float().cpu().numpy() - ref).max() <= 2e-2
+                assert np.array_equal(drv.kv_caches[j][0].float().cpu().numpy(), kc[j])
+                assert np.array_equal(drv.kv_caches[j][1].float().cpu().numpy(), vc[j])
+    assert drv.manager.free_stack() == model.free
