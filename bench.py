@@ -234,6 +234,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
                                                     "28-layer hybrid decode step (config 5)")
+    ap.add_argument("--only", choices=("prefill", "hybrid"), default=None,
+                    help="run just that section and print its JSON (short runs for profiling one kernel)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1",
@@ -245,6 +247,13 @@ def main():
     sb._native.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.only == "prefill":
+        print(json.dumps({"prefill": bench_prefill(sb, dev)}))
+        return
+    if args.only == "hybrid":
+        print(json.dumps({"hybrid_decode": bench_hybrid(sb, dev, steps=min(args.steps, 128))}))
+        return
 
     prob = build_config2(dev)
     kv, n_copies = prob["kv"], len(prob["kv"])

@@ -45,6 +45,7 @@ struct PrefillParams {
   const int32_t *tile_seq;    // [tiles] sequence of each 64-token query tile
   const int32_t *tile_q0;     // [tiles] first query (index inside its sequence) of the tile
   int G, head_begin;          // query heads per kv head; first of them handled by this launch
+  int num_tiles;
   int block_size, window_left;
   float scale_log2;
   int64_t q_sr, q_sh, o_sr, o_sh;  // elements
@@ -61,7 +62,12 @@ template <typename E, int NH>
 __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams p) {
   __shared__ __attribute__((aligned(16))) char smem[2 * 2 * kStage];  // [buffer][K|V]
 
-  const int tile = blockIdx.x;
+  // Workgroups are handed to the 8 XCDs round-robin by index, and each XCD has its own L2. Give XCD x
+  // the x-th contiguous eighth of the tiles, so that the workgroups resident on one XCD at a time are
+  // neighbouring tiles of one sequence and kv head, whose key windows overlap almost entirely.
+  const int per_xcd = (p.num_tiles + 7) >> 3;
+  const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (tile >= p.num_tiles) return;
   const int kvh = blockIdx.y;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -320,7 +326,7 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   if (!(a->scale > 0.f)) return fail(SB_ERR_INVALID, "sb_swa_prefill: scale must be positive");
   if (a->block_table && (a->block_size < 16 || a->block_size % 16 != 0))
     return fail(SB_ERR_INVALID, "sb_swa_prefill: block_size %d must be a multiple of 16", a->block_size);
-  if (a->num_tiles > 0x7fffffffLL || a->num_kv_heads > 65535)
+  if (a->num_tiles > 0x7ffffff0LL || a->num_kv_heads > 65535)
     return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: grid too large");
   const int64_t es[] = {a->q_stride_row, a->q_stride_head, a->out_stride_row, a->out_stride_head,
                         a->kv_stride_block, a->kv_stride_row, a->kv_stride_head};
@@ -341,8 +347,9 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   p.q_sr = a->q_stride_row; p.q_sh = a->q_stride_head; p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
   p.kv_sb = a->kv_stride_block * 2; p.kv_sr = a->kv_stride_row * 2; p.kv_sh = a->kv_stride_head * 2;
   p.bt_stride = a->block_table_stride;
+  p.num_tiles = (int)a->num_tiles;
 
-  const dim3 grid((unsigned)a->num_tiles, (unsigned)a->num_kv_heads);
+  const dim3 grid((unsigned)((a->num_tiles + 7) / 8 * 8), (unsigned)a->num_kv_heads);
   for (int h0 = 0; h0 < p.G; h0 += 4) {  // a GQA group is covered 4 heads at a time
     p.head_begin = h0;
     const int nh = p.G - h0 < 4 ? p.G - h0 : 4;
