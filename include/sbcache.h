@@ -273,6 +273,46 @@ typedef struct sb_swa_prefill_args {
 int sb_swa_prefill(const sb_swa_prefill_args *args);
 
 /* ------------------------------------------------------------------------------------
+ * Device-side decode-step advance for the sliding-window paged cache: every sequence of
+ * the batch takes one more token; seq_lens, slot_mapping and the window-ordered block
+ * tables of the step are produced on the GPU, and the window bookkeeping (evict the
+ * blocks that left the window, allocate the block a sequence grows into, LIFO free
+ * stack, sequences in batch-row order) is done there too.
+ * Window-aware analogue of ops.advance_step_flashattn as called from
+ *   vllm_hymeta/attention/meta_attention.py:338-409 (which bumps seq_lens and looks the
+ *   slot up in pre-grown block tables), so that consecutive decode steps - or a captured
+ *   graph of them - need no host-side metadata rebuild.
+ * State (device memory owned by the caller, updated in place):
+ *   n_tokens [B] int64   tokens each sequence has seen
+ *   lo, hi   [B] int32   lowest / highest resident logical block (hi < lo: none)
+ *   ring     [B, ring_blocks] int32   physical id of logical block j at ring[b][j % ring_blocks]
+ *   free_stack [num_blocks] int32, free_top [1] int32   free ids; the next allocation takes
+ *                                                     free_stack[free_top - 1]
+ * Outputs of the step:
+ *   slot_mapping [B] int64, seq_lens [B] int32 (keys visible through the table, the new
+ *   token included), block_tables [B, table_width] int32 (oldest resident block first,
+ *   0 beyond the last), status [1] int32 (sticky; bit 0 = out of blocks, bit 1 = a
+ *   sequence outgrew its ring; the caller reads it when it next synchronises).
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_window_advance_args {
+  int64_t *n_tokens;
+  int32_t *lo;
+  int32_t *hi;
+  int32_t *ring;
+  int32_t *free_stack;
+  int32_t *free_top;
+  int64_t *slot_mapping;
+  int32_t *seq_lens;
+  int32_t *block_tables;
+  int32_t *status;
+  int64_t batch;
+  int32_t ring_blocks, block_size, window_left, table_width, num_blocks;
+  void *stream;
+} sb_window_advance_args;
+
+int sb_window_advance(const sb_window_advance_args *args);
+
+/* ------------------------------------------------------------------------------------
  * Plain device-to-device streaming copy (non-temporal 16-byte lanes), `bytes` a multiple of
  * 16384. No counterpart in the reference: it is the measured bandwidth yardstick printed by
  * bench.py next to the kernels, and the launch of known size that the HBM byte counters

@@ -96,6 +96,16 @@ class SwaPrefillArgs(C.Structure):
     ]
 
 
+class WindowAdvanceArgs(C.Structure):
+    _fields_ = [
+        ("n_tokens", vp), ("lo", vp), ("hi", vp), ("ring", vp), ("free_stack", vp), ("free_top", vp),
+        ("slot_mapping", vp), ("seq_lens", vp), ("block_tables", vp), ("status", vp),
+        ("batch", i64),
+        ("ring_blocks", i32), ("block_size", i32), ("window_left", i32), ("table_width", i32), ("num_blocks", i32),
+        ("stream", vp),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/sbcache.h declares
 EXPORTS = {
     "sb_abi_version": (C.c_int, []),
@@ -108,6 +118,7 @@ EXPORTS = {
     "sb_copy_blocks": (C.c_int, [vp, vp, i64, i64, i64, vp]),
     "sb_window_shift": (C.c_int, [C.POINTER(WindowShiftArgs)]),
     "sb_swa_prefill": (C.c_int, [C.POINTER(SwaPrefillArgs)]),
+    "sb_window_advance": (C.c_int, [C.POINTER(WindowAdvanceArgs)]),
     "sb_stream_copy": (C.c_int, [vp, vp, i64, vp]),
 }
 

@@ -203,3 +203,76 @@ class WindowBlockManager:
         tables = np.where(j <= hi[:, None], self.ring[rows[:, None], j % R], 0).astype(np.int32)
         seqlens = np.where(nblk > 0, self.n_tokens[rows] - lo * bs, 0).astype(np.int32)
         return tables, seqlens, lo * bs
+
+
+class DeviceWindowState:
+    """The manager's state for a fixed decoding batch, resident on the GPU, advanced there one token
+    per sequence per call (`ops.window_advance`): the device-side counterpart of
+    `WindowBlockManager.decode_step` + `kernel_view`, with the same policy and therefore the same
+    slots, tables and free-stack order, bit for bit. The role ops.advance_step_flashattn plays for the
+    reference's multi-step decode (vllm_hymeta/attention/meta_attention.py:338-409), extended by the
+    window bookkeeping, so that a run of decode steps (or a captured graph of them) does no host work.
+
+    Built from a host manager (`upload`); `download` writes the advanced state back into it, e.g.
+    before sequences join or leave the batch (membership changes stay host-side)."""
+
+    def __init__(self, manager: WindowBlockManager, seq_ids: Sequence, device, table_width: Optional[int] = None):
+        import torch
+
+        from . import ops
+        self._torch, self._ops = torch, ops
+        self.manager, self.seq_ids = manager, list(seq_ids)
+        self.device = torch.device(device)
+        self.rows = np.fromiter((manager.row_of(s) for s in self.seq_ids), dtype=np.int64, count=len(self.seq_ids))
+        B = len(self.seq_ids)
+        self.table_width = manager.ring_blocks if table_width is None else int(table_width)
+        if self.table_width < manager.window_left // manager.block_size + 2:
+            raise ValueError("table_width cannot hold a full window")
+        i32, i64 = torch.int32, torch.int64
+        self.n_tokens = torch.empty(B, dtype=i64, device=self.device)
+        self.lo = torch.empty(B, dtype=i32, device=self.device)
+        self.hi = torch.empty(B, dtype=i32, device=self.device)
+        self.ring = torch.empty(B, manager.ring_blocks, dtype=i32, device=self.device)
+        self.free_stack = torch.empty(manager.num_blocks, dtype=i32, device=self.device)
+        self.free_top = torch.empty(1, dtype=i32, device=self.device)
+        self.slot_mapping = torch.full((B,), PAD_SLOT_ID, dtype=i64, device=self.device)
+        self.seq_lens = torch.zeros(B, dtype=i32, device=self.device)
+        self.block_tables = torch.zeros(B, self.table_width, dtype=i32, device=self.device)
+        self.status = torch.zeros(1, dtype=i32, device=self.device)
+        self.upload()
+
+    def upload(self) -> None:
+        """Host manager -> device (synchronous copies)."""
+        t, m, r = self._torch, self.manager, self.rows
+        self.n_tokens.copy_(t.from_numpy(m.n_tokens[r].astype(np.int64)))
+        self.lo.copy_(t.from_numpy(m.lo[r].astype(np.int32)))
+        self.hi.copy_(t.from_numpy(m.hi[r].astype(np.int32)))
+        self.ring.copy_(t.from_numpy(np.ascontiguousarray(m.ring[r])))
+        self.free_stack.copy_(t.from_numpy(m._stack))
+        self.free_top.fill_(int(m._top))
+
+    def advance(self) -> None:
+        """Enqueue one decode step for every sequence on the current stream (no synchronisation)."""
+        m = self.manager
+        self._ops.window_advance(self.n_tokens, self.lo, self.hi, self.ring, self.free_stack, self.free_top,
+                                 self.slot_mapping, self.seq_lens, self.block_tables, self.status,
+                                 block_size=m.block_size, window_left=m.window_left)
+
+    def check(self) -> None:
+        """Synchronise and raise if any advance since the last check ran out of blocks or ring."""
+        s = int(self.status.item())
+        if s & 1:
+            raise RuntimeError("out of KV cache blocks")
+        if s & 2:
+            raise RuntimeError("a sequence outgrew its block ring")
+
+    def download(self) -> None:
+        """Device -> host manager (synchronises)."""
+        self.check()
+        m, r = self.manager, self.rows
+        m.n_tokens[r] = self.n_tokens.cpu().numpy()
+        m.lo[r] = self.lo.cpu().numpy()
+        m.hi[r] = self.hi.cpu().numpy()
+        m.ring[r] = self.ring.cpu().numpy()
+        m._stack[:] = self.free_stack.cpu().numpy()
+        m._top = int(self.free_top.item())

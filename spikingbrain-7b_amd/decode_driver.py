@@ -22,7 +22,7 @@ import numpy as np
 import torch
 
 from . import ops
-from .block_manager import WindowBlockManager
+from .block_manager import DeviceWindowState, WindowBlockManager
 from .meta_attention import MetaAttentionBackend, MetaAttentionImpl, MetaAttentionMetadata
 
 
@@ -81,6 +81,42 @@ class HybridDecodeCache:
             max_prefill_seq_len=0, max_decode_seq_len=int(seqlens.max()), context_lens_tensor=None,
             block_tables=torch.from_numpy(tables).to(dev, non_blocking=True), use_cuda_graph=False,
             max_query_len=1, max_decode_query_len=1)
+
+    # -- device-side stepping: no host work between decode steps --------------------------------
+    def enable_device_advance(self) -> MetaAttentionMetadata:
+        """Move the block manager's state for this batch to the GPU. Returns the metadata object of
+        every following step: its slot_mapping / seq_lens / block_tables are the tensors the advance
+        kernels rewrite in place (`advance_device`), so one object (and one captured graph) serves
+        all steps."""
+        self.device_state = DeviceWindowState(self.manager, self.seq_ids, self.device)
+        st = self.device_state
+        B = self.batch
+        self.device_meta = MetaAttentionMetadata(
+            num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B,
+            slot_mapping=st.slot_mapping, seq_lens=None, seq_lens_tensor=st.seq_lens,
+            max_prefill_seq_len=0, max_decode_seq_len=st.table_width * self.bs, context_lens_tensor=None,
+            block_tables=st.block_tables, use_cuda_graph=True, max_query_len=1, max_decode_query_len=1)
+        return self.device_meta
+
+    def advance_device(self) -> None:
+        """Enqueue the step advance (eviction, allocation, slots, lengths, tables) on the GPU."""
+        self.device_state.advance()
+
+    def capture_step(self, run_layers) -> "torch.cuda.CUDAGraph":
+        """Capture `advance_device()` followed by `run_layers(meta)` (the caller's 28 layer calls on
+        static input tensors) into one graph; every replay is one whole decode step."""
+        meta = self.device_meta
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):      # warm up outside the capture: lazy allocations happen here
+            self.advance_device()
+            run_layers(meta)
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.advance_device()
+            run_layers(meta)
+        return graph
 
     def gla_layer(self, layer_idx: int, q, k, v, g, out=None) -> torch.Tensor:
         """q, k, v, g [B, H, 1, D]; the layer's state is advanced in place. Returns o [B, H, 1, D]."""

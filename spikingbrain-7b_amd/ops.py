@@ -436,3 +436,33 @@ def window_shift(src: Optional[torch.Tensor], dst: torch.Tensor, fresh: Optional
         fresh_stride_row_bytes=0 if fresh is None else fresh.stride(2) * esz,
         stream=N.stream_ptr(dev))
     N.check(N.lib().sb_window_shift(C.byref(a)), "window_shift")
+
+
+def window_advance(n_tokens: torch.Tensor, lo: torch.Tensor, hi: torch.Tensor, ring: torch.Tensor,
+                   free_stack: torch.Tensor, free_top: torch.Tensor, slot_mapping: torch.Tensor,
+                   seq_lens: torch.Tensor, block_tables: torch.Tensor, status: torch.Tensor, *,
+                   block_size: int, window_left: int) -> None:
+    """One decode token for every sequence, on the device: evict / allocate / slot / visible length /
+    block-table rows, with the host block manager's policy (see block_manager.DeviceWindowState).
+    All tensors are updated in place; nothing is allocated and nothing is read back."""
+    dev = N.require_gpu(n_tokens, lo, hi, ring, free_stack, free_top, slot_mapping, seq_lens, block_tables, status)
+    B = n_tokens.numel()
+    want = ((n_tokens, torch.int64, (B,)), (lo, torch.int32, (B,)), (hi, torch.int32, (B,)),
+            (free_top, torch.int32, (1,)), (slot_mapping, torch.int64, (B,)), (seq_lens, torch.int32, (B,)),
+            (status, torch.int32, (1,)))
+    for t, dt, shape in want:
+        if t.dtype != dt or tuple(t.shape) != shape or not t.is_contiguous():
+            raise ValueError(f"window_advance: expected a contiguous {dt} tensor of shape {shape}, got "
+                             f"{t.dtype} {tuple(t.shape)}")
+    for t, name in ((ring, "ring"), (block_tables, "block_tables")):
+        if t.dtype != torch.int32 or t.dim() != 2 or t.shape[0] != B or not t.is_contiguous():
+            raise ValueError(f"window_advance: {name} must be a contiguous int32 [batch, n] tensor")
+    if free_stack.dtype != torch.int32 or free_stack.dim() != 1 or not free_stack.is_contiguous():
+        raise ValueError("window_advance: free_stack must be a contiguous int32 vector")
+    a = N.WindowAdvanceArgs(
+        n_tokens=N.ptr(n_tokens), lo=N.ptr(lo), hi=N.ptr(hi), ring=N.ptr(ring), free_stack=N.ptr(free_stack),
+        free_top=N.ptr(free_top), slot_mapping=N.ptr(slot_mapping), seq_lens=N.ptr(seq_lens),
+        block_tables=N.ptr(block_tables), status=N.ptr(status), batch=B, ring_blocks=ring.shape[1],
+        block_size=int(block_size), window_left=int(window_left), table_width=block_tables.shape[1],
+        num_blocks=free_stack.numel(), stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_window_advance(C.byref(a)), "window_advance")

@@ -64,3 +64,86 @@ def test_hybrid_decode_steps_vs_oracle(sb, dev, ctx):
                 assert np.array_equal(drv.kv_caches[j][0].float().cpu().numpy(), kc[j])
                 assert np.array_equal(drv.kv_caches[j][1].float().cpu().numpy(), vc[j])
     assert drv.manager.free_stack() == model.free
+
+
+def test_captured_graph_replays_whole_steps(sb, dev):
+    """Device-side step advance + all layers captured once in a HIP graph; every replay is one decode
+    step on fresh inputs (copied into the static input tensors, with eager work and synchronisation
+    between replays) and is checked against the oracle: slots, tables, cache bytes, outputs."""
+    B, L, H, HKV, D, bs, wl, ctx = 4, 4, 8, 2, 128, 16, 48, 777
+    drv = sb.HybridDecodeCache(B, num_layers=L, num_heads=H, num_kv_heads=HKV, head_size=D, block_size=bs,
+                               window_left=wl, device=dev, randomize=True, seed=5)
+    drv.start(ctx)
+    model = P.WindowCacheModel(drv.num_blocks, bs, wl)
+    for s in range(B):
+        model.add_seq(s)
+        model.append_tokens(s, ctx, True)
+    drv.enable_device_advance()
+    # static inputs and outputs of the captured step
+    gl = [tuple(torch.zeros(B, H, 1, D, dtype=torch.bfloat16, device=dev) for _ in range(3))
+          + (torch.zeros(B, H, 1, D, dtype=torch.float32, device=dev),) for _ in range(L // 2)]
+    sw = [(torch.zeros(B, H, D, dtype=torch.bfloat16, device=dev), torch.zeros(B, HKV, D, dtype=torch.bfloat16, device=dev),
+           torch.zeros(B, HKV, D, dtype=torch.bfloat16, device=dev)) for _ in range(L // 2)]
+    g_out = [torch.zeros(B, H, 1, D, dtype=torch.bfloat16, device=dev) for _ in range(L // 2)]
+    s_out = [torch.zeros(B, H, D, dtype=torch.bfloat16, device=dev) for _ in range(L // 2)]
+
+    def run_layers(meta):
+        for li in range(L):
+            if li % 2 == 0:
+                drv.gla_layer(li, *gl[li // 2], out=g_out[li // 2])
+            else:
+                drv.swa_layer(li, *sw[li // 2], meta, s_out[li // 2])
+
+    g = torch.Generator().manual_seed(9)
+
+    def fresh_inputs():
+        host = []
+        for j in range(L // 2):
+            q, k, v = (torch.randn(B, H, 1, D, generator=g).bfloat16() for _ in range(3))
+            gate = torch.nn.functional.logsigmoid(torch.randn(B, H, 1, D, generator=g)) / 16
+            for dst, src in zip(gl[j], (q, k, v, gate)):
+                dst.copy_(src)
+            qs = torch.randn(B, H, D, generator=g).bfloat16()
+            ks = torch.randn(B, HKV, D, generator=g).bfloat16()
+            vs = torch.randn(B, HKV, D, generator=g).bfloat16()
+            for dst, src in zip(sw[j], (qs, ks, vs)):
+                dst.copy_(src)
+            host.append((q, k, v, gate, qs, ks, vs))
+        return host
+
+    # the capture's warm-up pass and the capture itself do not execute as checked steps: the warm-up
+    # is a real step (oracle follows it), the capture only records
+    warm = fresh_inputs()
+    graph = drv.capture_step(run_layers)
+    torch.cuda.synchronize()
+    kc = [c[0].float().cpu().numpy() for c in drv.kv_caches]
+    vc = [c[1].float().cpu().numpy() for c in drv.kv_caches]
+    state = drv.gla_state.cpu().numpy().astype(np.float64)
+    for s in range(B):
+        model.append_tokens(s, 1, False)        # the warm-up step (its cache writes are in kc/vc already)
+    del warm
+    for step in range(2 * bs + 2):
+        host = fresh_inputs()
+        graph.replay()
+        torch.cuda.synchronize()
+        slots = [model.append_tokens(s, 1, False)[0] for s in range(B)]
+        assert drv.device_state.slot_mapping.cpu().tolist() == slots, f"replay {step}"
+        views = [model.view(s) for s in range(B)]
+        lens = [v[1] for v in views]
+        assert drv.device_state.seq_lens.cpu().tolist() == lens
+        tables = np.zeros((B, drv.device_state.table_width), np.int32)
+        for s, v in enumerate(views):
+            tables[s, :len(v[0])] = v[0]
+        assert np.array_equal(drv.device_state.block_tables.cpu().numpy(), tables)
+        for j in range(L // 2):
+            q, k, v, gate, qs, ks, vs = host[j]
+            ref = G.gla_step(q.float().numpy()[:, :, 0], k.float().numpy()[:, :, 0], v.float().numpy()[:, :, 0],
+                             gate.numpy()[:, :, 0], state[j])
+            o = g_out[j].float().cpu().numpy()[:, :, 0]
+            assert (np.abs(o - ref) <= 2e-2 + np.abs(ref) * 2.0 ** -8).all()
+            P.kv_append(ks.float().numpy(), vs.float().numpy(), kc[j], vc[j], slots)
+            ref = A.paged_decode_attention(qs.float().numpy(), kc[j], vc[j], tables, lens, D ** -0.5, wl)
+            assert np.abs(s_out[j].float().cpu().numpy() - ref).max() <= 2e-2, f"replay {step} layer {2 * j + 1}"
+            assert np.array_equal(drv.kv_caches[j][0].float().cpu().numpy(), kc[j])
+    drv.device_state.download()
+    assert drv.manager.free_stack() == model.free
