@@ -6,25 +6,28 @@
 // the end of the key sequence).
 //
 // Work decomposition
-//   grid = (query tiles of 64 tokens, kv heads); 4 wavefronts per workgroup, wavefront w owns tokens
-//   16w..16w+15 of the tile for NH <= 4 query heads of the kv head (16*NH score rows, no padding); a
-//   GQA group wider than 4 heads is covered by several launches (7 = 4 + 3).
+//   grid = (query tiles of 64 tokens, kv heads); a workgroup covers up to 4 query heads of the kv head
+//   (a wider GQA group takes several launches, 7 = 4 + 3). Every wavefront owns two "column blocks" of
+//   16 tokens x 1 head (32 score columns, no padding): a pair of heads is served by 4 wavefronts (one
+//   per 16-token sub-tile), an odd last head by 2 wavefronts (two sub-tiles each) - 8 wavefronts for 4
+//   heads, 6 for 3. At 256 registers per wavefront two of them share a SIMD, so one wavefront's
+//   softmax arithmetic overlaps the other's matrix instructions and LDS waits.
 //   The workgroup walks the union of its tokens' windows in chunks of 32 keys. Each chunk of K and V
-//   (32 rows x 256 B each) is fetched from global memory ONCE per workgroup (wavefront w fetches rows
-//   8w..8w+7 with whole-row 16-byte lanes) into a double-buffered LDS stage whose rows are padded to
-//   272 B, which makes both operand read patterns bank-conflict free; all four wavefronts then read
-//   their MFMA operands from LDS. Global loads of chunk n+1 are in flight while chunk n is computed.
-//   Per chunk and head: S^T = K Q^T (8 MFMA 16x16x32, tokens on the N axis), softmax numerators per
-//   lane for token lane%16 in log2 units, O^T += V^T P^T (8 MFMA). P stays in the lane that produced
-//   it; V^T operands come from an in-register 8x8 transpose shared by the heads.
+//   (32 rows x 256 B each) is fetched from global memory ONCE per workgroup (the first four wavefronts
+//   fetch 8 rows each with whole-row 16-byte lanes) into a double-buffered LDS stage whose rows are
+//   padded to 272 B; all wavefronts then read their MFMA operands from LDS. Global loads of chunk n+1
+//   are in flight while chunk n is computed.
+//   Per chunk and column block: S^T = K Q^T (8 MFMA 16x16x32, tokens on the N axis), softmax numerators
+//   per lane for token lane%16 in log2 units, O^T += V^T P^T (8 MFMA). P stays in the lane that produced
+//   it; V^T operands come from an in-register 8x8 transpose shared by the two blocks.
+//   Workgroups are numbered so that each XCD (own L2) works through one contiguous run of tiles.
 //
 // Softmax reference point
 //   The numerators are exp2(s - m_ref) with a per-row reference m_ref that is only raised when some
 //   row of the wavefront scores more than kRaise (log2 units) above it, so they stay below 2^kRaise
 //   (exact in fp32 sums, inside fp16 range). Raising m_ref rescales the output accumulators; that code
-//   sits OUTSIDE the chunk loop (the loop is left and re-entered), because the accumulators live in the
-//   accumulation registers and any branch inside the loop that touches them makes the compiler carry
-//   all of them in vector registers and copy them to and fro on every chunk.
+//   sits OUTSIDE the chunk loop (the loop is left and re-entered), which keeps the loop body free of
+//   branches around the accumulators.
 #include "common.h"
 #include "mfma_util.h"
 
@@ -58,8 +61,22 @@ constexpr int kStage = 32 * kRowPad;  // one K or V chunk
 constexpr float kNegInf = kNegInfF;
 constexpr float kRaise = 8.f;
 
-template <typename E, int NH>
-__global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams p) {
+// NHEADS query heads of one kv head per workgroup; wavefronts own two column blocks each
+// (a column block = 16 tokens x 1 head): head pairs are served by 4 wavefronts (one per 16-token
+// sub-tile, both heads of the pair), an odd last head by 2 wavefronts (two sub-tiles each).
+template <int NHEADS>
+struct Shape {
+  static constexpr int kPairs = NHEADS / 2;
+  static constexpr int kWaves = 4 * kPairs + 2 * (NHEADS % 2);
+  static constexpr int kFetchWaves = kWaves < 4 ? kWaves : 4;   // wavefronts that move K/V into LDS
+  static constexpr int kLoads = 8 / kFetchWaves;                // 4-row loads per fetching lane, per K and per V
+};
+
+template <typename E, int NHEADS>
+__global__ __attribute__((amdgpu_flat_work_group_size(64 * Shape<NHEADS>::kWaves, 64 * Shape<NHEADS>::kWaves),
+                          amdgpu_waves_per_eu(2, 2)))
+void swa_prefill_kernel(const PrefillParams p) {
+  using S = Shape<NHEADS>;
   __shared__ __attribute__((aligned(16))) char smem[2 * 2 * kStage];  // [buffer][K|V]
 
   // Workgroups are handed to the 8 XCDs round-robin by index, and each XCD has its own L2. Give XCD x
@@ -92,31 +109,42 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
   const int first_tile = wg_lo >> 4, last_tile = (wg_hi - 1) >> 4;
   const int ch_begin = wg_lo >> 5, ch_end = ((wg_hi - 1) >> 5) + 1;
 
-  // this wavefront's 16 tokens (rows past the end of the sequence repeat its last token; never stored)
-  const int jw0 = min(q0 + 16 * wave, Lq - 1);
-  const int jw_last = min(q0 + 16 * wave + 15, Lq - 1);
-  const int j_mine = min(q0 + 16 * wave + c, Lq - 1);
-  const int my_pos = shift + j_mine;
-  const int my_lo = max(wl >= 0 ? my_pos - wl : 0, klo);
+  // this wavefront's two column blocks: 16-token sub-tile ts[b] of head hd[b]
+  int ts[2], hd[2];
+  if (wave < 4 * S::kPairs) {
+    ts[0] = ts[1] = wave & 3;
+    hd[0] = 2 * (wave >> 2);
+    hd[1] = hd[0] + 1;
+  } else {
+    ts[0] = 2 * (wave - 4 * S::kPairs);
+    ts[1] = ts[0] + 1;
+    hd[0] = hd[1] = NHEADS - 1;
+  }
   const int head0 = kvh * p.G + p.head_begin;
-
-  // Q^T operands: token lane%16, head h, dims of 16-byte piece 4s+g
-  uint4 qb[NH][4];
+  // (rows past the end of the sequence repeat its last token; they are never stored)
+  const int jw0 = min(q0 + 16 * ts[0], Lq - 1);            // first and last token of the wavefront
+  const int jw_last = min(q0 + 16 * ts[1] + 15, Lq - 1);
+  int my_pos[2], my_lo[2];
+  uint4 qb[2][4];  // Q^T operands: token lane%16 of the block, dims of 16-byte piece 4s+g
 #pragma unroll
-  for (int h = 0; h < NH; ++h)
+  for (int b = 0; b < 2; ++b) {
+    const int j_mine = min(q0 + 16 * ts[b] + c, Lq - 1);
+    my_pos[b] = shift + j_mine;
+    my_lo[b] = max(wl >= 0 ? my_pos[b] - wl : 0, klo);
 #pragma unroll
     for (int s = 0; s < 4; ++s)
-      qb[h][s] = *reinterpret_cast<const uint4 *>(
-          p.q + ((int64_t)(qrow0 + j_mine) * p.q_sr + (int64_t)(head0 + h) * p.q_sh + (4 * s + g) * 8) * 2);
+      qb[b][s] = *reinterpret_cast<const uint4 *>(
+          p.q + ((int64_t)(qrow0 + j_mine) * p.q_sr + (int64_t)(head0 + hd[b]) * p.q_sh + (4 * s + g) * 8) * 2);
+  }
 
-  f32x4_t acc[NH][8];
-  float m[NH], l[NH];  // m: reference point of the numerators (log2 units), l: this lane's share of the sum
+  f32x4_t acc[2][8];
+  float m[2], l[2];  // m: reference point of the numerators (log2 units), l: this lane's share of the sum
 #pragma unroll
-  for (int h = 0; h < NH; ++h) {
-    m[h] = kNegInf;
-    l[h] = 0.f;
+  for (int b = 0; b < 2; ++b) {
+    m[b] = kNegInf;
+    l[b] = 0.f;
 #pragma unroll
-    for (int mt = 0; mt < 8; ++mt) acc[h][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < 8; ++mt) acc[b][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
   const bool paged = p.block_table != nullptr;
@@ -132,36 +160,38 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
     return (dense_row0 + i0) * p.kv_sr + head_off;
   };
 
-  // ---- global -> registers: wavefront w fetches rows 8w..8w+7 of the chunk (K and V) ----------
+  // ---- global -> registers -> LDS: the first kFetchWaves wavefronts move the chunk (32 K rows and
+  // 32 V rows of 256 B); each of their loads covers 4 rows, all inside one 16-key tile of the table.
   // rows outside [wg_lo, wg_hi) are clamped onto the nearest visible key (masked for every token)
-  const int lrow = (wave & 1) * 8 + (lane >> 4);  // row inside the 16-key tile, +4 for the second load
-  uint4 stage_k[2], stage_v[2];
+  const bool fetcher = wave < S::kFetchWaves;
+  const int rows_per_wave = 32 / S::kFetchWaves;                         // 8 or 16
+  const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the 16-key tile, +4 per load
+  uint4 stage_k[S::kLoads], stage_v[S::kLoads];
   auto fetch = [&](int ch) {
-    const int t = min(max(2 * ch + (wave >> 1), first_tile), last_tile);
+    const int t = min(max(2 * ch + (wave * rows_per_wave) / 16, first_tile), last_tile);
     const int64_t base = tile_base(t);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < S::kLoads; ++u) {
       const int row = min(max((t << 4) + lrow + 4 * u, wg_lo), wg_hi - 1) - (t << 4);
       const int64_t off = base + (int64_t)row * p.kv_sr + c * 16;
       stage_k[u] = load_stream16(p.k + off);
       stage_v[u] = load_stream16(p.v + off);
     }
   };
-  // registers -> LDS stage `buf`
   auto stash = [&](int buf) {
     char *sk = smem + buf * 2 * kStage, *sv = sk + kStage;
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int kk = wave * 8 + (lane >> 4) + 4 * u;
+    for (int u = 0; u < S::kLoads; ++u) {
+      const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
       *reinterpret_cast<uint4 *>(sk + kk * kRowPad + c * 16) = stage_k[u];
       *reinterpret_cast<uint4 *>(sv + kk * kRowPad + c * 16) = stage_v[u];
     }
   };
 
-  float sc[NH][8];  // scores of the chunk in flight (raw dot products; -inf where masked)
-  float mx[NH];     // their row maxima, in log2 units
+  float sc[2][8];  // scores of the chunk in flight (raw dot products; -inf where masked)
+  float mx[2];     // their row maxima, in log2 units
 
-  // scores of chunk `ch` for every head; true when some row needs a higher reference point
+  // scores of chunk `ch` for both column blocks; true when some row needs a higher reference point
   auto scores = [&](int ch, int buf) -> bool {
     const char *sk = smem + buf * 2 * kStage;
     uint4 k0[4], k1[4];
@@ -171,35 +201,35 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
       k1[s] = *reinterpret_cast<const uint4 *>(sk + (16 + c) * kRowPad + (4 * s + g) * 16);
     }
     const int c0 = ch << 5;
-    // wholly visible to all 16 tokens: above every token's lower bound, at or below the first token
+    // wholly visible to all tokens of the wavefront: above every lower bound, at or below the first token
     const bool full = (wl < 0 || c0 >= shift + jw_last - wl) && c0 >= klo && (c0 + 31 <= shift + jw0);
     bool raise = false;
 #pragma unroll
-    for (int h = 0; h < NH; ++h) {
+    for (int b = 0; b < 2; ++b) {
       f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        s0 = Mma<E>::run(k0[s], qb[h][s], s0);
-        s1 = Mma<E>::run(k1[s], qb[h][s], s1);
+        s0 = Mma<E>::run(k0[s], qb[b][s], s0);
+        s1 = Mma<E>::run(k1[s], qb[b][s], s1);
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        sc[h][j] = s0[j];
-        sc[h][4 + j] = s1[j];
+        sc[b][j] = s0[j];
+        sc[b][4 + j] = s1[j];
       }
       if (!full) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int i = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-          if (i > my_pos || i < my_lo) sc[h][j] = kNegInf;
+          if (i > my_pos[b] || i < my_lo[b]) sc[b][j] = kNegInf;
         }
       }
-      float t = fmaxf(fmaxf(fmaxf(sc[h][0], sc[h][1]), fmaxf(sc[h][2], sc[h][3])),
-                      fmaxf(fmaxf(sc[h][4], sc[h][5]), fmaxf(sc[h][6], sc[h][7])));
+      float t = fmaxf(fmaxf(fmaxf(sc[b][0], sc[b][1]), fmaxf(sc[b][2], sc[b][3])),
+                      fmaxf(fmaxf(sc[b][4], sc[b][5]), fmaxf(sc[b][6], sc[b][7])));
       t = fmaxf(t, __shfl_xor(t, 16));
       t = fmaxf(t, __shfl_xor(t, 32));
-      mx[h] = t * p.scale_log2;
-      raise |= mx[h] > m[h] + kRaise;  // also true for the first finite score of a row (m = -inf)
+      mx[b] = t * p.scale_log2;
+      raise |= mx[b] > m[b] + kRaise;  // also true for the first finite score of a row (m = -inf)
     }
     return __builtin_amdgcn_ballot_w64(raise) != 0;
   };
@@ -207,19 +237,19 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
   // numerators against the current reference points, then O^T += V^T P^T
   auto accumulate = [&](int buf) {
     const char *sv = smem + buf * 2 * kStage + kStage;
-    uint4 pb[NH];
+    uint4 pb[2];
 #pragma unroll
-    for (int h = 0; h < NH; ++h) {
-      const float m_safe = (m[h] == kNegInf) ? 0.f : m[h];
+    for (int b = 0; b < 2; ++b) {
+      const float m_safe = (m[b] == kNegInf) ? 0.f : m[b];
       float psum = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        sc[h][j] = fast_exp2(fmaf(sc[h][j], p.scale_log2, -m_safe));
-        psum += sc[h][j];
+        sc[b][j] = fast_exp2(fmaf(sc[b][j], p.scale_log2, -m_safe));
+        psum += sc[b][j];
       }
-      l[h] += psum;
-      pb[h] = make_uint4(Mma<E>::pack(sc[h][0], sc[h][1]), Mma<E>::pack(sc[h][2], sc[h][3]),
-                         Mma<E>::pack(sc[h][4], sc[h][5]), Mma<E>::pack(sc[h][6], sc[h][7]));
+      l[b] += psum;
+      pb[b] = make_uint4(Mma<E>::pack(sc[b][0], sc[b][1]), Mma<E>::pack(sc[b][2], sc[b][3]),
+                         Mma<E>::pack(sc[b][4], sc[b][5]), Mma<E>::pack(sc[b][6], sc[b][7]));
     }
     uint4 v[8];
 #pragma unroll
@@ -229,23 +259,25 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
     }
 #pragma unroll
     for (int mt = 0; mt < 8; ++mt) {
-      const uint4 vt = v_transposed(v, mt);  // built once, used by every head
+      const uint4 vt = v_transposed(v, mt);  // built once, used by both blocks
 #pragma unroll
-      for (int h = 0; h < NH; ++h) acc[h][mt] = Mma<E>::run(vt, pb[h], acc[h][mt]);
+      for (int b = 0; b < 2; ++b) acc[b][mt] = Mma<E>::run(vt, pb[b], acc[b][mt]);
     }
   };
 
   // ---- chunk loop: one barrier per chunk, every wavefront visits every chunk -------------------
   // (chunks outside a wavefront's own band come out fully masked and add zero)
-  fetch(ch_begin);
-  stash(0);
+  if (fetcher) {
+    fetch(ch_begin);
+    stash(0);
+  }
   __syncthreads();
   int ch = ch_begin;
   for (;;) {
     bool raise = false;
     for (; ch < ch_end; ++ch) {
       const int buf = (ch - ch_begin) & 1;
-      const bool more = ch + 1 < ch_end;
+      const bool more = fetcher && ch + 1 < ch_end;
       if (more) fetch(ch + 1);  // global loads fly while this chunk is computed
       raise = scores(ch, buf);
       if (raise) break;
@@ -256,18 +288,18 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
     if (!raise) break;
     // rare: lift the reference points to the running maxima and rescale, then finish this chunk
 #pragma unroll
-    for (int h = 0; h < NH; ++h) {
-      const float m_new = fmaxf(m[h], mx[h]);
+    for (int b = 0; b < 2; ++b) {
+      const float m_new = fmaxf(m[b], mx[b]);
       const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
-      const float alpha = fast_exp2(m[h] - m_safe);
-      m[h] = m_new;
-      l[h] *= alpha;
+      const float alpha = fast_exp2(m[b] - m_safe);
+      m[b] = m_new;
+      l[b] *= alpha;
 #pragma unroll
-      for (int mt = 0; mt < 8; ++mt) acc[h][mt] *= alpha;
+      for (int mt = 0; mt < 8; ++mt) acc[b][mt] *= alpha;
     }
     {
       const int buf = (ch - ch_begin) & 1;
-      const bool more = ch + 1 < ch_end;
+      const bool more = fetcher && ch + 1 < ch_end;
       accumulate(buf);
       if (more) stash(buf ^ 1);
       __syncthreads();
@@ -275,23 +307,23 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
     }
   }
 
-  // ---- epilogue: lane (g, c) owns token c, dims 32g + 8i + mt of each head ---------------------
-  if (q0 + 16 * wave + c < Lq) {
-    const int64_t orow = (int64_t)(qrow0 + q0 + 16 * wave + c) * p.o_sr;
+  // ---- epilogue: lane (g, c) owns token c of each block, dims 32g + 8i + mt ---------------------
 #pragma unroll
-    for (int h = 0; h < NH; ++h) {
-      float lt = l[h];
-      lt += __shfl_xor(lt, 16);
-      lt += __shfl_xor(lt, 32);
+  for (int b = 0; b < 2; ++b) {
+    float lt = l[b];
+    lt += __shfl_xor(lt, 16);
+    lt += __shfl_xor(lt, 32);
+    if (q0 + 16 * ts[b] + c < Lq) {
       const float inv = lt > 0.f ? 1.f / lt : 0.f;
-      char *dst = p.out + (orow + (int64_t)(head0 + h) * p.o_sh + 32 * g) * 2;
+      char *dst = p.out + ((int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.o_sr + (int64_t)(head0 + hd[b]) * p.o_sh +
+                           32 * g) * 2;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         uint4 o;
-        o.x = E::pack(acc[h][0][i] * inv, acc[h][1][i] * inv);
-        o.y = E::pack(acc[h][2][i] * inv, acc[h][3][i] * inv);
-        o.z = E::pack(acc[h][4][i] * inv, acc[h][5][i] * inv);
-        o.w = E::pack(acc[h][6][i] * inv, acc[h][7][i] * inv);
+        o.x = E::pack(acc[b][0][i] * inv, acc[b][1][i] * inv);
+        o.y = E::pack(acc[b][2][i] * inv, acc[b][3][i] * inv);
+        o.z = E::pack(acc[b][4][i] * inv, acc[b][5][i] * inv);
+        o.w = E::pack(acc[b][6][i] * inv, acc[b][7][i] * inv);
         *reinterpret_cast<uint4 *>(dst + 16 * i) = o;
       }
     }
@@ -301,10 +333,10 @@ __global__ __launch_bounds__(256, 1) void swa_prefill_kernel(const PrefillParams
 template <typename E>
 void launch_prefill(int nh, dim3 grid, hipStream_t st, const PrefillParams &p) {
   switch (nh) {
-    case 1: hipLaunchKernelGGL((swa_prefill_kernel<E, 1>), grid, dim3(256), 0, st, p); break;
-    case 2: hipLaunchKernelGGL((swa_prefill_kernel<E, 2>), grid, dim3(256), 0, st, p); break;
-    case 3: hipLaunchKernelGGL((swa_prefill_kernel<E, 3>), grid, dim3(256), 0, st, p); break;
-    default: hipLaunchKernelGGL((swa_prefill_kernel<E, 4>), grid, dim3(256), 0, st, p); break;
+    case 1: hipLaunchKernelGGL((swa_prefill_kernel<E, 1>), grid, dim3(64 * Shape<1>::kWaves), 0, st, p); break;
+    case 2: hipLaunchKernelGGL((swa_prefill_kernel<E, 2>), grid, dim3(64 * Shape<2>::kWaves), 0, st, p); break;
+    case 3: hipLaunchKernelGGL((swa_prefill_kernel<E, 3>), grid, dim3(64 * Shape<3>::kWaves), 0, st, p); break;
+    default: hipLaunchKernelGGL((swa_prefill_kernel<E, 4>), grid, dim3(64 * Shape<4>::kWaves), 0, st, p); break;
   }
 }
 
