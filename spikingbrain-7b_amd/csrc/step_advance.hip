@@ -37,6 +37,7 @@ constexpr int kTopCache = 4096;     // stack entries simulated in LDS
 __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParams p) {
   __shared__ int s_evict_n[kRowsPerPass];    // blocks the row evicts
   __shared__ int s_evict_lo[kRowsPerPass];   // first logical block it evicts
+  __shared__ int s_evict_id[kRowsPerPass];   // physical id of the first of them (fetched in parallel)
   __shared__ int s_alloc[kRowsPerPass];      // logical block it allocates, -1 = none
   __shared__ int s_newid[kRowsPerPass];      // physical id that block got
   __shared__ int s_cache[kTopCache];         // stack entries [cache_base, cache_base + cache_n)
@@ -66,6 +67,7 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
       const int ev_end = min(lo_new, hi + 1);
       s_evict_lo[tid] = lo;
       s_evict_n[tid] = max(0, ev_end - lo);
+      if (ev_end > lo) s_evict_id[tid] = p.ring[(int64_t)r * R + lo % R];
       if (hi >= lo) {
         lo = max(lo, lo_new);
         if (lo > hi) { lo = 0; hi = -1; }
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
       for (int i = 0; i < rows; ++i) {
         const int en = s_evict_n[i];
         for (int k = 0; k < en; ++k) {
-          const int id = p.ring[(int64_t)(r0 + i) * R + (s_evict_lo[i] + k) % R];
+          const int id = k == 0 ? s_evict_id[i] : p.ring[(int64_t)(r0 + i) * R + (s_evict_lo[i] + k) % R];
           if (n == kTopCache) {  // cache full: spill it to the global stack and start afresh
             for (int u = 0; u < n; ++u) p.free_stack[base + u] = s_cache[u];
             base += n;
