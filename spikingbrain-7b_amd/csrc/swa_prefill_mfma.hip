@@ -224,10 +224,9 @@ void swa_prefill_kernel(const PrefillParams p) {
           if (i > my_pos[b] || i < my_lo[b]) sc[b][j] = kNegInf;
         }
       }
-      float t = fmaxf(fmaxf(fmaxf(sc[b][0], sc[b][1]), fmaxf(sc[b][2], sc[b][3])),
-                      fmaxf(fmaxf(sc[b][4], sc[b][5]), fmaxf(sc[b][6], sc[b][7])));
-      t = fmaxf(t, __shfl_xor(t, 16));
-      t = fmaxf(t, __shfl_xor(t, 32));
+      // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
+      const float t = fmaxf(fmaxf(fmaxf(sc[b][0], sc[b][1]), fmaxf(sc[b][2], sc[b][3])),
+                            fmaxf(fmaxf(sc[b][4], sc[b][5]), fmaxf(sc[b][6], sc[b][7])));
       mx[b] = t * p.scale_log2;
       raise |= mx[b] > m[b] + kRaise;  // also true for the first finite score of a row (m = -inf)
     }
@@ -289,7 +288,10 @@ void swa_prefill_kernel(const PrefillParams p) {
     // rare: lift the reference points to the running maxima and rescale, then finish this chunk
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      const float m_new = fmaxf(m[b], mx[b]);
+      float t = mx[b];  // row maximum over the four lanes that share a token
+      t = fmaxf(t, __shfl_xor(t, 16));
+      t = fmaxf(t, __shfl_xor(t, 32));
+      const float m_new = fmaxf(m[b], t);
       const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
       const float alpha = fast_exp2(m[b] - m_safe);
       m[b] = m_new;
