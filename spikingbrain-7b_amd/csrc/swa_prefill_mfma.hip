@@ -166,25 +166,25 @@ void swa_prefill_kernel(const PrefillParams p) {
   const bool fetcher = wave < S::kFetchWaves;
   const int rows_per_wave = 32 / S::kFetchWaves;                         // 8 or 16
   const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the 16-key tile, +4 per load
-  uint4 stage_k[S::kLoads], stage_v[S::kLoads];
-  auto fetch = [&](int ch) {
+  uint4 stage_k[2][S::kLoads], stage_v[2][S::kLoads];  // chunk x travels in set (x - ch_begin) & 1
+  auto fetch = [&](int ch, uint4 (&sk_)[S::kLoads], uint4 (&sv_)[S::kLoads]) {
     const int t = min(max(2 * ch + (wave * rows_per_wave) / 16, first_tile), last_tile);
     const int64_t base = tile_base(t);
 #pragma unroll
     for (int u = 0; u < S::kLoads; ++u) {
       const int row = min(max((t << 4) + lrow + 4 * u, wg_lo), wg_hi - 1) - (t << 4);
       const int64_t off = base + (int64_t)row * p.kv_sr + c * 16;
-      stage_k[u] = load_stream16(p.k + off);
-      stage_v[u] = load_stream16(p.v + off);
+      sk_[u] = load_stream16(p.k + off);
+      sv_[u] = load_stream16(p.v + off);
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf, const uint4 (&sk_)[S::kLoads], const uint4 (&sv_)[S::kLoads]) {
     char *sk = smem + buf * 2 * kStage, *sv = sk + kStage;
 #pragma unroll
     for (int u = 0; u < S::kLoads; ++u) {
       const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
-      *reinterpret_cast<uint4 *>(sk + kk * kRowPad + c * 16) = stage_k[u];
-      *reinterpret_cast<uint4 *>(sv + kk * kRowPad + c * 16) = stage_v[u];
+      *reinterpret_cast<uint4 *>(sk + kk * kRowPad + c * 16) = sk_[u];
+      *reinterpret_cast<uint4 *>(sv + kk * kRowPad + c * 16) = sv_[u];
     }
   };
 
@@ -264,28 +264,8 @@ void swa_prefill_kernel(const PrefillParams p) {
     }
   };
 
-  // ---- chunk loop: one barrier per chunk, every wavefront visits every chunk -------------------
-  // (chunks outside a wavefront's own band come out fully masked and add zero)
-  if (fetcher) {
-    fetch(ch_begin);
-    stash(0);
-  }
-  __syncthreads();
-  int ch = ch_begin;
-  for (;;) {
-    bool raise = false;
-    for (; ch < ch_end; ++ch) {
-      const int buf = (ch - ch_begin) & 1;
-      const bool more = fetcher && ch + 1 < ch_end;
-      if (more) fetch(ch + 1);  // global loads fly while this chunk is computed
-      raise = scores(ch, buf);
-      if (raise) break;
-      accumulate(buf);
-      if (more) stash(buf ^ 1);
-      __syncthreads();
-    }
-    if (!raise) break;
-    // rare: lift the reference points to the running maxima and rescale, then finish this chunk
+  // lift the reference points to the running maxima and rescale what has been accumulated
+  auto rescale = [&]() {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       float t = mx[b];  // row maximum over the four lanes that share a token
@@ -299,15 +279,34 @@ void swa_prefill_kernel(const PrefillParams p) {
 #pragma unroll
       for (int mt = 0; mt < 8; ++mt) acc[b][mt] *= alpha;
     }
-    {
-      const int buf = (ch - ch_begin) & 1;
-      const bool more = fetcher && ch + 1 < ch_end;
-      accumulate(buf);
-      if (more) stash(buf ^ 1);
-      __syncthreads();
-      ++ch;
-    }
+  };
+
+  // ---- chunk loop: one barrier per chunk, every wavefront visits every chunk -------------------
+  // (chunks outside a wavefront's own band come out fully masked and add zero)
+  // Global loads run TWO chunks ahead of the arithmetic, in two register sets used alternately; the
+  // loop is written out for both sets so that every register index is static. Loads are issued
+  // unconditionally (past the end they re-read the last rows), so the wait in front of each LDS store
+  // counts exactly the loads that may still be in flight.
+  auto body = [&](int x, auto par) {
+    constexpr int P = decltype(par)::value;
+    if (fetcher) fetch(x + 2, stage_k[P], stage_v[P]);
+    if (scores(x, P)) rescale();
+    accumulate(P);
+    if (fetcher) stash(P ^ 1, stage_k[P ^ 1], stage_v[P ^ 1]);
+    __syncthreads();
+  };
+  if (fetcher) {
+    fetch(ch_begin, stage_k[0], stage_v[0]);
+    fetch(ch_begin + 1, stage_k[1], stage_v[1]);
+    stash(0, stage_k[0], stage_v[0]);
   }
+  __syncthreads();
+  int ch = ch_begin;
+  for (; ch + 1 < ch_end; ch += 2) {
+    body(ch, std::integral_constant<int, 0>{});
+    body(ch + 1, std::integral_constant<int, 1>{});
+  }
+  if (ch < ch_end) body(ch, std::integral_constant<int, 0>{});
 
   // ---- epilogue: lane (g, c) owns token c of each block, dims 32g + 8i + mt ---------------------
 #pragma unroll
