@@ -169,6 +169,34 @@ def bench_prefill(sb, dev, S=16, L=8192, iters=5):
     return res
 
 
+def bench_gla_prompt(sb, dev, S=16, L=8192, H=28, iters=3):
+    """The GLA layers' share of BASELINE config 4 (16 prompts x 8192 tokens): one packed launch
+    over token-major [tokens, H, D] projections, states read from and left in the slot cache.
+    The kernel is bound by fp32 vector issue: 3 vector operations (multiply, two multiply-adds)
+    per state element and token; the peak quoted is the unpacked fp32 vector rate (half of the
+    157.3 TFLOP/s that counts packed operations, which this build does not emit)."""
+    g = torch.Generator().manual_seed(0)
+    tokens = S * L
+    q, k, v = (torch.randn(tokens, H, D, generator=g).bfloat16().to(dev) for _ in range(3))
+    gate = (torch.nn.functional.logsigmoid(torch.randn(tokens, H, D, generator=g)) / 16).to(dev)
+    cache = torch.zeros(S, H, D, D, device=dev)
+    cu = torch.arange(0, tokens + 1, L, dtype=torch.int32, device=dev)
+    slots = torch.arange(S, dtype=torch.int32, device=dev)
+    out = torch.empty_like(q)
+    sb.ops.gla_recurrent_packed(q, k, v, gate, cache, cu, slots, out=out, max_seq_len=L)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        sb.ops.gla_recurrent_packed(q, k, v, gate, cache, cu, slots, out=out, max_seq_len=L)
+        b.record()
+    torch.cuda.synchronize()
+    ms = statistics.mean(a.elapsed_time(b) for a, b in evs)
+    flop = tokens * H * D * D * 5
+    return {"workload": f"GLA layer over BASELINE config 4's prompts: {S} x {L} tokens, H={H}, bf16 q/k/v, fp32 gate and state",
+            "kernel": "gla_sequence_kernel", "kernel_ms": round(ms, 3), "prompt_tokens_per_s_layer": round(tokens / (ms * 1e-3), 0),
+            "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 2), "frac_fp32_vector_peak_unpacked": round(flop / (ms * 1e-3) / 1e12 / 78.6, 4)}
+
+
 def bench_hybrid(sb, dev, B=256, steps=128, warmup=4):
     """BASELINE config 5: the cache work of 128 consecutive decode steps of the 28-layer stack
     (14 GLA state layers + 14 paged SWA layers, one shared block table), B=256, every sequence at a
@@ -253,7 +281,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
                                                     "28-layer hybrid decode step (config 5)")
-    ap.add_argument("--only", choices=("prefill", "hybrid"), default=None,
+    ap.add_argument("--only", choices=("prefill", "hybrid", "gla_prompt"), default=None,
                     help="run just that section and print its JSON (short runs for profiling one kernel)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -269,6 +297,9 @@ def main():
 
     if args.only == "prefill":
         print(json.dumps({"prefill": bench_prefill(sb, dev)}))
+        return
+    if args.only == "gla_prompt":
+        print(json.dumps({"gla_prompt": bench_gla_prompt(sb, dev)}))
         return
     if args.only == "hybrid":
         print(json.dumps({"hybrid_decode": bench_hybrid(sb, dev, steps=min(args.steps, 128))}))
@@ -377,6 +408,8 @@ def main():
 
         del states
         line["prefill"] = bench_prefill(sb, dev)
+        torch.cuda.empty_cache()
+        line["gla_prompt"] = bench_gla_prompt(sb, dev)
         torch.cuda.empty_cache()
         line["hybrid_decode"] = bench_hybrid(sb, dev)
         torch.cuda.empty_cache()

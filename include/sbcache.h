@@ -162,7 +162,9 @@ int sb_swa_decode(const sb_swa_decode_args *args);
  * GLA recurrent step(s) with in-place, slot-indexed state.
  * Replaces my_fused_recurrent_gla (vllm_hymeta/model_for_7B/my_fused_recurrent.py:9-153,
  * called from vllm_hymeta/model_for_7B/gla_attention.py:232) for T = 1, and
- * fla.ops.gla.fused_recurrent_gla as called from hf_7B_model/gla_attention.py:153 for T >= 1.
+ * fla.ops.gla.fused_recurrent_gla as called from hf_7B_model/gla_attention.py:153 for T >= 1
+ * (and fla's fused_chunk_gla as called from vllm_hymeta/model_for_7B/gla_attention.py:207-208:
+ * the same recurrence over a prompt, final state handed to the slot cache).
  * Per (b, h), for t = 0..T-1:
  *     S  <- exp(g_t)[:,None] * S + k_t[:,None] * v_t[None,:]        (S is [dk, dv])
  *     o_t = sum_dk (q_t*scale)[:,None] * S                          (uses the updated S)
@@ -191,6 +193,12 @@ typedef struct sb_gla_recurrent_args {
   int64_t state_stride_slot, state_stride_head;
   int64_t num_slots; /* bound for documentation; slot_idx values are trusted */
   void *stream;
+  /* Optional packed (varlen) form, the prefill loop of vllm_hymeta/model_for_7B/gla_attention.py:179-221
+   * (one fused_chunk_gla call per request, state copied into the slot cache) as ONE launch: when
+   * cu_seqlens ([batch+1] int32) is given, batch row b owns tokens cu_seqlens[b] .. cu_seqlens[b+1]-1 of
+   * q/k/v/g/out laid out [total_tokens, H, 128]; the *_stride_b fields are ignored, the *_stride_t
+   * fields are the token strides, and seq_len is only an upper bound of the row lengths. */
+  const int32_t *cu_seqlens;
 } sb_gla_recurrent_args;
 
 int sb_gla_recurrent(const sb_gla_recurrent_args *args);

@@ -67,7 +67,7 @@ class GlaRecurrentArgs(C.Structure):
         ("g_stride_b", i64), ("g_stride_h", i64), ("g_stride_t", i64),
         ("out_stride_b", i64), ("out_stride_h", i64), ("out_stride_t", i64),
         ("state_stride_slot", i64), ("state_stride_head", i64),
-        ("num_slots", i64), ("stream", vp),
+        ("num_slots", i64), ("stream", vp), ("cu_seqlens", vp),
     ]
 
 

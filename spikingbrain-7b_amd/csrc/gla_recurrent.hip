@@ -24,6 +24,7 @@ struct GlaParams {
   int64_t g_sb, g_sh, g_st;
   int64_t o_sb, o_sh, o_st;
   int64_t s_slot, s_head;
+  const int32_t *cu;  // packed form: tokens of row b are cu[b] .. cu[b+1]-1, or null
 };
 
 __device__ __forceinline__ float load_scalar(const void *p, int64_t i, int dtype) {
@@ -103,10 +104,10 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(const GlaParams p) {
     for (int i = 0; i < 16; ++i) {
       const int row = i * 8 + rg;
       const float kk = s_k[row], eg = s_eg[row], qq = s_q[row];
-      S[i].x = fmaf(eg, S[i].x, kk * vv.x);
-      S[i].y = fmaf(eg, S[i].y, kk * vv.y);
-      S[i].z = fmaf(eg, S[i].z, kk * vv.z);
-      S[i].w = fmaf(eg, S[i].w, kk * vv.w);
+      S[i].x = fmaf(kk, vv.x, eg * S[i].x);
+      S[i].y = fmaf(kk, vv.y, eg * S[i].y);
+      S[i].z = fmaf(kk, vv.z, eg * S[i].z);
+      S[i].w = fmaf(kk, vv.w, eg * S[i].w);
       o.x = fmaf(qq, S[i].x, o.x);
       o.y = fmaf(qq, S[i].y, o.y);
       o.z = fmaf(qq, S[i].z, o.z);
@@ -124,6 +125,180 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(const GlaParams p) {
 
 #pragma unroll
   for (int i = 0; i < 16; ++i) store_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4, S[i]);
+}
+
+// ---- many steps per call (prompts) ---------------------------------------------------------
+// The one-workgroup kernel above pays a global-memory round trip and two barriers per step. For
+// prompts the state is cut into four 32-column blocks, one single-wavefront workgroup each (no
+// barrier anywhere): lane = (column quad cq = lane / 8, row group rg = lane % 8) keeps rows
+// 16*rg .. 16*rg+15 of columns 4*cq .. 4*cq+3 of its block (64 values), the q.S reduction over the
+// row groups is three DPP adds inside each run of 8 lanes, and q, k, g, v of kSeqBlock steps are
+// fetched one block ahead as 4-element vectors (13 loads per block and lane, element types fixed
+// at compile time so that no load is followed by a type branch that would wait for it), then
+// converted and parked in LDS for the broadcast reads. Needs 4-element alignment of every
+// pointer and stride; the host falls back to the kernel above otherwise.
+constexpr int kSeqBlock = 8;
+constexpr int kSeqKernelMinSteps = 4;  // shorter calls (decode, speculative decode) use the kernel above
+
+__device__ __forceinline__ float sum8(float x) {  // sum over the 8 lanes of a run; every lane gets it
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));
+  return x;
+}
+
+// Four consecutive elements of type DT, as loaded (Raw) and as floats.
+template <int DT>
+struct Quad {
+  using Raw = u32x2_t;
+  static __device__ __forceinline__ Raw load(const void *p, int64_t i) {
+    return *reinterpret_cast<const Raw *>(reinterpret_cast<const uint16_t *>(p) + i);
+  }
+  static __device__ __forceinline__ float4 widen(Raw w) {
+    if (DT == SB_BF16) return make_float4(sb::bf16_lo(w.x), sb::bf16_hi(w.x), sb::bf16_lo(w.y), sb::bf16_hi(w.y));
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 a = __builtin_bit_cast(h2, w.x), b = __builtin_bit_cast(h2, w.y);
+    return make_float4((float)a.x, (float)a.y, (float)b.x, (float)b.y);
+  }
+  static __device__ __forceinline__ void store(void *p, int64_t i, float4 o) {
+    Raw w;
+    if (DT == SB_BF16) {
+      w.x = sb::pack_bf16(o.x, o.y);
+      w.y = sb::pack_bf16(o.z, o.w);
+    } else {
+      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+      const h2 a = {(_Float16)o.x, (_Float16)o.y}, b = {(_Float16)o.z, (_Float16)o.w};
+      w.x = __builtin_bit_cast(unsigned int, a);
+      w.y = __builtin_bit_cast(unsigned int, b);
+    }
+    *reinterpret_cast<Raw *>(reinterpret_cast<uint16_t *>(p) + i) = w;
+  }
+};
+template <>
+struct Quad<SB_F32> {
+  using Raw = f32x4_t;
+  static __device__ __forceinline__ Raw load(const void *p, int64_t i) {
+    return *reinterpret_cast<const Raw *>(reinterpret_cast<const float *>(p) + i);
+  }
+  static __device__ __forceinline__ float4 widen(Raw w) { return make_float4(w.x, w.y, w.z, w.w); }
+  static __device__ __forceinline__ void store(void *p, int64_t i, float4 o) {
+    const Raw w = {o.x, o.y, o.z, o.w};
+    *reinterpret_cast<Raw *>(reinterpret_cast<float *>(p) + i) = w;
+  }
+};
+
+template <bool kStateF32, int DT, int GDT>
+__global__ __launch_bounds__(64) void gla_sequence_kernel(const GlaParams p) {
+  using In = Quad<DT>;
+  using Gate = Quad<GDT>;
+  const int cb = blockIdx.x & 3;
+  const int bh = blockIdx.x >> 2;
+  const int b = bh / p.H;
+  const int h = bh - b * p.H;
+  const int64_t slot = p.slot_idx ? (int64_t)p.slot_idx[b] : (int64_t)b;
+  if (slot < 0) return;
+  int T = p.T;
+  int64_t qo, ko, vo, go, oo;  // element offset of this (row, head)'s first token
+  if (p.cu) {
+    const int64_t t0 = p.cu[b];
+    T = p.cu[b + 1] - (int)t0;
+    qo = t0 * p.q_st; ko = t0 * p.k_st; vo = t0 * p.v_st; go = t0 * p.g_st; oo = t0 * p.o_st;
+  } else {
+    qo = b * p.q_sb; ko = b * p.k_sb; vo = b * p.v_sb; go = b * p.g_sb; oo = b * p.o_sb;
+  }
+  if (T <= 0) return;
+  const int lane = threadIdx.x;
+  const int rg = lane & 7, cq = lane >> 3;
+  // loads: q, k, g as (step parity lane / 32, elements 4*(lane % 32) ..), v as (step lane / 8,
+  // columns 4*(lane % 8) .. of this block)
+  const int lstep = lane >> 5, lcol = (lane & 31) * 4;
+  qo += h * p.q_sh + lcol; ko += h * p.k_sh + lcol; go += h * p.g_sh + lcol;
+  vo += h * p.v_sh + cb * 32 + rg * 4;
+  oo += h * p.o_sh + cb * 32 + cq * 4;
+
+  __shared__ __attribute__((aligned(16))) float s_q[kSeqBlock][128];
+  __shared__ __attribute__((aligned(16))) float s_k[kSeqBlock][128];
+  __shared__ __attribute__((aligned(16))) float s_e[kSeqBlock][128];
+  __shared__ __attribute__((aligned(16))) float s_v[kSeqBlock][32];
+
+  char *sbase = reinterpret_cast<char *>(p.state) +
+                (slot * p.s_slot + (int64_t)h * p.s_head) * (kStateF32 ? 4 : 2);
+  float4 S[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) S[i] = load_state4<kStateF32>(sbase, (rg * 16 + i) * 32 + cb * 8 + cq);
+
+  typename In::Raw rq[kSeqBlock / 2], rk[kSeqBlock / 2], rv;
+  typename Gate::Raw rgt[kSeqBlock / 2];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < kSeqBlock / 2; ++i) {
+      const int64_t t = min(t0 + 2 * i + lstep, T - 1);  // past the end: the last token again, never used
+      rq[i] = In::load(p.q, qo + t * p.q_st);
+      rk[i] = In::load(p.k, ko + t * p.k_st);
+      rgt[i] = Gate::load(p.g, go + t * p.g_st);
+    }
+    rv = In::load(p.v, vo + (int64_t)min(t0 + cq, T - 1) * p.v_st);
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < T; t0 += kSeqBlock) {
+#pragma unroll
+    for (int i = 0; i < kSeqBlock / 2; ++i) {
+      float4 x = In::widen(rq[i]);
+      x.x *= p.scale; x.y *= p.scale; x.z *= p.scale; x.w *= p.scale;
+      *reinterpret_cast<float4 *>(&s_q[2 * i + lstep][lcol]) = x;
+      *reinterpret_cast<float4 *>(&s_k[2 * i + lstep][lcol]) = In::widen(rk[i]);
+      float4 e = Gate::widen(rgt[i]);
+      e.x = expf(e.x); e.y = expf(e.y); e.z = expf(e.z); e.w = expf(e.w);
+      *reinterpret_cast<float4 *>(&s_e[2 * i + lstep][lcol]) = e;
+    }
+    *reinterpret_cast<float4 *>(&s_v[cq][rg * 4]) = In::widen(rv);
+    if (t0 + kSeqBlock < T) fetch(t0 + kSeqBlock);  // in flight while this block is computed
+    auto step = [&](int s) {
+      const float4 vv = reinterpret_cast<const float4 *>(s_v[s])[cq];
+      float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float4 k4 = reinterpret_cast<const float4 *>(s_k[s])[rg * 4 + j];
+        const float4 e4 = reinterpret_cast<const float4 *>(s_e[s])[rg * 4 + j];
+        const float4 q4 = reinterpret_cast<const float4 *>(s_q[s])[rg * 4 + j];
+        const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, ee[4] = {e4.x, e4.y, e4.z, e4.w},
+                    qq[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float4 &Sr = S[4 * j + r];
+          Sr.x = fmaf(kk[r], vv.x, ee[r] * Sr.x);
+          Sr.y = fmaf(kk[r], vv.y, ee[r] * Sr.y);
+          Sr.z = fmaf(kk[r], vv.z, ee[r] * Sr.z);
+          Sr.w = fmaf(kk[r], vv.w, ee[r] * Sr.w);
+          o.x = fmaf(qq[r], Sr.x, o.x);
+          o.y = fmaf(qq[r], Sr.y, o.y);
+          o.z = fmaf(qq[r], Sr.z, o.z);
+          o.w = fmaf(qq[r], Sr.w, o.w);
+        }
+      }
+      o.x = sum8(o.x); o.y = sum8(o.y); o.z = sum8(o.z); o.w = sum8(o.w);
+      if (rg == 0) In::store(p.out, oo + (int64_t)(t0 + s) * p.o_st, o);
+    };
+    // (the state update is written as k*v + (e*S): both operations then work in place on the
+    // state's register; with e*S as the multiply-add every state register is copied once per step)
+    const int steps = min(kSeqBlock, T - t0);
+    for (int s = 0; s < steps; ++s) step(s);
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) store_state4<kStateF32>(sbase, (rg * 16 + i) * 32 + cb * 8 + cq, S[i]);
+}
+
+template <bool kStateF32, int DT>
+void launch_sequence(const GlaParams &p, int gdt, dim3 grid, hipStream_t st) {
+  if (gdt == SB_F32) gla_sequence_kernel<kStateF32, DT, SB_F32><<<grid, 64, 0, st>>>(p);
+  else if (gdt == SB_BF16) gla_sequence_kernel<kStateF32, DT, SB_BF16><<<grid, 64, 0, st>>>(p);
+  else gla_sequence_kernel<kStateF32, DT, SB_F16><<<grid, 64, 0, st>>>(p);
+}
+template <bool kStateF32>
+void launch_sequence(const GlaParams &p, dim3 grid, hipStream_t st) {
+  if (p.dtype == SB_F32) launch_sequence<kStateF32, SB_F32>(p, p.g_dtype, grid, st);
+  else if (p.dtype == SB_BF16) launch_sequence<kStateF32, SB_BF16>(p, p.g_dtype, grid, st);
+  else launch_sequence<kStateF32, SB_F16>(p, p.g_dtype, grid, st);
 }
 
 }  // namespace
@@ -162,6 +337,31 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
   p.o_sb = a->out_stride_b; p.o_sh = a->out_stride_h; p.o_st = a->out_stride_t;
   p.s_slot = a->state_stride_slot; p.s_head = a->state_stride_head;
 
+  p.cu = a->cu_seqlens;
+
+  // the prompt kernel moves q, k, v, g, out as 4-element vectors
+  auto quad_aligned = [](const void *ptr, int dt, int64_t sb_, int64_t sh, int64_t st) {
+    const uintptr_t bytes = dt == SB_F32 ? 16 : 8;
+    return (reinterpret_cast<uintptr_t>(ptr) % bytes) == 0 && sb_ % 4 == 0 && sh % 4 == 0 && st % 4 == 0;
+  };
+  const bool vectors_ok = quad_aligned(a->q, a->dtype, p.q_sb, p.q_sh, p.q_st) &&
+                          quad_aligned(a->k, a->dtype, p.k_sb, p.k_sh, p.k_st) &&
+                          quad_aligned(a->v, a->dtype, p.v_sb, p.v_sh, p.v_st) &&
+                          quad_aligned(a->g, a->g_dtype, p.g_sb, p.g_sh, p.g_st) &&
+                          quad_aligned(a->out, a->dtype, p.o_sb, p.o_sh, p.o_st);
+  if (a->cu_seqlens && !vectors_ok)
+    return fail(SB_ERR_UNSUPPORTED,
+                "sb_gla_recurrent: the packed form needs pointers and strides of q, k, v, g, out aligned to 4 elements");
+  if (a->cu_seqlens || (a->seq_len >= kSeqKernelMinSteps && vectors_ok)) {
+    // prompts: one wavefront per (row, head, 32-column block of the state), inputs staged ahead
+    if (groups * 4 > 0x7fffffffLL) return fail(SB_ERR_UNSUPPORTED, "sb_gla_recurrent: batch*heads too large");
+    const dim3 sgrid((unsigned)(groups * 4));
+    if (a->state_dtype == SB_F32)
+      launch_sequence<true>(p, sgrid, (hipStream_t)a->stream);
+    else
+      launch_sequence<false>(p, sgrid, (hipStream_t)a->stream);
+    return check_launch("gla_sequence_kernel");
+  }
   const dim3 grid((unsigned)groups), block(256);
   if (a->state_dtype == SB_F32)
     hipLaunchKernelGGL(gla_recurrent_kernel<true>, grid, block, 0, (hipStream_t)a->stream, p);

@@ -15,8 +15,8 @@
 //   The workgroup walks the union of its tokens' windows in chunks of 32 keys. Each chunk of K and V
 //   (32 rows x 256 B each) is fetched from global memory ONCE per workgroup (the first four wavefronts
 //   fetch 8 rows each with whole-row 16-byte lanes) into a double-buffered LDS stage whose rows are
-//   padded to 272 B; all wavefronts then read their MFMA operands from LDS. Global loads of chunk n+1
-//   are in flight while chunk n is computed.
+//   padded to 272 B; all wavefronts then read their MFMA operands from LDS. Global loads run two chunks
+//   ahead of the arithmetic (two register sets used alternately, the loop written out for both).
 //   Per chunk and column block: S^T = K Q^T (8 MFMA 16x16x32, tokens on the N axis), softmax numerators
 //   per lane for token lane%16 in log2 units, O^T += V^T P^T (8 MFMA). P stays in the lane that produced
 //   it; V^T operands come from an in-register 8x8 transpose shared by the two blocks.
@@ -25,9 +25,9 @@
 // Softmax reference point
 //   The numerators are exp2(s - m_ref) with a per-row reference m_ref that is only raised when some
 //   row of the wavefront scores more than kRaise (log2 units) above it, so they stay below 2^kRaise
-//   (exact in fp32 sums, inside fp16 range). Raising m_ref rescales the output accumulators; that code
-//   sits OUTSIDE the chunk loop (the loop is left and re-entered), which keeps the loop body free of
-//   branches around the accumulators.
+//   (exact in fp32 sums, inside fp16 range). The check uses each lane's own 8 keys, so the common case
+//   has no cross-lane traffic; raising m_ref (rare after the first chunks) takes the row maximum over
+//   the four lanes of a token and rescales the output accumulators.
 #include "common.h"
 #include "mfma_util.h"
 

@@ -78,6 +78,37 @@ def fused_recurrent_gla(
     return o, (state if output_final_state else None)
 
 
+def fused_chunk_gla(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    scale: float = -1,
+    initial_state: Optional[torch.Tensor] = None,
+    output_final_state: bool = False,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Name and call shape of fla's chunked GLA kernel as the reference's prefill loop uses it
+    (vllm_hymeta/model_for_7B/gla_attention.py:207-208): q, k, v, g [B, H, T, D], returns
+    (o [B, H, T, D], final_state [B, H, D, D] fp32 or None). Computed by the many-step recurrent
+    kernel (same mathematics, state crossing HBM once); scale -1 means D^-0.5 as in fla."""
+    return fused_recurrent_gla(q, k, v, g, None if scale == -1 else scale, initial_state, output_final_state)
+
+
+def gla_prefill_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gk: torch.Tensor, kv_cache: torch.Tensor,
+                       state_indices_tensor: torch.Tensor, query_start_loc: torch.Tensor, num_prefills: int,
+                       max_query_len: Optional[int] = None) -> torch.Tensor:
+    """The prefill half of `_prefill_and_mix_infer` (vllm_hymeta/model_for_7B/gla_attention.py:179-214)
+    as ONE launch: q, k, v, gk [num_tokens, H, D] with the prefill tokens first; prompt i owns tokens
+    query_start_loc[i] .. query_start_loc[i+1]-1, starts from the state in kv_cache[slot_i] (the
+    runner zeroes the slots of new prompts, `clear_prefill_slots`) and leaves its final state there,
+    with no per-request Python loop, slice copies or state copy. Returns o for the prefill tokens
+    [num_prefill_tokens, H, D] (before g_norm)."""
+    n = int(num_prefills)
+    cu = query_start_loc[:n + 1].to(torch.int32).contiguous()
+    slots = state_indices_tensor[:n].to(torch.int32).contiguous()
+    return ops.gla_recurrent_packed(q, k, v, gk, kv_cache, cu, slots, max_seq_len=max_query_len)
+
+
 @dataclass
 class GLACacheParams:
     """gla_cache.py:7-14."""

@@ -384,6 +384,56 @@ def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
     return out
 
 
+def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
+                         cu_seqlens: torch.Tensor, slot_idx: Optional[torch.Tensor] = None,
+                         scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                         max_seq_len: Optional[int] = None) -> torch.Tensor:
+    """The same recurrence over packed prompts: q, k, v, g [total_tokens, H, D] (token/head strides
+    free, contiguous D), sequence b owning tokens cu_seqlens[b] .. cu_seqlens[b+1]-1 (int32 device
+    vector [B+1]); its state is state[slot_idx[b]] (default b), advanced in place. One launch for
+    all sequences. Returns o [total_tokens, H, D]."""
+    dev = N.require_gpu(q, k, v, g, state, cu_seqlens, slot_idx, out)
+    if q.dim() != 3 or k.shape != q.shape or v.shape != q.shape or g.shape != q.shape:
+        raise ValueError("q, k, v, g must all be [total_tokens, H, D]")
+    Tt, H, D = q.shape
+    if not (k.dtype == q.dtype and v.dtype == q.dtype):
+        raise ValueError("q, k, v must share one dtype")
+    if state.dim() != 4 or state.shape[1:] != (H, D, D) or state.stride(3) != 1 or state.stride(2) != D:
+        raise ValueError(f"state must be [slots, {H}, {D}, {D}] with contiguous matrices")
+    if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2 or not cu_seqlens.is_contiguous():
+        raise ValueError("cu_seqlens must be a contiguous int32 vector [B+1]")
+    B = cu_seqlens.numel() - 1
+    for t, n in ((q, "q"), (k, "k"), (v, "v"), (g, "g")):
+        _inner_contiguous(t, n)
+    if slot_idx is not None:
+        if slot_idx.dtype != torch.int32 or slot_idx.dim() != 1 or slot_idx.numel() < B or not slot_idx.is_contiguous():
+            raise ValueError("slot_idx must be a contiguous int32 vector with one entry per sequence")
+    elif state.shape[0] < B:
+        raise ValueError(f"state has {state.shape[0]} slots for {B} sequences and no slot_idx")
+    if scale is None:
+        scale = D ** -0.5
+    if out is None:
+        out = torch.empty((Tt, H, D), dtype=q.dtype, device=dev)
+    elif out.shape != q.shape or out.dtype != q.dtype or out.stride(-1) != 1:
+        raise ValueError("out must match q in shape and dtype, with a contiguous last dimension")
+    if Tt == 0:
+        return out
+    a = N.GlaRecurrentArgs(
+        q=N.ptr(q), k=N.ptr(k), v=N.ptr(v), g=N.ptr(g), state=N.ptr(state), out=N.ptr(out),
+        slot_idx=N.ptr(slot_idx), batch=B, num_heads=H, seq_len=int(max_seq_len or Tt), head_dim=D,
+        dtype=N.dtype_code(q.dtype), g_dtype=N.dtype_code(g.dtype), state_dtype=N.dtype_code(state.dtype),
+        scale=float(scale),
+        q_stride_b=0, q_stride_h=q.stride(1), q_stride_t=q.stride(0),
+        k_stride_b=0, k_stride_h=k.stride(1), k_stride_t=k.stride(0),
+        v_stride_b=0, v_stride_h=v.stride(1), v_stride_t=v.stride(0),
+        g_stride_b=0, g_stride_h=g.stride(1), g_stride_t=g.stride(0),
+        out_stride_b=0, out_stride_h=out.stride(1), out_stride_t=out.stride(0),
+        state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
+        num_slots=state.shape[0], stream=N.stream_ptr(dev), cu_seqlens=N.ptr(cu_seqlens))
+    N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
+    return out
+
+
 def copy_blocks(cache_half: torch.Tensor, pairs: torch.Tensor) -> None:
     """cache_half [num_blocks, ...] with contiguous blocks; pairs [n, 2] int64 (src, dst) on the
     same device. One half (K or V) per call, as ops.copy_blocks does per layer at

@@ -144,3 +144,95 @@ def test_argument_errors(sb, dev):
         sb.ops.gla_recurrent(q64, q64, q64, q64, torch.zeros(2, 4, 64, 64, device=dev))
     with pytest.raises(RuntimeError, match="no CPU path"):
         sb.ops.gla_recurrent(q.cpu(), q.cpu(), q.cpu(), q.cpu(), st.cpu())
+
+
+@pytest.mark.parametrize("state_dtype", [torch.float32, torch.bfloat16])
+def test_packed_prompts_vs_oracle(sb, dev, state_dtype):
+    """Ragged prompts packed token-major [tokens, H, D] (the layout of the vLLM prefill loop,
+    vllm_hymeta/model_for_7B/gla_attention.py:179-214): one launch, each prompt starting from its
+    slot's state and leaving its final state there; lengths cover 1, below/at/above the 8-step
+    register block, and an empty prompt; one slot is -1 (skipped)."""
+    H, D = 4, 128
+    lens = [1, 7, 8, 9, 0, 37, 16]
+    n = len(lens)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    total = int(cu[-1])
+    q, k, v, gate = make(1, H, total, D, 77, relu=True)
+    q, k, v, gate = (x[0].transpose(0, 1).contiguous() for x in (q, k, v, gate))   # [tokens, H, D]
+    g = torch.Generator().manual_seed(3)
+    slots = 11
+    state = (torch.randn(slots, H, D, D, generator=g) * 0.02).to(state_dtype)
+    slot_idx = torch.randperm(slots, generator=g)[:n].to(torch.int32)
+    slot_idx[2] = -1
+    st = state.clone().to(dev)
+    sentinel = 7.0
+    out = torch.full((total, H, D), sentinel, dtype=q.dtype, device=dev)
+    sb.ops.gla_recurrent_packed(q.to(dev), k.to(dev), v.to(dev), gate.to(dev), st, torch.from_numpy(cu).to(dev),
+                                slot_idx.to(dev), out=out)
+    torch.cuda.synchronize()
+    got_o, got_S = out.float().cpu().numpy(), st.double().cpu().numpy()
+    tol = STATE_RTOL if state_dtype == torch.float32 else 2 ** -8
+    touched = set()
+    for i in range(n):
+        a, b = int(cu[i]), int(cu[i + 1])
+        s = int(slot_idx[i])
+        if s < 0:
+            assert (got_o[a:b] == sentinel).all()
+            continue
+        touched.add(s)
+        if a == b:
+            assert np.array_equal(got_S[s], state[s].double().numpy())
+            continue
+        hf = lambda x: x[a:b].transpose(0, 1)[None].float().numpy()      # [1, H, T, D]
+        ref_o, ref_S = G.gla_recurrent(hf(q), hf(k), hf(v), hf(gate), state[s:s + 1].double().numpy())
+        assert rel(got_S[s], ref_S[0]) <= tol, i
+        assert out_close(got_o[a:b], ref_o[0].transpose(1, 0, 2)), i
+    rest = sorted(set(range(slots)) - touched)
+    assert np.array_equal(got_S[rest], state.double().numpy()[rest])
+
+
+def test_packed_matches_per_prompt_calls_and_wrapper(sb, dev):
+    """The packed launch leaves bit-identical states and outputs to one call per prompt on the
+    head-first layout (both run the same per-element fp32 operations in the same order), and
+    `gla_prefill_packed` is that launch behind the argument order of the reference's prefill loop."""
+    H, D = 28, 128
+    lens = [130, 5, 64]
+    cu = torch.tensor([0, 130, 135, 199], dtype=torch.int32)
+    q, k, v, gate = make(1, H, 199, D, 5)
+    q, k, v, gate = (x[0].transpose(0, 1).contiguous().to(dev) for x in (q, k, v, gate))
+    cache = torch.zeros(6, H, D, D, device=dev)
+    slots = torch.tensor([4, 0, 2, 5], dtype=torch.int32, device=dev)        # one more than prefills
+    qsl = torch.tensor([0, 130, 135, 199, 200], dtype=torch.int32, device=dev)
+    o = sb.gla.gla_prefill_packed(q, k, v, gate, cache, slots, qsl, num_prefills=3)
+    assert o.shape == (199, H, D)
+    for i, s in enumerate([4, 0, 2]):
+        a, b = int(cu[i]), int(cu[i + 1])
+        hf = lambda x: x[a:b].transpose(0, 1).unsqueeze(0)
+        o_i, S_i = sb.gla.fused_chunk_gla(hf(q), hf(k), hf(v), hf(gate), initial_state=None, output_final_state=True)
+        assert torch.equal(S_i[0], cache[s])
+        assert torch.equal(o_i[0].transpose(0, 1), o[a:b])
+    assert (cache[[1, 3, 5]] == 0).all()
+
+
+def test_long_prompt_properties(sb, dev):
+    """T = 2048 steps: (1) with g = 0 and q = k = e_0 the state's row 0 is the running sum of v
+    and o_t = scale * sum_{s<=t} v_s (closed form); (2) splitting the prompt into two calls at a
+    step that is not a multiple of the register block reproduces the one-call result bit for bit."""
+    B, H, T, D = 2, 3, 2048, 128
+    g = torch.Generator().manual_seed(21)
+    v = torch.randn(B, H, T, D, generator=g).to(dev)
+    e0 = torch.zeros(B, H, T, D, device=dev); e0[..., 0] = 1.0
+    zero = torch.zeros(B, H, T, D, device=dev)
+    o, S = sb.fused_recurrent_gla(e0, e0, v, zero, scale=1.0, output_final_state=True)
+    run = v.double().cumsum(2)
+    assert (o.double() - run).abs().max().item() <= 5e-3
+    assert (S[:, :, 0].double() - run[:, :, -1]).abs().max().item() <= 5e-3
+    assert (S[:, :, 1:] == 0).all()
+    q, k, v2, gate = (x.to(dev) for x in make(B, H, T, D, 8, dtype=torch.float32))
+    o1, S1 = sb.fused_recurrent_gla(q, k, v2, gate, output_final_state=True)
+    cut = 1003
+    oa, Sa = sb.fused_recurrent_gla(q[:, :, :cut], k[:, :, :cut], v2[:, :, :cut], gate[:, :, :cut], output_final_state=True)
+    ob, Sb = sb.fused_recurrent_gla(q[:, :, cut:], k[:, :, cut:], v2[:, :, cut:], gate[:, :, cut:],
+                                    initial_state=Sa, output_final_state=True)
+    assert torch.equal(Sb, S1)
+    assert torch.equal(torch.cat([oa, ob], 2), o1)
