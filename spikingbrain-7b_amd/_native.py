@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libsbcache.so")
 SB_BF16, SB_F16, SB_F32 = 0, 1, 2
 SB_ERR_INVALID, SB_ERR_UNSUPPORTED, SB_ERR_WORKSPACE = -1, -2, -3
 SB_DECODE_FORCE_VALU = 1
+SB_DECODE_BALANCED = 2
 ABI_VERSION = 1
 
 _DTYPES = {torch.bfloat16: SB_BF16, torch.float16: SB_F16, torch.float32: SB_F32}
@@ -113,6 +114,7 @@ EXPORTS = {
     "sb_kv_append": (C.c_int, [C.POINTER(KvAppendArgs)]),
     "sb_swa_decode_auto_split": (i32, [i64, i32, i32, i32]),
     "sb_swa_decode_workspace_bytes": (sz, [i64, i32, i32, i32]),
+    "sb_swa_decode_prefer_balanced": (i32, [C.POINTER(i32), i64, i32, i32]),
     "sb_swa_decode": (C.c_int, [C.POINTER(SwaDecodeArgs)]),
     "sb_gla_recurrent": (C.c_int, [C.POINTER(GlaRecurrentArgs)]),
     "sb_copy_blocks": (C.c_int, [vp, vp, i64, i64, i64, vp]),

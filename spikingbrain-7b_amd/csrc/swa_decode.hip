@@ -321,6 +321,76 @@ __global__ __launch_bounds__(128) void swa_decode_merge_kernel(const DecodeParam
   if (d == 0 && p.lse) p.lse[rh] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
 }
 
+// Merge for the balanced split: the partials of row r are numbers w + r for the workgroups w whose
+// runs of chunks touch the row; which those are follows from seq_lens exactly as in the split kernel.
+template <typename E>
+__global__ __launch_bounds__(128) void swa_decode_merge_balanced_kernel(const DecodeParams p) {
+  const int64_t rh = blockIdx.x;  // r*Hq + hq
+  const int r = (int)(rh / p.Hq);
+  const int hq = (int)(rh - (int64_t)r * p.Hq);
+  const int d = threadIdx.x;
+  const int lane = d & 63;
+  int total = 0, before = 0;
+  for (int base = 0; base < p.rows; base += 64) {
+    const int rr = base + lane;
+    int n = 0;
+    if (rr < p.rows) {
+      const int hi = p.seq_lens[rr];
+      int lo = p.window_left >= 0 ? max(0, hi - 1 - p.window_left) : 0;
+      if (p.key_lo) lo = max(lo, p.key_lo[rr]);
+      n = hi > lo ? ((hi - 1) >> 5) - (lo >> 5) + 1 : 0;
+    }
+    int t = n, b = rr < r ? n : 0;
+#pragma unroll
+    for (int k = 1; k < 64; k <<= 1) {
+      t += __shfl_xor(t, k);
+      b += __shfl_xor(b, k);
+    }
+    total += t;
+    before += b;
+  }
+  int n_r = 0;
+  {
+    const int hi = p.seq_lens[r];
+    int lo = p.window_left >= 0 ? max(0, hi - 1 - p.window_left) : 0;
+    if (p.key_lo) lo = max(lo, p.key_lo[r]);
+    n_r = hi > lo ? ((hi - 1) >> 5) - (lo >> 5) + 1 : 0;
+  }
+  float tot = 0.f, L = 0.f, M = kNegInf;
+  if (n_r > 0) {
+    const int per = (total + p.n_wg - 1) / p.n_wg;
+    const int w_lo = before / per, w_hi = (before + n_r - 1) / per;
+    // a long row among short ones can have hundreds of partials: loads go out eight at a time
+    for (int w = w_lo; w <= w_hi; w += 8) {
+      float ms[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ms[j] = p.ws_ml[((int64_t)(min(w + j, w_hi) + r) * p.Hq + hq) * 2];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) M = fmaxf(M, ms[j]);
+    }
+    if (M != kNegInf) {
+      for (int w = w_lo; w <= w_hi; w += 8) {
+        float ms[8], ls[8], av[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int64_t part = (int64_t)(min(w + j, w_hi) + r) * p.Hq + hq;
+          ms[j] = p.ws_ml[part * 2];
+          ls[j] = p.ws_ml[part * 2 + 1];
+          av[j] = p.ws_acc[part * 128 + d];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float f = (w + j > w_hi || ms[j] == kNegInf) ? 0.f : fast_exp2(ms[j] - M);
+          tot = fmaf(av[j], f, tot);
+          L = fmaf(ls[j], f, L);
+        }
+      }
+    }
+  }
+  store_out<E>(p.out, (int64_t)r * p.o_sr + (int64_t)hq * p.o_sh + d, L > 0.f ? tot / L : 0.f);
+  if (d == 0 && p.lse) p.lse[rh] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
+}
+
 template <typename E>
 int launch_for_group(int G, dim3 grid, hipStream_t st, const DecodeParams &p) {
   switch (G) {
@@ -367,10 +437,48 @@ extern "C" int32_t sb_swa_decode_auto_split(int64_t num_rows, int32_t num_kv_hea
   return (int32_t)n;
 }
 
+// Rows up to which the balanced split is used (every wavefront sums over all rows' lengths).
+constexpr int64_t kBalancedMaxRows = 1024;
+
+// Workgroups per kv-head group of the balanced split: one per CU when the fixed split would have
+// launched about that many anyway, else as many as the fixed split.
+static int64_t balanced_workgroups(int64_t num_rows, int64_t n_split) {
+  const int64_t fixed = num_rows * n_split, cus = device_cu_count();
+  return (fixed * 2 >= cus && fixed <= cus * 2) ? cus : fixed;
+}
+
+// Partials of a launch: rows * n_split for the fixed split; the balanced split numbers them
+// workgroup + row. Sized for whichever is larger.
+static int64_t partial_slots(int64_t num_rows, int64_t n_split) {
+  const int64_t fixed = num_rows * n_split;
+  if (num_rows > kBalancedMaxRows) return fixed;
+  const int64_t balanced = balanced_workgroups(num_rows, n_split) + num_rows;
+  return balanced > fixed ? balanced : fixed;
+}
+
+extern "C" int32_t sb_swa_decode_prefer_balanced(const int32_t *host_seq_lens, int64_t num_rows,
+                                                 int32_t window_left, int32_t n_split) {
+  if (!host_seq_lens || num_rows <= 0 || num_rows > kBalancedMaxRows || n_split <= 1) return 0;
+  int64_t total = 0, longest = 0;
+  for (int64_t r = 0; r < num_rows; ++r) {
+    const int64_t hi = host_seq_lens[r];
+    const int64_t lo = (window_left >= 0 && hi - 1 - window_left > 0) ? hi - 1 - window_left : 0;
+    const int64_t n = hi > lo ? ((hi - 1) >> 5) - (lo >> 5) + 1 : 0;
+    total += n;
+    if (n > longest) longest = n;
+  }
+  const int64_t n_wg = balanced_workgroups(num_rows, n_split);
+  const int64_t fixed_run = (longest + n_split - 1) / n_split;  // chunks of the busiest workgroup
+  const int64_t balanced_run = (total + n_wg - 1) / n_wg;
+  // Working out the runs and restarting at a row boundary cost a balanced workgroup about as much
+  // as streaming 4 chunks (measured: even batches are 5 % faster with the fixed split).
+  return balanced_run + 4 < fixed_run ? 1 : 0;
+}
+
 extern "C" size_t sb_swa_decode_workspace_bytes(int64_t num_rows, int32_t num_q_heads,
                                                 int32_t head_size, int32_t n_split) {
   if (n_split <= 1 || num_rows <= 0 || num_q_heads <= 0 || head_size <= 0) return 0;
-  const int64_t parts = num_rows * num_q_heads * (int64_t)n_split;
+  const int64_t parts = partial_slots(num_rows, n_split) * num_q_heads;
   return (size_t)(round_up(parts * head_size * 4, 256) + round_up(parts * 2 * 4, 256));
 }
 
@@ -424,11 +532,12 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   p.out = (char *)a->out; p.lse = a->lse;
   p.block_table = a->block_table; p.kv_start = a->kv_start; p.row_seq = a->row_seq;
   p.seq_lens = a->seq_lens; p.key_lo = a->key_lo;
-  const int64_t parts = a->num_rows * a->num_q_heads * (int64_t)n_split;
+  const int64_t parts = partial_slots(a->num_rows, n_split) * a->num_q_heads;
   p.ws_acc = (float *)a->workspace;
   p.ws_ml = need ? (float *)((char *)a->workspace + round_up(parts * 128 * 4, 256)) : nullptr;
   p.Hq = a->num_q_heads; p.block_size = a->block_size > 0 ? a->block_size : 16;
   p.window_left = a->window_left; p.n_split = n_split;
+  p.rows = (int)a->num_rows; p.n_wg = 0;
   p.scale_log2 = a->scale * sb::kLog2e;
   p.q_sr = a->q_stride_row; p.q_sh = a->q_stride_head;
   p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
@@ -486,6 +595,8 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
       if (arc != SB_OK) return arc;
     }
   }
+  if (mfma && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
+    p.n_wg = (int)balanced_workgroups(a->num_rows, n_split);
   if (a->phases != 2) {
     if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
                                            (a->flags >> 4) & 7, st, p);
@@ -497,6 +608,11 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   if (rc != SB_OK || n_split == 1 || a->phases == 1) return rc;
 
   const dim3 mgrid((unsigned)(a->num_rows * a->num_q_heads));
+  if (p.n_wg > 0) {
+    if (a->dtype == SB_BF16) hipLaunchKernelGGL(swa_decode_merge_balanced_kernel<BF16>, mgrid, dim3(128), 0, st, p);
+    else hipLaunchKernelGGL(swa_decode_merge_balanced_kernel<F16>, mgrid, dim3(128), 0, st, p);
+    return check_launch("swa_decode_merge_balanced_kernel");
+  }
   if (a->dtype == SB_BF16) hipLaunchKernelGGL(swa_decode_merge_kernel<BF16>, mgrid, dim3(128), 0, st, p);
   else if (a->dtype == SB_F16) hipLaunchKernelGGL(swa_decode_merge_kernel<F16>, mgrid, dim3(128), 0, st, p);
   else hipLaunchKernelGGL(swa_decode_merge_kernel<F32>, mgrid, dim3(128), 0, st, p);

@@ -48,34 +48,33 @@ struct Chunk {
   uint4 v[8];          // V rows of this lane's 8 keys, dims 8c..8c+7
 };
 
-// kDepth = chunks in flight per wavefront besides the one being computed; kMaxThreads bounds the
-// workgroup size, which with one workgroup per CU fixes the register budget (256 threads: one
-// wavefront per SIMD, 512 registers; 512 threads: two per SIMD, 256 registers).
-template <typename E, int kDepth, int kMaxThreads>
-__global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(const DecodeParams p, const int G,
-                                                                                const int Hkv) {
-  const int64_t r = blockIdx.x;
-  const int split = blockIdx.z;
-  const int tid = threadIdx.x;
-  const int kvh = blockIdx.y * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(tid >> 6);
-  if (kvh >= Hkv) return;  // whole wavefront; there is no barrier in this kernel
-  const int lane = tid & 63;
+// Visible keys [lo, hi) of query row r and the 32-key chunks they touch: returns their number,
+// `first_chunk` = index of the first.
+__device__ __forceinline__ int row_chunks(const DecodeParams &p, const int32_t *seq_lens, int64_t r, int &lo, int &hi,
+                                          int &first_chunk) {
+  hi = seq_lens[r];
+  lo = p.window_left >= 0 ? max(0, hi - 1 - p.window_left) : 0;
+  if (p.key_lo) lo = max(lo, p.key_lo[r]);
+  first_chunk = lo >> 5;
+  return hi > lo ? ((hi - 1) >> 5) - first_chunk + 1 : 0;
+}
+
+// One wavefront's work on chunks [cb, ce) of row r for kv head kvh: attention over those keys
+// with an online softmax of its own, result written as the row's output (`direct`) or as the
+// fp32 partial number part_base + head * part_hs. kDepth = chunks in flight besides the one being
+// computed. `owns_newest`: this range ends the row's window (with a fused append it stores the
+// step's K/V row into the cache).
+template <typename E, int kDepth>
+__device__ __forceinline__ void split_segment(const DecodeParams &p, const int32_t *block_table, const int G,
+                                              const int kvh, const int lane, const int64_t r, const int lo,
+                                              const int hi, const int cb, const int ce, const bool owns_newest,
+                                              const bool direct, const int64_t part_base, const int part_hs) {
   const int g = lane >> 4;
   const int c = lane & 15;
-
   const int64_t seq = p.row_seq ? (int64_t)p.row_seq[r] : r;
-  const int hi = p.seq_lens[r];
-  int lo = p.window_left >= 0 ? max(0, hi - 1 - p.window_left) : 0;
-  if (p.key_lo) lo = max(lo, p.key_lo[r]);
   const bool any = hi > lo;
-
   const int first_tile = lo >> 4;
   const int last_tile = any ? (hi - 1) >> 4 : first_tile;
-  const int first_chunk = first_tile >> 1;
-  const int n_chunks = any ? (last_tile >> 1) - first_chunk + 1 : 0;
-  const int cps = (n_chunks + p.n_split - 1) / p.n_split;
-  const int cb = first_chunk + split * cps;
-  const int ce = min(cb + cps, first_chunk + n_chunks);
 
   // Q^T operands: head c of the group, dims of chunk 4s+g; zero rows pad the group to 16 heads
   uint4 qb[4];
@@ -92,7 +91,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
   for (int mt = 0; mt < 8; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = kNegInf, l = 0.f;
 
-  const bool paged = p.block_table != nullptr;
+  const bool paged = block_table != nullptr;
   const int64_t dense_row0 = (!paged && p.kv_start) ? p.kv_start[seq] : 0;
   const int64_t head_off = (int64_t)kvh * p.kv_sh;
 
@@ -101,7 +100,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
     const int i0 = t << 4;
     if (paged) {
       const int bi = i0 / p.block_size;
-      const int64_t blk = p.block_table[seq * p.bt_stride + bi];
+      const int64_t blk = block_table[seq * p.bt_stride + bi];
       return blk * p.kv_sb + (int64_t)(i0 - bi * p.block_size) * p.kv_sr + head_off;
     }
     return (dense_row0 + i0) * p.kv_sr + head_off;
@@ -285,7 +284,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
   }
 
   // ---- fused append: store the newest K/V row at its slot ---------------------------------
-  if (fused && any && ce == first_chunk + n_chunks && cb < ce && lane < 32) {
+  if (fused && any && owns_newest && cb < ce && lane < 32) {
     const int64_t slot = p.slot_mapping[r];
     if (slot >= 0) {
       const int64_t blk = slot / p.block_size;
@@ -304,7 +303,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
   // ---- this wavefront's result: lane (g, c < G) owns head c, dims 32g + 8i + mt --------------
   if (c < G) {
     const int hq = kvh * G + c;
-    if (p.n_split == 1) {
+    if (direct) {
       const float inv = l > 0.f ? 1.f / l : 0.f;
       char *dst = p.out + (r * p.o_sr + (int64_t)hq * p.o_sh + 32 * g) * 2;
 #pragma unroll
@@ -318,7 +317,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
       }
       if (g == 0 && p.lse) p.lse[r * p.Hq + hq] = l > 0.f ? (m + log2f(l)) * kLn2 : kNegInf;
     } else {
-      const int64_t part = (r * p.Hq + hq) * p.n_split + split;
+      const int64_t part = part_base + (int64_t)hq * part_hs;
       float *dst = p.ws_acc + part * 128 + 32 * g;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -333,19 +332,115 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
   }
 }
 
+// Fixed split: grid = (query rows, kv-head groups, splits); every row's chunks are cut into
+// n_split equal runs. kMaxThreads bounds the workgroup size, which with one workgroup per CU fixes
+// the register budget (256 threads: one wavefront per SIMD, 512 registers).
+template <typename E, int kDepth, int kMaxThreads>
+__global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(const DecodeParams p, const int G,
+                                                                                const int Hkv) {
+  const int64_t r = blockIdx.x;
+  const int split = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int kvh = blockIdx.y * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (kvh >= Hkv) return;  // whole wavefront; there is no barrier in this kernel
+  int lo, hi, first_chunk;
+  const int n_chunks = row_chunks(p, p.seq_lens, r, lo, hi, first_chunk);
+  const int cps = (n_chunks + p.n_split - 1) / p.n_split;
+  const int cb = first_chunk + split * cps;
+  const int ce = min(cb + cps, first_chunk + n_chunks);
+  split_segment<E, kDepth>(p, p.block_table, G, kvh, tid & 63, r, lo, hi, cb, ce, ce == first_chunk + n_chunks,
+                           p.n_split == 1, r * p.Hq * p.n_split + split, p.n_split);
+}
+
+__device__ __forceinline__ int wave_sum(int x) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) x += __shfl_xor(x, d);
+  return x;
+}
+__device__ __forceinline__ int wave_inclusive_scan(int x, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int y = __shfl_up(x, d);
+    if (lane >= d) x += y;
+  }
+  return x;
+}
+
+// Balanced split: the chunks of all rows, laid end to end in row order, are cut into gridDim.x
+// equal runs, one per workgroup, whatever the rows' lengths (a fixed split leaves the workgroups
+// of short rows idle while the longest finish). A run may cover the end of one row, whole short
+// rows and the start of another: one partial per (workgroup w, row r) it touches, stored as
+// partial number w + r (both grow along the runs, so the sum is unique). Every wavefront works
+// out the runs from seq_lens by itself: a few wave-wide sums, no communication. The tables are
+// separate restrict-qualified parameters: the partial stores of one row come before the table
+// lookups of the next, and only with the no-alias guarantee do those lookups stay scalar loads
+// (as vector loads each would wait for every K/V load in flight).
+template <typename E, int kDepth, int kMaxThreads>
+__global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_balanced_mfma_kernel(
+    const DecodeParams p, const int32_t *__restrict__ block_table, const int32_t *__restrict__ seq_lens, const int G,
+    const int Hkv) {
+  const int tid = threadIdx.x;
+  const int kvh = blockIdx.y * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (kvh >= Hkv) return;
+  const int lane = tid & 63;
+  const int w = blockIdx.x, n_wg = gridDim.x;
+  int total = 0;
+  for (int base = 0; base < p.rows; base += 64) {
+    int lo, hi, fc;
+    total += wave_sum(base + lane < p.rows ? row_chunks(p, seq_lens, base + lane, lo, hi, fc) : 0);
+  }
+  total = __builtin_amdgcn_readfirstlane(total);
+  const int per = (total + n_wg - 1) / n_wg;
+  const int c0 = w * per, c1 = min(c0 + per, total);
+  if (c0 >= c1) return;
+  int before = 0;  // chunks of the rows below `base`
+  for (int base = 0; base < p.rows && before < c1; base += 64) {
+    int lo, hi, fc;
+    const int n = base + lane < p.rows ? row_chunks(p, seq_lens, base + lane, lo, hi, fc) : 0;
+    const int incl = wave_inclusive_scan(n, lane);
+    const int start = before + incl - n;  // this lane's row begins at this chunk of the whole
+    uint64_t todo = __builtin_amdgcn_ballot_w64(n > 0 && start < c1 && start + n > c0);
+    while (todo) {
+      const int i = __builtin_ctzll(todo);
+      todo &= todo - 1;
+      const int r_start = __builtin_amdgcn_readlane(start, i);
+      const int64_t r = base + i;
+      int rlo, rhi, rfc;
+      const int rn = row_chunks(p, seq_lens, r, rlo, rhi, rfc);  // uniform: scalar loads
+      const int cb = rfc + max(c0 - r_start, 0), ce = rfc + min(c1 - r_start, rn);
+      split_segment<E, kDepth>(p, block_table, G, kvh, lane, r, rlo, rhi, cb, ce, ce == rfc + rn, false,
+                               (int64_t)(w + r) * p.Hq, 1);
+    }
+    before += __builtin_amdgcn_readlane(incl, 63);
+  }
+}
+
 }  // namespace
 
 namespace sb_host {
 
 // Launches the matrix-core split kernel (dtype bf16 or fp16, group size <= 16).
 // `rows`, `n_split` give grid x and z; the kv heads are spread over wavefronts and grid y.
+// With p.n_wg > 0 the balanced kernel runs instead: p.n_wg workgroups per kv-head group.
 void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
                                   hipStream_t st, const sb::DecodeParams &p) {
   // up to 4 wavefronts (kv heads) per workgroup: one per SIMD, each with the whole register file
   const int waves = Hkv < 4 ? Hkv : 4;
-  const dim3 grid(rows, (unsigned)((Hkv + waves - 1) / waves), n_split), block(64 * waves);
+  const unsigned ygroups = (unsigned)((Hkv + waves - 1) / waves);
+  const dim3 block(64 * waves);
   // measured on the 7B decode shape: one chunk of prefetch is as fast as two or three
   if (depth <= 0) depth = 1;
+  if (p.n_wg > 0) {
+    const dim3 grid((unsigned)p.n_wg, ygroups);
+    if (dtype == SB_BF16)
+      hipLaunchKernelGGL((swa_decode_balanced_mfma_kernel<sb::BF16, 1, 256>), grid, block, 0, st, p, p.block_table,
+                         p.seq_lens, G, Hkv);
+    else
+      hipLaunchKernelGGL((swa_decode_balanced_mfma_kernel<sb::F16, 1, 256>), grid, block, 0, st, p, p.block_table,
+                         p.seq_lens, G, Hkv);
+    return;
+  }
+  const dim3 grid(rows, ygroups, n_split);
 #define SB_LAUNCH(E, D) hipLaunchKernelGGL((swa_decode_split_mfma_kernel<E, D, 256>), grid, block, 0, st, p, G, Hkv)
   if (dtype == SB_BF16) {
     if (depth == 1) SB_LAUNCH(sb::BF16, 1);

@@ -18,6 +18,7 @@ struct DecodeParams {
   float *ws_acc;  // [rows, Hq, n_split, 128]
   float *ws_ml;   // [rows, Hq, n_split, 2]
   int Hq, block_size, window_left, n_split;
+  int rows, n_wg;  // balanced split: query rows, workgroups per kv-head group (0 = fixed split)
   float scale_log2;
   int64_t q_sr, q_sh, o_sr, o_sh;  // elements
   int64_t kv_sb, kv_sr, kv_sh;     // bytes

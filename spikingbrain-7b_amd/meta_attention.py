@@ -131,6 +131,7 @@ class MetaAttentionMetadata:
     query_lens: Optional[List[int]] = None
     host_seq_lens: Optional[List[int]] = None
     _prefill_plan: Any = None
+    _decode_balanced: Any = None     # split policy of this step's decode launch, decided once for all layers
 
     def prefill_plan(self, device) -> Any:
         """Tile layout of this (sub)step for ops.swa_prefill_attention, built once and shared by
@@ -484,11 +485,17 @@ class MetaAttentionImpl:
                 if fuse_append:
                     fused = dict(new_key=key[:n], new_value=value[:n],
                                  new_slot_mapping=decode_meta.slot_mapping.flatten()[:n].contiguous())
+                if decode_meta._decode_balanced is None:
+                    host_lens = decode_meta.host_seq_lens
+                    decode_meta._decode_balanced = bool(
+                        host_lens is not None and len(host_lens) >= n and
+                        ops.plan_decode_split(n, self.num_kv_heads, decode_meta.max_decode_seq_len or max(host_lens[:n]),
+                                              window_left, host_lens[:n]))
                 ops.swa_decode_attention(
                     decode_query, key_cache, value_cache, decode_meta.seq_lens_tensor[:n],
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
                     out=output[num_prefill_query_tokens:],
-                    max_seq_len=decode_meta.max_decode_seq_len or None, **fused)
+                    max_seq_len=decode_meta.max_decode_seq_len or None, balanced=decode_meta._decode_balanced, **fused)
         return output
 
     # -- multi-query forms: every query token becomes one row of the single-query kernel ----

@@ -92,6 +92,8 @@ def swa_decode_attention(
     n_split: int = 0,
     phases: int = 0,
     force_valu: bool = False,
+    balanced: Optional[bool] = None,
+    host_seq_lens=None,
     pipeline_depth: int = 0,
     new_key: Optional[torch.Tensor] = None,
     new_value: Optional[torch.Tensor] = None,
@@ -113,7 +115,11 @@ def swa_decode_attention(
     max_seq_len (a host int bounding seq_lens) only sizes the split; it defaults to a bound
     derived from the table/window shapes so that no device value is read back.
     phases: 0 = whole op; 1 = split kernel only, 2 = merge kernel only (profiling aid).
-    force_valu: run bf16/fp16 on the vector-ALU split kernel instead of the matrix-core one."""
+    force_valu: run bf16/fp16 on the vector-ALU split kernel instead of the matrix-core one.
+    balanced: cut the chunks of all rows, laid end to end, into equal runs (one per CU) instead of
+    cutting each row into n_split runs (bf16/fp16, <= 1024 rows): faster when the rows' lengths differ
+    a lot, a little slower when they do not. Default: decided from host_seq_lens (the same numbers
+    as seq_lens, as Python ints) when the caller has them, else off."""
     dev = N.require_gpu(q, key_cache, value_cache, seq_lens, block_table, kv_start, row_seq, key_lo, out)
     if q.dim() != 3:
         raise ValueError(f"q must be [rows, num_heads, head_size], got {tuple(q.shape)}")
@@ -176,8 +182,11 @@ def swa_decode_attention(
     if window_left >= 0:
         max_seq_len = max(1, max_seq_len)
     L = N.lib()
+    auto_balance = balanced is None
     if n_split == 0:
         n_split = L.sb_swa_decode_auto_split(R, Hkv, int(max_seq_len), int(window_left))
+    if auto_balance:
+        balanced = prefer_balanced_split(host_seq_lens, window_left, n_split) if host_seq_lens is not None else False
     ws_bytes = L.sb_swa_decode_workspace_bytes(R, Hq, D, n_split)
     ws = _workspace(dev, ws_bytes)
     a = N.SwaDecodeArgs(
@@ -187,7 +196,8 @@ def swa_decode_attention(
         workspace=N.ptr(ws), workspace_bytes=0 if ws is None else ws.numel(),
         num_rows=R, num_q_heads=Hq, num_kv_heads=Hkv, head_size=D, block_size=bs,
         window_left=int(window_left), max_seq_len=int(min(max_seq_len, 2**31 - 1)), n_split=int(n_split),
-        dtype=N.dtype_code(q.dtype), phases=int(phases), flags=(N.SB_DECODE_FORCE_VALU if force_valu else 0) | ((int(pipeline_depth) & 7) << 4),
+        dtype=N.dtype_code(q.dtype), phases=int(phases),
+        flags=(N.SB_DECODE_FORCE_VALU if force_valu else 0) | (N.SB_DECODE_BALANCED if balanced else 0) | ((int(pipeline_depth) & 7) << 4),
         scale=float(scale),
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
@@ -195,6 +205,23 @@ def swa_decode_attention(
         block_table_stride=bt_stride, stream=N.stream_ptr(dev), **fused)
     N.check(L.sb_swa_decode(C.byref(a)), "swa_decode")
     return (out, lse) if return_lse else out
+
+
+def prefer_balanced_split(host_seq_lens, window_left: int, n_split: int) -> bool:
+    """Whether the balanced split is expected to beat the fixed one for rows of these lengths
+    (host ints; no device access)."""
+    n = len(host_seq_lens)
+    if n == 0 or n_split <= 1:
+        return False
+    arr = (C.c_int32 * n)(*[int(x) for x in host_seq_lens])
+    return bool(N.lib().sb_swa_decode_prefer_balanced(arr, n, int(window_left), int(n_split)))
+
+
+def plan_decode_split(num_rows: int, num_kv_heads: int, max_seq_len: int, window_left: int, host_seq_lens) -> bool:
+    """The `balanced` choice swa_decode_attention would make for this step, for callers that run
+    many layers on the same lengths and want to decide once."""
+    n_split = N.lib().sb_swa_decode_auto_split(int(num_rows), int(num_kv_heads), int(max_seq_len), int(window_left))
+    return prefer_balanced_split(host_seq_lens, window_left, n_split)
 
 
 PREFILL_TILE = 64  # query tokens per workgroup of the prefill kernel

@@ -72,6 +72,24 @@ def test_auto_split_and_workspace(sb):
     assert need >= 64 * 28 * 8 * 130 * 4
 
 
+def test_balanced_split_policy_and_workspace(sb):
+    """Host-side rule for the balanced split: even, window-saturated batches keep the fixed split,
+    ragged ones take the balanced one; the workspace covers the partial numbering of both."""
+    L = sb._native.lib()
+
+    def prefer(lens, wl, n):
+        return L.sb_swa_decode_prefer_balanced((C.c_int32 * len(lens))(*lens), len(lens), wl, n)
+
+    assert prefer([4097 + 16 * i for i in range(64)], 4096, 4) == 0          # all rows fill the window
+    assert prefer([32768] + [256] * 31, -1, 8) == 1                          # one long row among short ones
+    assert prefer([100 + 120 * i for i in range(64)], -1, 4) == 1            # lengths spread over 100..7660
+    assert prefer([5000] * 8, 4096, 1) == 0                                  # nothing to balance without a split
+    assert prefer([], 4096, 4) == 0
+    # balanced numbering: (workgroups, here one per CU = 256) + rows partial slots per head
+    assert L.sb_swa_decode_workspace_bytes(48, 28, 128, 5) >= (256 + 48) * 28 * 130 * 4
+    assert L.sb_swa_decode_workspace_bytes(64, 28, 128, 8) >= 64 * 8 * 28 * 130 * 4
+
+
 def test_wrappers_refuse_cpu_tensors(sb):
     import torch
     k = torch.zeros(2, 4, 128, dtype=torch.bfloat16)

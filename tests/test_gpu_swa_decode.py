@@ -245,3 +245,78 @@ def test_argument_errors(sb, dev):
         sb.ops.swa_decode_attention(torch.zeros(2, 68, 128, device=dev, dtype=torch.bfloat16), kv[0], kv[1], sl, block_table=bt)
     with pytest.raises(ValueError, match="dense mode"):
         sb.ops.swa_decode_attention(q, kv[0], kv[1], sl)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", ["ragged", "many_rows", "tiny", "one_row"])
+def test_balanced_split_vs_oracle_and_fixed_split(sb, dev, dtype, case):
+    """The balanced split (runs of chunks cut across row boundaries) against the oracle and
+    against the fixed split, with rows that take a fraction of a run, rows that take several,
+    empty rows, more than 64 rows (two passes of the row scan), and a fused append."""
+    Hq, Hkv, D, bs = 28, 4, 128, 16
+    g = torch.Generator().manual_seed({"ragged": 1, "many_rows": 2, "tiny": 3, "one_row": 4}[case])
+    if case == "ragged":
+        lens, wl, n_split = [1, 700, 33, 0, 2049, 5, 64, 1300, 31, 32, 900, 0], 1023, 4
+    elif case == "many_rows":
+        lens, wl, n_split = [int(x) for x in torch.randint(0, 400, (150,), generator=g)], 255, 3
+    elif case == "tiny":
+        lens, wl, n_split = [3, 1, 2], -1, 5          # fewer chunks than workgroups
+    else:
+        lens, wl, n_split = [4000], 2047, 16
+    B = len(lens)
+    kv, tables = paged_problem(lens, bs, Hkv, D, dtype, 11)
+    q = torch.randn(B, Hq, D, generator=g).to(dtype)
+    scale = D ** -0.5
+    ref, ref_lse = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(),
+                                            tables.numpy(), lens, scale, wl, return_lse=True)
+    out, lse = run_paged(sb, dev, q, kv, tables, lens, wl, scale, n_split=n_split, balanced=True, return_lse=True)
+    fixed = run_paged(sb, dev, q, kv, tables, lens, wl, scale, n_split=n_split, balanced=False)
+    got = out.float().cpu().numpy()
+    live = [b for b in range(B) if lens[b] > 0]
+    dead = [b for b in range(B) if lens[b] == 0]
+    assert np.abs(got[live] - ref[live]).max() <= TOL[dtype]
+    assert np.abs(lse.cpu().numpy()[live] - ref_lse[live]).max() <= 2e-3
+    assert (got[dead] == 0).all() and np.isneginf(lse.cpu().numpy()[dead]).all()
+    assert (out.float() - fixed.float()).abs().max().item() <= 4e-3
+    # the same call twice gives the same bits (no dependence on workgroup arrival order)
+    again = run_paged(sb, dev, q, kv, tables, lens, wl, scale, n_split=n_split, balanced=True)
+    assert torch.equal(again, out)
+
+
+def test_balanced_split_fused_append(sb, dev):
+    """Fused append under the balanced split: cache and output equal append-then-attend."""
+    Hq, Hkv, D, bs, wl = 28, 4, 128, 16, 300
+    lens = [17, 301, 1200, 1, 640, 333, 96, 2000]
+    B = len(lens)
+    g = torch.Generator().manual_seed(5)
+    kv, tables = paged_problem(lens, bs, Hkv, D, torch.bfloat16, 13)
+    q = torch.randn(B, Hq, D, generator=g).bfloat16().to(dev)
+    nk, nv = (torch.randn(B, Hkv, D, generator=g).bfloat16().to(dev) for _ in range(2))
+    slots = torch.tensor([int(tables[b, (lens[b] - 1) // bs]) * bs + (lens[b] - 1) % bs for b in range(B)],
+                         dtype=torch.int64, device=dev)
+    slots[3] = -1                                       # padded row: nothing stored
+    sl = torch.tensor(lens, dtype=torch.int32, device=dev)
+    a, b_ = kv.clone().to(dev), kv.clone().to(dev)
+    sb.ops.kv_append(nk, nv, a[0], a[1], slots)
+    ref = sb.ops.swa_decode_attention(q, a[0], a[1], sl, block_table=tables.to(dev), window_left=wl, n_split=4, balanced=False)
+    out = sb.ops.swa_decode_attention(q, b_[0], b_[1], sl, block_table=tables.to(dev), window_left=wl, n_split=4,
+                                      balanced=True, new_key=nk, new_value=nv, new_slot_mapping=slots)
+    assert torch.equal(a, b_)
+    keep = [b for b in range(B) if b != 3]              # row 3's newest key is in neither cache
+    assert (out[keep].float() - ref[keep].float()).abs().max().item() <= 4e-3
+
+
+def test_split_policy_from_host_lengths(sb, dev):
+    """With host_seq_lens the op decides fixed/balanced itself: a ragged batch takes the balanced
+    split (bit-identical to asking for it), an even one the fixed split."""
+    Hq, Hkv, D, bs = 28, 4, 128, 16
+    g = torch.Generator().manual_seed(8)
+    for lens, expect in (([6000] + [200] * 15, True), ([1500] * 16, False)):
+        kv, tables = paged_problem(lens, bs, Hkv, D, torch.bfloat16, 17)
+        q = torch.randn(len(lens), Hq, D, generator=g).bfloat16()
+        n_split = sb._native.lib().sb_swa_decode_auto_split(len(lens), Hkv, max(lens), -1)
+        assert n_split > 1
+        assert sb.ops.plan_decode_split(len(lens), Hkv, max(lens), -1, lens) is expect
+        auto = run_paged(sb, dev, q, kv, tables, lens, -1, D ** -0.5, max_seq_len=max(lens), host_seq_lens=lens)
+        forced = run_paged(sb, dev, q, kv, tables, lens, -1, D ** -0.5, max_seq_len=max(lens), balanced=expect)
+        assert torch.equal(auto, forced)
