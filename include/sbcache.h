@@ -286,9 +286,37 @@ typedef struct sb_swa_prefill_args {
   int64_t kv_stride_block, kv_stride_row, kv_stride_head; /* elements; block stride unused when dense */
   int64_t block_table_stride;
   void *stream;
+  float *lse;      /* optional, fp32 [total_q, Hq], natural log: log-sum-exp of each query's scaled scores,
+                      the second result of _flash_attn_varlen_forward that fa_kernel_metatoken.py:254-257 merges on */
 } sb_swa_prefill_args;
 
 int sb_swa_prefill(const sb_swa_prefill_args *args);
+
+/* ------------------------------------------------------------------------------------
+ * Merge of two attention results over disjoint key sets by their log-sum-exps, in place:
+ *   lse' = lse - logsigmoid(lse - block_lse)
+ *   out' = out - sigmoid(block_lse - lse) * (out - block_out)      (fp32, rounded once to dtype)
+ * Replaces the TorchScript `_update_out_and_lse` of
+ *   vllm_hymeta/attention/fa_kernel_metatoken.py:110-122
+ * with which the window attention (out, lse) is combined with the attention of the same queries
+ * over the cached meta tokens (block_out, block_lse) at :189 and :277. A side whose lse is -inf
+ * (no visible key) contributes nothing; if both are -inf the row stays as it is.
+ * out, block_out: [rows, heads, head_size] of dtype (bf16/fp16/fp32), inner dimension contiguous,
+ * head_size a multiple of 8; lse, block_lse: fp32 [rows, heads] contiguous, natural log.
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_lse_merge_args {
+  void *out;
+  float *lse;
+  const void *block_out;
+  const float *block_lse;
+  int64_t rows;
+  int32_t heads, head_size, dtype;
+  int64_t out_stride_row, out_stride_head;             /* elements */
+  int64_t block_out_stride_row, block_out_stride_head;
+  void *stream;
+} sb_lse_merge_args;
+
+int sb_lse_merge(const sb_lse_merge_args *args);
 
 /* ------------------------------------------------------------------------------------
  * Device-side decode-step advance for the sliding-window paged cache: every sequence of

@@ -141,3 +141,36 @@ def lse_merge(out_a: np.ndarray, lse_a: np.ndarray, out_b: np.ndarray, lse_b: np
     logsig = -np.logaddexp(0.0, -d)          # logsigmoid(lse - lse_b)
     sig_rev = 1.0 / (1.0 + np.exp(d))        # sigmoid(lse_b - lse)
     return out_a - sig_rev[..., None] * (out_a - out_b), lse_a - logsig
+
+
+def metatoken_attention(q1: np.ndarray, q2: Optional[np.ndarray], k1: np.ndarray, k2: np.ndarray,
+                        v1: np.ndarray, v2: np.ndarray, scale: float, sliding_window: int) -> np.ndarray:
+    """The dense masked-softmax statement of meta-token attention,
+    vllm_hymeta/attention/fa_kernel_metatoken.py:372-405, for one sequence: ONE softmax per query
+    over [k2 | k1]. Query i of q1 (Lq queries, bottom-right aligned on the Lk keys of k1) sees every
+    meta token and the keys k with 0 <= pos_i - k < sliding_window (sliding_window <= 0: no window
+    limit); the meta tokens' own queries q2 see the meta tokens only. q1 [Lq, Hq, D], q2 [M, Hq, D]
+    or None, k1/v1 [Lk, Hkv, D], k2/v2 [M, Hkv, D]. Returns [Lq (+ M), Hq, D] float64, rows in the
+    order (q1, q2) as at :388 (the flash path moves the q2 rows to the front, :278-279)."""
+    Lq, Hq, D = q1.shape
+    Lk, Hkv, _ = k1.shape
+    M = k2.shape[0]
+    G = Hq // Hkv
+    q_id = Lk - Lq + np.arange(Lq)
+    k_id = np.arange(Lk)
+    visible = np.ones((Lq, M + Lk), bool)
+    win = q_id[:, None] >= k_id[None, :]
+    if sliding_window > 0:
+        win &= (q_id[:, None] - k_id[None, :]) < sliding_window
+    visible[:, M:] = win
+    q = q1
+    if q2 is not None:
+        q = np.concatenate([q1, q2], 0)
+        meta_rows = np.concatenate([np.ones((M, M), bool), np.zeros((M, Lk), bool)], 1)
+        visible = np.concatenate([visible, meta_rows], 0)
+    k = np.concatenate([k2, k1], 0).astype(np.float64)
+    v = np.concatenate([v2, v1], 0).astype(np.float64)
+    out = np.zeros((q.shape[0], Hq, D))
+    for h in range(Hq):
+        out[:, h] = masked_softmax_attention(q[:, h].astype(np.float64), k[:, h // G], v[:, h // G], ~visible, scale)
+    return out

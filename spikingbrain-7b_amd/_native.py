@@ -93,6 +93,16 @@ class SwaPrefillArgs(C.Structure):
         ("out_stride_row", i64), ("out_stride_head", i64),
         ("kv_stride_block", i64), ("kv_stride_row", i64), ("kv_stride_head", i64),
         ("block_table_stride", i64),
+        ("stream", vp), ("lse", vp),
+    ]
+
+
+class LseMergeArgs(C.Structure):
+    _fields_ = [
+        ("out", vp), ("lse", vp), ("block_out", vp), ("block_lse", vp),
+        ("rows", i64), ("heads", i32), ("head_size", i32), ("dtype", i32),
+        ("out_stride_row", i64), ("out_stride_head", i64),
+        ("block_out_stride_row", i64), ("block_out_stride_head", i64),
         ("stream", vp),
     ]
 
@@ -121,6 +131,7 @@ EXPORTS = {
     "sb_window_shift": (C.c_int, [C.POINTER(WindowShiftArgs)]),
     "sb_swa_prefill": (C.c_int, [C.POINTER(SwaPrefillArgs)]),
     "sb_window_advance": (C.c_int, [C.POINTER(WindowAdvanceArgs)]),
+    "sb_lse_merge": (C.c_int, [C.POINTER(LseMergeArgs)]),
     "sb_stream_copy": (C.c_int, [vp, vp, i64, vp]),
 }
 

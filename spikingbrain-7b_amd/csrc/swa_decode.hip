@@ -391,6 +391,50 @@ __global__ __launch_bounds__(128) void swa_decode_merge_balanced_kernel(const De
   if (d == 0 && p.lse) p.lse[rh] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
 }
 
+struct LseMergeParams {
+  char *out;
+  float *lse;
+  const char *block_out;
+  const float *block_lse;
+  int64_t pairs;  // rows * heads
+  int heads, vecs;  // 8-element vectors per (row, head)
+  int64_t o_sr, o_sh, b_sr, b_sh;  // elements
+};
+
+// One thread per 8 elements of a (row, head) pair. In log2-free form: with w = sigmoid(block_lse - lse),
+// out' = out - w (out - block_out) and lse' = lse - logsigmoid(lse - block_lse) = max + log(1 + exp(-|d|)).
+template <typename E>
+__global__ __launch_bounds__(256) void lse_merge_kernel(const LseMergeParams p) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t pair = t / p.vecs;
+  if (pair >= p.pairs) return;
+  const int vec = (int)(t - pair * p.vecs);
+  const int64_t r = pair / p.heads;
+  const int h = (int)(pair - r * p.heads);
+  const float la = p.lse[pair], lb = p.block_lse[pair];
+  if (lb == kNegInf) return;  // nothing to merge in (also covers both sides empty)
+  const float w = (la == kNegInf) ? 1.f : 1.f / (1.f + __expf(la - lb));
+  constexpr int kEsz = E::kPackWords == 8 ? 4 : 2;
+  char *op = p.out + (r * p.o_sr + (int64_t)h * p.o_sh + vec * 8) * kEsz;
+  const char *bp = p.block_out + (r * p.b_sr + (int64_t)h * p.b_sh + vec * 8) * kEsz;
+  float a[8], b[8];
+  unpack<E>(load_pack<E>(op), a);
+  unpack<E>(load_pack<E>(bp), b);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = a[i] - w * (a[i] - b[i]);
+  if constexpr (E::kPackWords == 8) {
+    reinterpret_cast<float4 *>(op)[0] = make_float4(a[0], a[1], a[2], a[3]);
+    reinterpret_cast<float4 *>(op)[1] = make_float4(a[4], a[5], a[6], a[7]);
+  } else {
+    *reinterpret_cast<uint4 *>(op) =
+        make_uint4(E::pack(a[0], a[1]), E::pack(a[2], a[3]), E::pack(a[4], a[5]), E::pack(a[6], a[7]));
+  }
+  if (vec == 0) {
+    const float hi = fmaxf(la, lb), lo = fminf(la, lb);
+    p.lse[pair] = (lo == kNegInf) ? hi : hi + log1pf(__expf(lo - hi));
+  }
+}
+
 template <typename E>
 int launch_for_group(int G, dim3 grid, hipStream_t st, const DecodeParams &p) {
   switch (G) {
@@ -617,4 +661,41 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   else if (a->dtype == SB_F16) hipLaunchKernelGGL(swa_decode_merge_kernel<F16>, mgrid, dim3(128), 0, st, p);
   else hipLaunchKernelGGL(swa_decode_merge_kernel<F32>, mgrid, dim3(128), 0, st, p);
   return check_launch("swa_decode_merge_kernel");
+}
+
+extern "C" int sb_lse_merge(const sb_lse_merge_args *a) {
+  using namespace sb_host;
+  if (!a) return fail(SB_ERR_INVALID, "sb_lse_merge: null args");
+  if (a->rows < 0 || a->heads < 0) return fail(SB_ERR_INVALID, "sb_lse_merge: negative size");
+  if (a->rows == 0 || a->heads == 0) return SB_OK;
+  if (!a->out || !a->lse || !a->block_out || !a->block_lse)
+    return fail(SB_ERR_INVALID, "sb_lse_merge: null tensor pointer");
+  if (a->head_size <= 0 || a->head_size % 8 != 0)
+    return fail(SB_ERR_UNSUPPORTED, "sb_lse_merge: head_size %d must be a positive multiple of 8", a->head_size);
+  int esz;
+  switch (a->dtype) {
+    case SB_BF16:
+    case SB_F16: esz = 2; break;
+    case SB_F32: esz = 4; break;
+    default: return fail(SB_ERR_UNSUPPORTED, "sb_lse_merge: unknown dtype %d", a->dtype);
+  }
+  const int64_t es[] = {a->out_stride_row, a->out_stride_head, a->block_out_stride_row, a->block_out_stride_head};
+  for (int64_t s : es)
+    if ((s * esz) % 16 != 0)
+      return fail(SB_ERR_INVALID, "sb_lse_merge: stride %lld elements is not 16-byte aligned", (long long)s);
+  if ((reinterpret_cast<uintptr_t>(a->out) | reinterpret_cast<uintptr_t>(a->block_out)) & 15u)
+    return fail(SB_ERR_INVALID, "sb_lse_merge: out/block_out base not 16-byte aligned");
+  LseMergeParams p;
+  p.out = (char *)a->out; p.lse = a->lse; p.block_out = (const char *)a->block_out; p.block_lse = a->block_lse;
+  p.pairs = a->rows * a->heads; p.heads = a->heads; p.vecs = a->head_size / 8;
+  p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
+  p.b_sr = a->block_out_stride_row; p.b_sh = a->block_out_stride_head;
+  const int64_t threads = p.pairs * p.vecs;
+  if ((threads + 255) / 256 > 0x7fffffffLL) return fail(SB_ERR_UNSUPPORTED, "sb_lse_merge: too many rows");
+  const dim3 grid((unsigned)((threads + 255) / 256));
+  hipStream_t st = (hipStream_t)a->stream;
+  if (a->dtype == SB_BF16) hipLaunchKernelGGL(lse_merge_kernel<BF16>, grid, dim3(256), 0, st, p);
+  else if (a->dtype == SB_F16) hipLaunchKernelGGL(lse_merge_kernel<F16>, grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL(lse_merge_kernel<F32>, grid, dim3(256), 0, st, p);
+  return check_launch("lse_merge_kernel");
 }

@@ -40,6 +40,7 @@ struct PrefillParams {
   const char *k;
   const char *v;
   char *out;
+  float *lse;                 // [total_q, Hq] natural-log log-sum-exp, or null
   const int32_t *block_table;
   const int64_t *kv_start;
   const int32_t *key_lo;      // [S] first visible key of each sequence, or null
@@ -48,6 +49,7 @@ struct PrefillParams {
   const int32_t *tile_seq;    // [tiles] sequence of each 64-token query tile
   const int32_t *tile_q0;     // [tiles] first query (index inside its sequence) of the tile
   int G, head_begin;          // query heads per kv head; first of them handled by this launch
+  int Hq;
   int num_tiles;
   int block_size, window_left;
   float scale_log2;
@@ -327,6 +329,9 @@ void swa_prefill_kernel(const PrefillParams p) {
         o.w = E::pack(acc[b][6][i] * inv, acc[b][7][i] * inv);
         *reinterpret_cast<uint4 *>(dst + 16 * i) = o;
       }
+      if (p.lse && g == 0)
+        p.lse[(int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.Hq + head0 + hd[b]] =
+            lt > 0.f ? (m[b] + log2f(lt)) * kLn2 : kNegInf;
     }
   }
 }
@@ -372,6 +377,7 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
 
   PrefillParams p;
   p.q = (const char *)a->q; p.k = (const char *)a->k; p.v = (const char *)a->v; p.out = (char *)a->out;
+  p.lse = a->lse; p.Hq = a->num_q_heads;
   p.block_table = a->block_table; p.kv_start = a->kv_start; p.key_lo = a->key_lo;
   p.cu_q = a->cu_seqlens_q; p.seq_lens_k = a->seq_lens_k; p.tile_seq = a->tile_seq; p.tile_q0 = a->tile_q0;
   p.G = a->num_q_heads / a->num_kv_heads; p.head_begin = 0;

@@ -423,9 +423,20 @@ class MetaAttentionImpl:
                                  "metadata attributes.")
         if attn_type != AttentionType.DECODER:
             raise NotImplementedError("only decoder self-attention is built on the gfx950 path")
-        if query2 is not None or key2 is not None or value2 is not None:
-            raise NotImplementedError("meta-token attention (query2/key2/value2) is not built; "
-                                      "the 7B model never passes it")
+        # Meta tokens (:817-819, fa_kernel_metatoken.py:124-280): every query also attends, without a
+        # mask, to num_meta_tokens cached rows key2/value2 shared by all sequences; in a prompt step
+        # the meta tokens' own queries (query2) attend to those rows only and their outputs come
+        # first in `output`.
+        with_meta = key2 is not None or value2 is not None
+        if query2 is not None and not with_meta:
+            raise ValueError("query2 needs key2 and value2")
+        if with_meta:
+            if key2 is None or value2 is None:
+                raise ValueError("key2 and value2 go together")
+            key2 = key2.view(-1, self.num_kv_heads, self.head_size)
+            value2 = value2.view(-1, self.num_kv_heads, self.head_size)
+            if key2.shape[0] != self.num_meta_tokens or value2.shape != key2.shape:
+                raise AssertionError(f"key2/value2 must hold num_meta_tokens = {self.num_meta_tokens} rows")
 
         window_left = self.sliding_window[0]
         query = query.view(-1, self.num_heads, self.head_size)
@@ -450,6 +461,22 @@ class MetaAttentionImpl:
 
         num_prefill_query_tokens = attn_metadata.num_prefill_tokens
         num_decode_query_tokens = attn_metadata.num_decode_tokens
+        num_meta_prefill_tokens = num_prefill_query_tokens
+        if query2 is not None:
+            query2 = query2.view(-1, self.num_heads, self.head_size)
+            if query2.shape[0] != self.num_meta_tokens:
+                raise AssertionError(f"query2 must hold num_meta_tokens = {self.num_meta_tokens} rows")
+            num_meta_prefill_tokens += self.num_meta_tokens
+            output[:self.num_meta_tokens] = ops.meta_token_attention(query2, key2, value2, self.scale)[0]
+        prefill_output = output[num_meta_prefill_tokens - num_prefill_query_tokens:num_meta_prefill_tokens]
+        decode_output = output[num_meta_prefill_tokens:]
+
+        def merge_meta(q_part, out_part, lse_part):
+            """out_part (attention over the window, log-sum-exp lse_part) takes in the meta tokens."""
+            if with_meta and q_part.shape[0] > 0:
+                meta_out, meta_lse = ops.meta_token_attention(q_part, key2, value2, self.scale)
+                ops.lse_merge(out_part, lse_part, meta_out, meta_lse)
+
         decode_query = query[num_prefill_query_tokens:]
         query = query[:num_prefill_query_tokens]
         assert query.shape[0] == num_prefill_query_tokens
@@ -458,25 +485,26 @@ class MetaAttentionImpl:
         if prefill_meta := attn_metadata.prefill_metadata:
             if kv_cache.numel() == 0 or prefill_meta.block_tables is None or prefill_meta.block_tables.numel() == 0:
                 # plain prompt run: keys and values are the in-flight tensors (:835-884)
-                self._varlen_inflight(query, key[:num_prefill_query_tokens], value[:num_prefill_query_tokens],
-                                      prefill_meta, output[:num_prefill_query_tokens], window_left)
+                lse = self._varlen_inflight(query, key[:num_prefill_query_tokens], value[:num_prefill_query_tokens],
+                                            prefill_meta, prefill_output, window_left, return_lse=with_meta)
             else:
                 # prefix hit / chunked prefill: keys and values come from the paged cache (:885-919)
                 assert prefill_meta.seq_lens is not None
                 assert prefill_meta.query_start_loc is not None
-                self._varlen_paged(query, key_cache, value_cache, prefill_meta.query_start_loc,
-                                   prefill_meta.seq_lens_tensor, prefill_meta.block_tables,
-                                   max(prefill_meta.seq_lens), output[:num_prefill_query_tokens], window_left,
-                                   meta=prefill_meta)
+                lse = self._varlen_paged(query, key_cache, value_cache, prefill_meta.query_start_loc,
+                                         prefill_meta.seq_lens_tensor, prefill_meta.block_tables,
+                                         max(prefill_meta.seq_lens), prefill_output, window_left,
+                                         meta=prefill_meta, return_lse=with_meta)
+            merge_meta(query, prefill_output, lse)
         if decode_meta := attn_metadata.decode_metadata:
             assert decode_meta.max_decode_query_len is not None
             if decode_meta.max_decode_query_len > 1:
                 # several query tokens per decoding sequence (:924-953)
                 assert decode_meta.query_start_loc is not None
-                self._varlen_paged(decode_query, key_cache, value_cache, decode_meta.query_start_loc,
-                                   decode_meta.seq_lens_tensor, decode_meta.block_tables,
-                                   decode_meta.max_decode_seq_len, output[num_prefill_query_tokens:], window_left,
-                                   meta=decode_meta)
+                lse = self._varlen_paged(decode_query, key_cache, value_cache, decode_meta.query_start_loc,
+                                         decode_meta.seq_lens_tensor, decode_meta.block_tables,
+                                         decode_meta.max_decode_seq_len, decode_output, window_left,
+                                         meta=decode_meta, return_lse=with_meta)
             else:
                 # one query token per sequence (:954-981); K/V were appended above, or are appended
                 # by this very launch when the step is a pure decode step
@@ -491,11 +519,13 @@ class MetaAttentionImpl:
                         host_lens is not None and len(host_lens) >= n and
                         ops.plan_decode_split(n, self.num_kv_heads, decode_meta.max_decode_seq_len or max(host_lens[:n]),
                                               window_left, host_lens[:n]))
-                ops.swa_decode_attention(
+                res = ops.swa_decode_attention(
                     decode_query, key_cache, value_cache, decode_meta.seq_lens_tensor[:n],
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
-                    out=output[num_prefill_query_tokens:],
+                    out=decode_output, return_lse=with_meta,
                     max_seq_len=decode_meta.max_decode_seq_len or None, balanced=decode_meta._decode_balanced, **fused)
+                lse = res[1] if with_meta else None
+            merge_meta(decode_query, decode_output, lse)
         return output
 
     # -- multi-query forms: every query token becomes one row of the single-query kernel ----
@@ -520,39 +550,44 @@ class MetaAttentionImpl:
             return None
         return plan
 
-    def _varlen_inflight(self, q, k, v, meta, out, window_left):
+    def _varlen_inflight(self, q, k, v, meta, out, window_left, return_lse=False):
+        """Returns the fp32 [T, Hq] log-sum-exp when asked for, else None."""
         T = q.shape[0]
         if T == 0:
-            return
+            return None
         if k.stride() != v.stride():
             v = v.contiguous()
             k = k.contiguous()
         plan = self._plan_for(meta, q)
         if plan is not None and plan.total_k <= k.shape[0]:
-            ops.swa_prefill_attention(q, k, v, plan=plan, window_left=window_left, scale=self.scale, out=out,
-                                      kv_start=meta.seq_start_loc.to(torch.int64)[:-1].contiguous())
-            return
+            res = ops.swa_prefill_attention(q, k, v, plan=plan, window_left=window_left, scale=self.scale, out=out,
+                                            kv_start=meta.seq_start_loc.to(torch.int64)[:-1].contiguous(),
+                                            return_lse=return_lse)
+            return res[1] if return_lse else None
         row_seq, j, _ = self._rows(meta.query_start_loc, T)
         seq_lens_row = (j + 1).to(torch.int32)
-        ops.swa_decode_attention(
+        res = ops.swa_decode_attention(
             q, k, v, seq_lens_row, kv_start=meta.seq_start_loc.to(torch.int64)[:-1].contiguous(),
             row_seq=row_seq.to(torch.int32), kv_strides=(0, k.stride(0), k.stride(1)),
             num_kv_heads=self.num_kv_heads, window_left=window_left, scale=self.scale, out=out,
-            max_seq_len=meta.max_prefill_seq_len or None)
+            max_seq_len=meta.max_prefill_seq_len or None, return_lse=return_lse)
+        return res[1] if return_lse else None
 
     def _varlen_paged(self, q, key_cache, value_cache, query_start_loc, seq_lens_tensor, block_tables,
-                      max_seq_len, out, window_left, meta=None):
+                      max_seq_len, out, window_left, meta=None, return_lse=False):
         T = q.shape[0]
         if T == 0:
-            return
+            return None
         plan = self._plan_for(meta, q) if meta is not None else None
         if plan is not None and block_tables.shape[1] * key_cache.shape[1] >= plan.max_k:
-            ops.swa_prefill_attention(q, key_cache, value_cache, plan=plan, block_table=block_tables,
-                                      window_left=window_left, scale=self.scale, out=out)
-            return
+            res = ops.swa_prefill_attention(q, key_cache, value_cache, plan=plan, block_table=block_tables,
+                                            window_left=window_left, scale=self.scale, out=out, return_lse=return_lse)
+            return res[1] if return_lse else None
         row_seq, j, lens = self._rows(query_start_loc, T)
         # query j of a run of n queries in a sequence of L keys sits at key index L - n + j
         seq_lens_row = (seq_lens_tensor.to(torch.int64)[row_seq] - lens[row_seq] + j + 1).to(torch.int32)
-        ops.swa_decode_attention(
+        res = ops.swa_decode_attention(
             q, key_cache, value_cache, seq_lens_row, block_table=block_tables, row_seq=row_seq.to(torch.int32),
-            window_left=window_left, scale=self.scale, out=out, max_seq_len=max_seq_len or None)
+            window_left=window_left, scale=self.scale, out=out, max_seq_len=max_seq_len or None,
+            return_lse=return_lse)
+        return res[1] if return_lse else None

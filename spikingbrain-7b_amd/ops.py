@@ -274,8 +274,10 @@ def swa_prefill_attention(
     window_left: int = -1,
     scale: Optional[float] = None,
     out: Optional[torch.Tensor] = None,
+    return_lse: bool = False,
 ):
     """Causal sliding-window attention for q [total_q, Hq, D] packed sequence after sequence.
+    With return_lse also the fp32 [total_q, Hq] natural-log log-sum-exp of each query's scores.
 
     query_lens / seq_lens_k: per-sequence host ints (keys default to the queries: plain prompt), or a
     prebuilt `plan`. Query j of a sequence sits at key position seq_len_k - query_len + j.
@@ -346,8 +348,9 @@ def swa_prefill_attention(
         if out.shape != q.shape or out.dtype != q.dtype:
             raise ValueError("out must match q in shape and dtype")
         _inner_contiguous(out, "out")
+    lse = torch.full((Tq, Hq), float("-inf"), dtype=torch.float32, device=dev) if return_lse else None
     if plan.num_tiles == 0:
-        return out
+        return (out, lse) if return_lse else out
     a = N.SwaPrefillArgs(
         q=N.ptr(q), k=N.ptr(k), v=N.ptr(v), out=N.ptr(out),
         block_table=N.ptr(block_table), kv_start=N.ptr(kv_start) if block_table is None else None,
@@ -358,9 +361,50 @@ def swa_prefill_attention(
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
         kv_stride_block=strides[0], kv_stride_row=strides[1], kv_stride_head=strides[2],
-        block_table_stride=bt_stride, stream=N.stream_ptr(dev))
+        block_table_stride=bt_stride, stream=N.stream_ptr(dev), lse=N.ptr(lse))
     N.check(N.lib().sb_swa_prefill(C.byref(a)), "swa_prefill")
-    return out
+    return (out, lse) if return_lse else out
+
+
+def lse_merge(out: torch.Tensor, lse: torch.Tensor, block_out: torch.Tensor, block_lse: torch.Tensor) -> None:
+    """In place: (out, lse) becomes the attention over the union of the key sets behind (out, lse)
+    and (block_out, block_lse). out/block_out [rows, H, D]; lse/block_lse fp32 [rows, H], natural log."""
+    dev = N.require_gpu(out, lse, block_out, block_lse)
+    if out.dim() != 3 or block_out.shape != out.shape or block_out.dtype != out.dtype:
+        raise ValueError("out and block_out must be [rows, heads, head_size] of one dtype")
+    R, H, D = out.shape
+    for t, name in ((lse, "lse"), (block_lse, "block_lse")):
+        if t.shape != (R, H) or t.dtype != torch.float32 or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous float32 [rows, heads] tensor")
+    _inner_contiguous(out, "out")
+    _inner_contiguous(block_out, "block_out")
+    a = N.LseMergeArgs(out=N.ptr(out), lse=N.ptr(lse), block_out=N.ptr(block_out), block_lse=N.ptr(block_lse),
+                       rows=R, heads=H, head_size=D, dtype=N.dtype_code(out.dtype),
+                       out_stride_row=out.stride(0), out_stride_head=out.stride(1),
+                       block_out_stride_row=block_out.stride(0), block_out_stride_head=block_out.stride(1),
+                       stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_lse_merge(C.byref(a)), "lse_merge")
+
+
+def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, scale: Optional[float] = None):
+    """Non-causal attention of every query row over the same few cached meta tokens
+    (k2, v2 [M, Hkv, D]), as the second attention of fa_kernel_metatoken.py:174-188 / 261-275.
+    Returns (out [rows, Hq, D], lse fp32 [rows, Hq]). Runs on the single-query kernel: every row is
+    a query at position M-1 of one shared dense sequence."""
+    dev = N.require_gpu(q, k2, v2)
+    R = q.shape[0]
+    M, Hkv, D = k2.shape
+    if v2.shape != k2.shape or k2.dtype != q.dtype or v2.dtype != q.dtype:
+        raise ValueError("k2 and v2 must be [meta_tokens, num_kv_heads, head_size] of q's dtype")
+    _inner_contiguous(k2, "k2")
+    _inner_contiguous(v2, "v2")
+    if k2.stride() != v2.stride():
+        raise ValueError("k2 and v2 must share their strides")
+    zeros32 = torch.zeros(R, dtype=torch.int32, device=dev)
+    return swa_decode_attention(
+        q, k2, v2, torch.full((R,), M, dtype=torch.int32, device=dev), kv_start=torch.zeros(1, dtype=torch.int64, device=dev),
+        row_seq=zeros32, kv_strides=(0, k2.stride(0), k2.stride(1)), num_kv_heads=Hkv, window_left=-1, scale=scale,
+        return_lse=True, max_seq_len=M, n_split=1)
 
 
 def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,

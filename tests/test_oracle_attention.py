@@ -133,3 +133,37 @@ def test_lse_merge_equals_attention_over_union():
     o, l = A.lse_merge(oA, lA, oB, lB)
     np.testing.assert_allclose(o, oU, rtol=1e-10)
     np.testing.assert_allclose(l, lU, rtol=1e-10)
+
+
+def test_metatoken_attention_is_window_attention_merged_with_meta_attention():
+    """The one-softmax statement (fa_kernel_metatoken.py:372-405) against the two-attention +
+    log-sum-exp merge the flash path runs (:124-194): pins both to the same mathematics; also the
+    closed case of no cached keys visible beyond the meta tokens."""
+    r = rng(21)
+    Hq, Hkv, D, M, Lk, Lq, W = 4, 2, 8, 6, 11, 3, 5
+    q1 = r.standard_normal((Lq, Hq, D)); q2 = r.standard_normal((M, Hq, D))
+    k1 = r.standard_normal((Lk, Hkv, D)); v1 = r.standard_normal((Lk, Hkv, D))
+    k2 = r.standard_normal((M, Hkv, D)); v2 = r.standard_normal((M, Hkv, D))
+    out = A.metatoken_attention(q1, q2, k1, k2, v1, v2, 0.3, W)
+    assert out.shape == (Lq + M, Hq, D)
+    G = Hq // Hkv
+    none = np.zeros((1, 1), bool)
+    for h in range(Hq):
+        for i in range(Lq):
+            pos = Lk - Lq + i
+            ks = slice(max(0, pos - W + 1), pos + 1)
+            oa, la = A.masked_softmax_attention(q1[i:i + 1, h], k1[ks, h // G], v1[ks, h // G], none, 0.3, return_lse=True)
+            ob, lb = A.masked_softmax_attention(q1[i:i + 1, h], k2[:, h // G], v2[:, h // G], none, 0.3, return_lse=True)
+            o, _ = A.lse_merge(oa, la, ob, lb)
+            np.testing.assert_allclose(out[i, h], o[0], rtol=1e-10)
+        om = A.masked_softmax_attention(q2[:, h], k2[:, h // G], v2[:, h // G], none, 0.3)
+        np.testing.assert_allclose(out[Lq:, h], om, rtol=1e-10)
+    # meta values all equal to c and a query orthogonal to every window key: result between c and the window average
+    v2c = np.full_like(v2, 2.0)
+    k1z = np.zeros_like(k1)
+    k2z = np.zeros_like(k2)
+    o = A.metatoken_attention(q1, None, k1z, k2z, np.full_like(v1, 5.0), v2c, 0.3, W)
+    # equal scores everywhere: M meta tokens (value 2) and min(W, pos+1) window keys (value 5)
+    for i in range(Lq):
+        n = min(W, Lk - Lq + i + 1)
+        np.testing.assert_allclose(o[i], (2.0 * M + 5.0 * n) / (M + n), rtol=1e-12)
