@@ -293,6 +293,52 @@ typedef struct sb_swa_prefill_args {
 int sb_swa_prefill(const sb_swa_prefill_args *args);
 
 /* ------------------------------------------------------------------------------------
+ * Per-row symmetric INT8 K/V (W8ASpike/window_attention.py:183-186 with quantize_sym, :227-237):
+ *   scale = clamp(max|row| / 127, 1e-5, 1e4); code = clamp(round_half_even(x / scale), -128, 127)
+ * for every (token, kv head) row of head_size = 128 values. The reference re-quantises the whole
+ * window at every step (and dequantises at once: "fake" quantisation); here a row is quantised
+ * once, when it enters the cache, and stays 1 byte per value in HBM: half the bytes a decode
+ * step reads. Codes and scales are bit-identical to quantize_sym's.
+ *
+ * sb_kv_append_int8: slot-mapped append (same slot_mapping contract as sb_kv_append).
+ *   key, value      [num_tokens, num_kv_heads, 128] of dtype (bf16/fp16/fp32)
+ *   k_cache, v_cache int8 [num_blocks, block_size, num_kv_heads, 128] (strides in bytes = elements)
+ *   k_scale, v_scale fp32 [num_blocks, num_kv_heads, block_size] contiguous (head-major inside a
+ *                   block: the 16 scales a 16-key tile of one head needs are one 64-byte run)
+ * sb_quantize_sym: out = (code * scale) rounded to dtype, i.e. quantize_sym itself, for K/V that
+ *   are attended to before they are cached (the prompt step); in == out is allowed.
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_kv_append_int8_args {
+  const void *key;
+  const void *value;
+  void *k_cache;
+  void *v_cache;
+  float *k_scale;
+  float *v_scale;
+  const int64_t *slot_mapping;
+  int64_t num_tokens;
+  int32_t num_kv_heads, head_size, block_size, dtype;
+  int64_t key_stride_token, key_stride_head;     /* elements */
+  int64_t value_stride_token, value_stride_head;
+  int64_t cache_stride_block, cache_stride_row, cache_stride_head; /* bytes */
+  void *stream;
+} sb_kv_append_int8_args;
+
+int sb_kv_append_int8(const sb_kv_append_int8_args *args);
+
+typedef struct sb_quantize_sym_args {
+  const void *in;  /* [rows, heads, 128] */
+  void *out;
+  int64_t rows;
+  int32_t heads, head_size, dtype;
+  int64_t in_stride_row, in_stride_head;   /* elements */
+  int64_t out_stride_row, out_stride_head;
+  void *stream;
+} sb_quantize_sym_args;
+
+int sb_quantize_sym(const sb_quantize_sym_args *args);
+
+/* ------------------------------------------------------------------------------------
  * Merge of two attention results over disjoint key sets by their log-sum-exps, in place:
  *   lse' = lse - logsigmoid(lse - block_lse)
  *   out' = out - sigmoid(block_lse - lse) * (out - block_out)      (fp32, rounded once to dtype)

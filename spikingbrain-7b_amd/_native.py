@@ -107,6 +107,26 @@ class LseMergeArgs(C.Structure):
     ]
 
 
+class KvAppendInt8Args(C.Structure):
+    _fields_ = [
+        ("key", vp), ("value", vp), ("k_cache", vp), ("v_cache", vp), ("k_scale", vp), ("v_scale", vp),
+        ("slot_mapping", vp), ("num_tokens", i64),
+        ("num_kv_heads", i32), ("head_size", i32), ("block_size", i32), ("dtype", i32),
+        ("key_stride_token", i64), ("key_stride_head", i64),
+        ("value_stride_token", i64), ("value_stride_head", i64),
+        ("cache_stride_block", i64), ("cache_stride_row", i64), ("cache_stride_head", i64),
+        ("stream", vp),
+    ]
+
+
+class QuantizeSymArgs(C.Structure):
+    _fields_ = [
+        ("in_", vp), ("out", vp), ("rows", i64), ("heads", i32), ("head_size", i32), ("dtype", i32),
+        ("in_stride_row", i64), ("in_stride_head", i64), ("out_stride_row", i64), ("out_stride_head", i64),
+        ("stream", vp),
+    ]
+
+
 class WindowAdvanceArgs(C.Structure):
     _fields_ = [
         ("n_tokens", vp), ("lo", vp), ("hi", vp), ("ring", vp), ("free_stack", vp), ("free_top", vp),
@@ -132,6 +152,8 @@ EXPORTS = {
     "sb_swa_prefill": (C.c_int, [C.POINTER(SwaPrefillArgs)]),
     "sb_window_advance": (C.c_int, [C.POINTER(WindowAdvanceArgs)]),
     "sb_lse_merge": (C.c_int, [C.POINTER(LseMergeArgs)]),
+    "sb_kv_append_int8": (C.c_int, [C.POINTER(KvAppendInt8Args)]),
+    "sb_quantize_sym": (C.c_int, [C.POINTER(QuantizeSymArgs)]),
     "sb_stream_copy": (C.c_int, [vp, vp, i64, vp]),
 }
 

@@ -207,6 +207,65 @@ def swa_decode_attention(
     return (out, lse) if return_lse else out
 
 
+def alloc_int8_kv_cache(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int, device):
+    """(kv int8 [2, num_blocks, block_size, Hkv, D], scales fp32 [2, num_blocks, Hkv, block_size]),
+    zero-filled: the paged K/V cache in its per-row INT8 form."""
+    kv = torch.zeros((2, num_blocks, block_size, num_kv_heads, head_size), dtype=torch.int8, device=device)
+    scales = torch.zeros((2, num_blocks, num_kv_heads, block_size), dtype=torch.float32, device=device)
+    return kv, scales
+
+
+def kv_append_int8(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   k_scale: torch.Tensor, v_scale: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+    """Quantise this step's K/V rows (per row: 128 signed bytes + one fp32 scale) and store them at
+    their slots; slots < 0 are skipped. Caches int8 [nb, bs, Hkv, 128], scales fp32 [nb, Hkv, bs]."""
+    dev = N.require_gpu(key, value, k_cache, v_cache, k_scale, v_scale, slot_mapping)
+    if key.dim() != 3 or value.shape != key.shape or value.dtype != key.dtype:
+        raise ValueError("key and value must be [tokens, num_kv_heads, head_size] of one dtype")
+    T, Hkv, D = key.shape
+    if k_cache.dtype != torch.int8 or v_cache.dtype != torch.int8 or k_cache.dim() != 4 or v_cache.shape != k_cache.shape \
+            or k_cache.stride() != v_cache.stride():
+        raise ValueError("k_cache and v_cache must be int8 [num_blocks, block_size, num_kv_heads, head_size] with equal strides")
+    nb, bs = k_cache.shape[0], k_cache.shape[1]
+    if k_cache.shape[2:] != (Hkv, D) or k_cache.stride(3) != 1:
+        raise ValueError(f"cache rows must be [{Hkv}, {D}] with a contiguous head dimension")
+    for t, name in ((k_scale, "k_scale"), (v_scale, "v_scale")):
+        if t.shape != (nb, Hkv, bs) or t.dtype != torch.float32 or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous float32 [num_blocks, num_kv_heads, block_size] tensor")
+    _inner_contiguous(key, "key")
+    _inner_contiguous(value, "value")
+    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous() or slot_mapping.numel() < T:
+        raise ValueError("slot_mapping must be a contiguous int64 vector with one entry per token")
+    a = N.KvAppendInt8Args(
+        key=N.ptr(key), value=N.ptr(value), k_cache=N.ptr(k_cache), v_cache=N.ptr(v_cache),
+        k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale), slot_mapping=N.ptr(slot_mapping), num_tokens=T,
+        num_kv_heads=Hkv, head_size=D, block_size=bs, dtype=N.dtype_code(key.dtype),
+        key_stride_token=key.stride(0), key_stride_head=key.stride(1),
+        value_stride_token=value.stride(0), value_stride_head=value.stride(1),
+        cache_stride_block=k_cache.stride(0), cache_stride_row=k_cache.stride(1), cache_stride_head=k_cache.stride(2),
+        stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_kv_append_int8(C.byref(a)), "kv_append_int8")
+
+
+def quantize_sym(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """quantize_sym of W8ASpike/window_attention.py:227-237 on x [rows, heads, 128]: every row replaced
+    by its INT8 codes times its scale, rounded to x's dtype. out may be x."""
+    dev = N.require_gpu(x, out)
+    if x.dim() != 3:
+        raise ValueError("x must be [rows, heads, head_size]")
+    _inner_contiguous(x, "x")
+    if out is None:
+        out = torch.empty_like(x)
+    elif out.shape != x.shape or out.dtype != x.dtype:
+        raise ValueError("out must match x in shape and dtype")
+    _inner_contiguous(out, "out")
+    a = N.QuantizeSymArgs(in_=N.ptr(x), out=N.ptr(out), rows=x.shape[0], heads=x.shape[1], head_size=x.shape[2],
+                          dtype=N.dtype_code(x.dtype), in_stride_row=x.stride(0), in_stride_head=x.stride(1),
+                          out_stride_row=out.stride(0), out_stride_head=out.stride(1), stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_quantize_sym(C.byref(a)), "quantize_sym")
+    return out
+
+
 def prefer_balanced_split(host_seq_lens, window_left: int, n_split: int) -> bool:
     """Whether the balanced split is expected to beat the fixed one for rows of these lengths
     (host ints; no device access)."""
