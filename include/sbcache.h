@@ -106,6 +106,8 @@ int sb_kv_append(const sb_kv_append_args *args);
  * num_q_heads/num_kv_heads <= 16; fp32 (and SB_DECODE_FORCE_VALU) runs on the vector ALUs with
  * group sizes {1,2,4,7,8}.
  * ------------------------------------------------------------------------------------ */
+#define SB_KV_NONE 0
+#define SB_KV_INT8 1
 #define SB_DECODE_FORCE_VALU 1 /* bf16/fp16: use the vector-ALU split kernel instead of the matrix-core one */
 /* bf16/fp16, n_split > 1, up to 1024 rows: cut the chunks of ALL rows, laid end to end, into equal runs
  * (about one per CU) instead of cutting every row into n_split runs, so that rows of different
@@ -153,6 +155,13 @@ typedef struct sb_swa_decode_args {
   int64_t new_key_stride_row, new_key_stride_head;
   int64_t new_value_stride_row, new_value_stride_head;
   void *stream;
+  /* Per-row INT8 cache (kv_quant = SB_KV_INT8): k_cache/v_cache hold int8 codes
+   * [num_blocks, block_size, Hkv, 128] (kv strides in bytes), k_scale/v_scale the fp32 scales
+   * [num_blocks, Hkv, block_size] that sb_kv_append_int8 wrote. Paged mode, q/out bf16 or fp16, fixed
+   * split; the append is not fused (new_key etc. must be NULL: quantise and append first). */
+  const float *k_scale;
+  const float *v_scale;
+  int32_t kv_quant;
 } sb_swa_decode_args;
 
 /* Split count the auto rule (n_split = 0) would use for these shapes. */

@@ -18,6 +18,7 @@ SB_BF16, SB_F16, SB_F32 = 0, 1, 2
 SB_ERR_INVALID, SB_ERR_UNSUPPORTED, SB_ERR_WORKSPACE = -1, -2, -3
 SB_DECODE_FORCE_VALU = 1
 SB_DECODE_BALANCED = 2
+SB_KV_NONE, SB_KV_INT8 = 0, 1
 ABI_VERSION = 1
 
 _DTYPES = {torch.bfloat16: SB_BF16, torch.float16: SB_F16, torch.float32: SB_F32}
@@ -53,7 +54,7 @@ class SwaDecodeArgs(C.Structure):
         ("new_key", vp), ("new_value", vp), ("new_slot_mapping", vp),
         ("new_key_stride_row", i64), ("new_key_stride_head", i64),
         ("new_value_stride_row", i64), ("new_value_stride_head", i64),
-        ("stream", vp),
+        ("stream", vp), ("k_scale", vp), ("v_scale", vp), ("kv_quant", i32),
     ]
 
 

@@ -20,6 +20,8 @@
 namespace sb_host {
 void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
                                   hipStream_t st, const sb::DecodeParams &p);
+void launch_swa_decode_split_i8(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, hipStream_t st,
+                                const sb::DecodeParams &p);
 }
 
 namespace {
@@ -549,11 +551,29 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
     case SB_F32: esz = 4; break;
     default: return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: unknown dtype %d", a->dtype);
   }
-  const int64_t es[] = {a->q_stride_row, a->q_stride_head, a->kv_stride_block, a->kv_stride_row,
-                        a->kv_stride_head};
+  const bool int8_kv = a->kv_quant == SB_KV_INT8;
+  if (a->kv_quant != SB_KV_NONE && !int8_kv)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: unknown kv_quant %d", a->kv_quant);
+  const int kv_esz = int8_kv ? 1 : esz;
+  if (int8_kv) {
+    if (a->dtype == SB_F32 || (a->flags & SB_DECODE_FORCE_VALU))
+      return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: the INT8 cache needs bf16 or fp16 queries on the matrix-core path");
+    if (!a->block_table || !a->k_scale || !a->v_scale)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: the INT8 cache needs paged mode and both scale tensors");
+    if (a->new_key || a->new_value || a->new_slot_mapping)
+      return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: no fused append into the INT8 cache (call sb_kv_append_int8 first)");
+    if ((reinterpret_cast<uintptr_t>(a->k_scale) | reinterpret_cast<uintptr_t>(a->v_scale)) & 15u)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: scale tensors not 16-byte aligned");
+  }
+  const int64_t es[] = {a->q_stride_row, a->q_stride_head};
   for (int64_t s : es)
     if ((s * esz) % 16 != 0)
       return fail(SB_ERR_INVALID, "sb_swa_decode: stride %lld elements is not 16-byte aligned",
+                  (long long)s);
+  const int64_t kes[] = {a->kv_stride_block, a->kv_stride_row, a->kv_stride_head};
+  for (int64_t s : kes)
+    if ((s * kv_esz) % 16 != 0)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: cache stride %lld elements is not 16-byte aligned",
                   (long long)s);
   if ((reinterpret_cast<uintptr_t>(a->q) | reinterpret_cast<uintptr_t>(a->k_cache) |
        reinterpret_cast<uintptr_t>(a->v_cache)) & 15u)
@@ -585,8 +605,9 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   p.scale_log2 = a->scale * sb::kLog2e;
   p.q_sr = a->q_stride_row; p.q_sh = a->q_stride_head;
   p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
-  p.kv_sb = a->kv_stride_block * esz; p.kv_sr = a->kv_stride_row * esz; p.kv_sh = a->kv_stride_head * esz;
+  p.kv_sb = a->kv_stride_block * kv_esz; p.kv_sr = a->kv_stride_row * kv_esz; p.kv_sh = a->kv_stride_head * kv_esz;
   p.bt_stride = a->block_table_stride;
+  p.k_scale = a->k_scale; p.v_scale = a->v_scale;
 
   const int G = a->num_q_heads / a->num_kv_heads;
   const dim3 grid((unsigned)a->num_rows, (unsigned)a->num_kv_heads, (unsigned)n_split);
@@ -597,7 +618,7 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   const bool mfma = (a->dtype != SB_F32) && !(a->flags & SB_DECODE_FORCE_VALU);
   if (mfma ? (G > 16) : (G != 1 && G != 2 && G != 4 && G != 7 && G != 8))
     return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: GQA group size %d (built: up to 16 for bf16/fp16; 1, 2, 4, 7, 8 for fp32)", G);
-  if (mfma && (a->kv_stride_row <= 0 || a->kv_stride_row * esz * 16 >= (1LL << 31)))
+  if (mfma && (a->kv_stride_row <= 0 || a->kv_stride_row * kv_esz * 16 >= (1LL << 31)))
     return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: kv row stride %lld does not fit the kernel's 32-bit in-tile offsets",
                 (long long)a->kv_stride_row);
   if (mfma && ((reinterpret_cast<uintptr_t>(a->out) & 15u) || (a->out_stride_row * esz) % 16 ||
@@ -639,10 +660,11 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
       if (arc != SB_OK) return arc;
     }
   }
-  if (mfma && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
+  if (mfma && !int8_kv && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
     p.n_wg = (int)balanced_workgroups(a->num_rows, n_split);
   if (a->phases != 2) {
-    if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
+    if (int8_kv) launch_swa_decode_split_i8(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p);
+    else if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
                                            (a->flags >> 4) & 7, st, p);
     else if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
     else if (a->dtype == SB_F16) rc = launch_for_group<F16>(G, grid, st, p);

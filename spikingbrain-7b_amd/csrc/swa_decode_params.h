@@ -28,6 +28,9 @@ struct DecodeParams {
   const char *new_v;
   const int64_t *slot_mapping;
   int64_t nk_st, nk_sh, nv_st, nv_sh;  // bytes
+  // INT8 cache: per-row scales [num_blocks, Hkv, block_size]
+  const float *k_scale;
+  const float *v_scale;
 };
 
 }  // namespace sb

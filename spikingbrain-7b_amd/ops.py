@@ -94,6 +94,8 @@ def swa_decode_attention(
     force_valu: bool = False,
     balanced: Optional[bool] = None,
     host_seq_lens=None,
+    k_scale: Optional[torch.Tensor] = None,
+    v_scale: Optional[torch.Tensor] = None,
     pipeline_depth: int = 0,
     new_key: Optional[torch.Tensor] = None,
     new_value: Optional[torch.Tensor] = None,
@@ -119,13 +121,26 @@ def swa_decode_attention(
     balanced: cut the chunks of all rows, laid end to end, into equal runs (one per CU) instead of
     cutting each row into n_split runs (bf16/fp16, <= 1024 rows): faster when the rows' lengths differ
     a lot, a little slower when they do not. Default: decided from host_seq_lens (the same numbers
-    as seq_lens, as Python ints) when the caller has them, else off."""
+    as seq_lens, as Python ints) when the caller has them, else off.
+    k_scale, v_scale (fp32 [num_blocks, Hkv, block_size]): the caches are per-row INT8 codes as
+    kv_append_int8 wrote them (paged mode, bf16/fp16 queries, append not fused)."""
     dev = N.require_gpu(q, key_cache, value_cache, seq_lens, block_table, kv_start, row_seq, key_lo, out)
     if q.dim() != 3:
         raise ValueError(f"q must be [rows, num_heads, head_size], got {tuple(q.shape)}")
     R, Hq, D = q.shape
     _inner_contiguous(q, "q")
-    if key_cache.dtype != q.dtype or value_cache.dtype != q.dtype:
+    int8_kv = k_scale is not None or v_scale is not None
+    if int8_kv:
+        N.require_gpu(q, k_scale, v_scale)
+        if k_scale is None or v_scale is None or block_table is None:
+            raise ValueError("the INT8 cache needs k_scale, v_scale and paged mode")
+        if key_cache.dtype != torch.int8 or value_cache.dtype != torch.int8:
+            raise ValueError("with k_scale/v_scale the caches must be int8")
+        if q.dtype not in (torch.bfloat16, torch.float16) or force_valu:
+            raise NotImplementedError("the INT8 cache needs bf16 or fp16 queries on the matrix-core path")
+        if new_key is not None or new_value is not None or new_slot_mapping is not None:
+            raise NotImplementedError("no fused append into the INT8 cache: call kv_append_int8 first")
+    elif key_cache.dtype != q.dtype or value_cache.dtype != q.dtype:
         raise ValueError("q and the caches must share one dtype")
     if block_table is not None:
         if key_cache.dim() != 4 or value_cache.shape != key_cache.shape:
@@ -139,6 +154,10 @@ def swa_decode_attention(
             raise ValueError("block_table must be a 2-D int32 tensor with contiguous rows")
         bt_stride = block_table.stride(0)
         bound = block_table.shape[1] * bs
+        if int8_kv:
+            for t, name in ((k_scale, "k_scale"), (v_scale, "v_scale")):
+                if t.shape != (nb, Hkv, bs) or t.dtype != torch.float32 or not t.is_contiguous():
+                    raise ValueError(f"{name} must be a contiguous float32 [num_blocks, num_kv_heads, block_size] tensor")
     else:
         if kv_strides is None or num_kv_heads is None:
             raise ValueError("dense mode needs kv_strides and num_kv_heads")
@@ -202,7 +221,8 @@ def swa_decode_attention(
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
         kv_stride_block=kv_strides[0], kv_stride_row=kv_strides[1], kv_stride_head=kv_strides[2],
-        block_table_stride=bt_stride, stream=N.stream_ptr(dev), **fused)
+        block_table_stride=bt_stride, stream=N.stream_ptr(dev),
+        k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale), kv_quant=N.SB_KV_INT8 if int8_kv else N.SB_KV_NONE, **fused)
     N.check(L.sb_swa_decode(C.byref(a)), "swa_decode")
     return (out, lse) if return_lse else out
 

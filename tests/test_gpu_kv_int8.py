@@ -50,3 +50,79 @@ def test_quantize_sym_bit_exact(sb, dev, dtype, name):
     assert np.array_equal(y.float().cpu().numpy(), ref)
     sb.ops.quantize_sym(xd, out=xd)              # in place
     assert torch.equal(xd, y)
+
+
+def int8_problem(sb, dev, lens, bs, Hkv, dtype, seed):
+    """Paged INT8 cache holding lens[b] keys per sequence, filled through kv_append_int8; returns the
+    device tensors and the oracle's float view of what attention should see (dequantised rows)."""
+    g = torch.Generator().manual_seed(seed)
+    need = [(n + bs - 1) // bs for n in lens]
+    nb = sum(need) + 3
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(len(lens), max(max(need), 1), dtype=torch.int32)
+    p = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[p:p + n]; p += n
+    T = sum(lens)
+    k = (torch.randn(T, Hkv, D, generator=g) * (0.5 + torch.rand(T, Hkv, 1, generator=g))).to(dtype)
+    v = (torch.randn(T, Hkv, D, generator=g) * (1 + torch.rand(T, Hkv, 1, generator=g))).to(dtype)
+    slots = torch.cat([torch.tensor([int(tables[b, i // bs]) * bs + i % bs for i in range(n)], dtype=torch.int64)
+                       for b, n in enumerate(lens)]) if T else torch.zeros(0, dtype=torch.int64)
+    kv, sc = sb.ops.alloc_int8_kv_cache(nb, bs, Hkv, D, dev)
+    sc.fill_(float("nan"))                      # rows never written must not leak into any result
+    sb.ops.kv_append_int8(k.to(dev), v.to(dev), kv[0], kv[1], sc[0], sc[1], slots.to(dev))
+    name = {torch.bfloat16: "bf16", torch.float16: "f16"}[dtype]
+    views = []
+    for rounding in (name, "f32"):      # as the reference rounds them (to the tensor's dtype) / code * scale exactly
+        kd = Q.quantize_sym(k.float().numpy(), rounding); vd = Q.quantize_sym(v.float().numpy(), rounding)
+        kc = np.zeros((nb, bs, Hkv, D)); vc = np.zeros((nb, bs, Hkv, D))
+        for t, s in enumerate(slots.tolist()):
+            kc[s // bs, s % bs] = kd[t]; vc[s // bs, s % bs] = vd[t]
+        views.append((kc, vc))
+    return kv, sc, tables, views
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Hq,Hkv", [(28, 4), (8, 8), (16, 2)])
+@pytest.mark.parametrize("wl,n_split", [(64, 1), (100, 3), (-1, 2), (0, 1)])
+def test_decode_over_int8_cache_vs_oracle(sb, dev, dtype, Hq, Hkv, wl, n_split):
+    bs = 16
+    lens = [1, 17, 64, 65, 300, 0, 129]
+    kv, sc, tables, views = int8_problem(sb, dev, lens, bs, Hkv, dtype, Hq + wl)
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(len(lens), Hq, D, generator=g).to(dtype)
+    scale = D ** -0.5
+    (ref, ref_lse), (exact, exact_lse) = (A.paged_decode_attention(q.float().numpy(), kc, vc, tables.numpy(), lens, scale,
+                                                                   wl, return_lse=True) for kc, vc in views)
+    out, lse = sb.ops.swa_decode_attention(q.to(dev), kv[0], kv[1], torch.tensor(lens, dtype=torch.int32, device=dev),
+                                           block_table=tables.to(dev), window_left=wl, scale=scale, n_split=n_split,
+                                           k_scale=sc[0], v_scale=sc[1], return_lse=True)
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    live = [b for b, n in enumerate(lens) if n > 0]
+    # 2e-2 max-abs on the fp32 result, plus the half ulp that storing it in the 16-bit type adds
+    # (|o| reaches 5 here: V rows are scaled by 1..2)
+    ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+    assert (np.abs(got[live] - ref[live]) <= 2e-2 + ulp * np.abs(ref[live])).all()
+    # The reference rounds code * scale to the tensor's dtype before attending; the kernel applies the
+    # scales in fp32 to scores and probabilities. Against the unrounded rows it is therefore tighter.
+    assert np.abs(lse.cpu().numpy()[live] - ref_lse[live]).max() <= 1e-2
+    assert np.abs(lse.cpu().numpy()[live] - exact_lse[live]).max() <= 2e-3
+    assert (np.abs(got[live] - exact[live]) <= 2e-2 + ulp * np.abs(exact[live])).all()
+    assert (got[5] == 0).all()
+
+
+def test_int8_cache_argument_errors(sb, dev):
+    kv, sc = sb.ops.alloc_int8_kv_cache(4, 16, 4, D, dev)
+    q = torch.zeros(2, 28, D, dtype=torch.bfloat16, device=dev)
+    sl = torch.ones(2, dtype=torch.int32, device=dev)
+    bt = torch.zeros(2, 2, dtype=torch.int32, device=dev)
+    with pytest.raises(ValueError):
+        sb.ops.swa_decode_attention(q, kv[0], kv[1], sl, block_table=bt, k_scale=sc[0])
+    with pytest.raises(NotImplementedError):
+        sb.ops.swa_decode_attention(q.float(), kv[0], kv[1], sl, block_table=bt, k_scale=sc[0], v_scale=sc[1])
+    with pytest.raises(NotImplementedError):
+        sb.ops.swa_decode_attention(q, kv[0], kv[1], sl, block_table=bt, k_scale=sc[0], v_scale=sc[1],
+                                    new_key=q[:, :4], new_value=q[:, :4], new_slot_mapping=torch.zeros(2, dtype=torch.int64, device=dev))
+    with pytest.raises(ValueError):
+        sb.ops.kv_append_int8(q[:, :4], q[:, :4], kv[0], kv[1], sc[0][:, :2], sc[1], torch.zeros(2, dtype=torch.int64, device=dev))
