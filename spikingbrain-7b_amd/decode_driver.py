@@ -30,7 +30,12 @@ class HybridDecodeCache:
     def __init__(self, batch: int, *, num_layers: int = 28, num_heads: int = 28, num_kv_heads: int = 4,
                  head_size: int = 128, block_size: int = 16, window_left: int = 4096,
                  dtype: torch.dtype = torch.bfloat16, device="cuda:0", num_blocks: Optional[int] = None,
-                 randomize: bool = False, seed: int = 0):
+                 randomize: bool = False, seed: int = 0, kv_quant: Optional[str] = None):
+        """kv_quant="int8": the SWA layers keep their K/V as per-row INT8 codes + fp32 scales
+        (quantize_sym of W8ASpike/window_attention.py:227-237 applied once, at append time)."""
+        if kv_quant not in (None, "int8"):
+            raise ValueError(f"kv_quant {kv_quant!r} (None or 'int8')")
+        self.kv_quant = kv_quant
         self.device = torch.device(device)
         self.batch, self.num_layers = batch, num_layers
         self.H, self.Hkv, self.D, self.bs, self.wl = num_heads, num_kv_heads, head_size, block_size, window_left
@@ -48,7 +53,17 @@ class HybridDecodeCache:
                     if dt != torch.float32 else torch.randn(shape, dtype=dt, device=self.device, generator=g).mul_(std)
             return torch.zeros(shape, dtype=dt, device=self.device)
 
-        self.kv_caches: List[torch.Tensor] = [alloc(shape, dtype, 1.0) for _ in self.swa_layers]
+        if kv_quant == "int8":
+            self.kv_caches, self.kv_scales = [], []
+            for _ in self.swa_layers:
+                codes, scales = ops.alloc_int8_kv_cache(self.num_blocks, block_size, num_kv_heads, head_size, self.device)
+                if randomize:
+                    codes.random_(-127, 128, generator=g)
+                    scales.uniform_(0.005, 0.03, generator=g)
+                self.kv_caches.append(codes)
+                self.kv_scales.append(scales)
+        else:
+            self.kv_caches: List[torch.Tensor] = [alloc(shape, dtype, 1.0) for _ in self.swa_layers]
         # [n_gla_layers, slots, H, D, D] fp32, as vllm_hymeta/model_for_7B/modeling_gla_swa.py:348-356
         self.gla_state = alloc((len(self.gla_layers), batch, num_heads, head_size, head_size), torch.float32, 0.02)
         self.slot_idx = torch.arange(batch, dtype=torch.int32, device=self.device)
@@ -126,14 +141,26 @@ class HybridDecodeCache:
 
     def swa_layer(self, layer_idx: int, q, k, v, meta: MetaAttentionMetadata, out) -> torch.Tensor:
         """q [B, Hq, D], k/v [B, Hkv, D]: append + window attention for one SWA layer."""
+        if self.kv_quant == "int8":
+            codes, scales = self.kv_caches[layer_idx // 2], self.kv_scales[layer_idx // 2]
+            n = q.shape[0]
+            ops.kv_append_int8(k, v, codes[0], codes[1], scales[0], scales[1], meta.slot_mapping.flatten()[:n])
+            return ops.swa_decode_attention(
+                q, codes[0], codes[1], meta.seq_lens_tensor[:n], block_table=meta.block_tables, window_left=self.wl,
+                scale=self.D ** -0.5, out=out, max_seq_len=meta.max_decode_seq_len or None,
+                k_scale=scales[0], v_scale=scales[1])
         return self.impl.forward(self._layer, q, k, v, None, None, None, self.kv_caches[layer_idx // 2], meta, out)
 
     def bytes_per_step(self) -> int:
         """Algorithmic HBM bytes of one decode step over all layers (window-saturated sequences)."""
-        e = self.kv_caches[0].element_size()
+        e = self._gla_out.element_size()
         n_keys = np.minimum(self.manager.n_tokens[:self.batch], self.wl + 1)
-        swa = int(n_keys.sum()) * self.Hkv * self.D * 2 * e + self.batch * (2 * self.H * self.D * e
-                                                                           + 4 * self.Hkv * self.D * e)
+        if self.kv_quant == "int8":     # per key and kv head: 2 x 128 code bytes + 2 fp32 scales; new row read in e, written as codes
+            swa = int(n_keys.sum()) * self.Hkv * (2 * self.D + 8) + self.batch * (
+                2 * self.H * self.D * e + 2 * self.Hkv * self.D * e + self.Hkv * (2 * self.D + 8))
+        else:
+            swa = int(n_keys.sum()) * self.Hkv * self.D * 2 * e + self.batch * (2 * self.H * self.D * e
+                                                                               + 4 * self.Hkv * self.D * e)
         gla = self.batch * self.H * (2 * self.D * self.D * 4 + 3 * self.D * e + self.D * 4 + self.D * e)
         return len(self.swa_layers) * swa + len(self.gla_layers) * gla
 

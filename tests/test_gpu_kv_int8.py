@@ -126,3 +126,36 @@ def test_int8_cache_argument_errors(sb, dev):
                                     new_key=q[:, :4], new_value=q[:, :4], new_slot_mapping=torch.zeros(2, dtype=torch.int64, device=dev))
     with pytest.raises(ValueError):
         sb.ops.kv_append_int8(q[:, :4], q[:, :4], kv[0], kv[1], sc[0][:, :2], sc[1], torch.zeros(2, dtype=torch.int64, device=dev))
+
+
+def test_hybrid_decode_driver_with_int8_kv(sb, dev):
+    """The decode driver with kv_quant="int8": every step appends quantised rows and attends over the
+    INT8 cache; host-stepped and device-advanced runs leave identical caches and outputs, and the
+    outputs match the oracle's attention over the dequantised history of one sequence."""
+    B, wl, bs = 3, 40, 16
+    runs = []
+    for device_advance in (False, True):
+        c = sb.HybridDecodeCache(B, num_layers=2, window_left=wl, block_size=bs, device=dev, kv_quant="int8")
+        c.start(0)
+        g = torch.Generator().manual_seed(9)
+        hist_k, hist_v, outs = [], [], []
+        meta = c.enable_device_advance() if device_advance else None
+        for step in range(3 * bs):
+            q = torch.randn(B, 28, D, generator=g).bfloat16()
+            k = torch.randn(B, 4, D, generator=g).bfloat16()
+            v = torch.randn(B, 4, D, generator=g).bfloat16()
+            if device_advance:
+                c.advance_device()
+            else:
+                meta = c.step_metadata()
+            out = torch.empty(B, 28, D, dtype=torch.bfloat16, device=dev)
+            c.swa_layer(1, q.to(dev), k.to(dev), v.to(dev), meta, out)
+            hist_k.append(k[0]); hist_v.append(v[0]); outs.append(out.cpu())
+            if step in (0, wl + 3, 3 * bs - 1):
+                kd = Q.quantize_sym(torch.stack(hist_k).float().numpy(), "bf16")
+                vd = Q.quantize_sym(torch.stack(hist_v).float().numpy(), "bf16")
+                ref = A.varlen_window_attention(q[0:1].float().numpy(), kd, vd, [0, 1], [0, len(kd)], D ** -0.5, wl)
+                assert np.abs(out[0:1].float().cpu().numpy() - ref).max() <= 2e-2, step
+        runs.append((torch.stack(outs), c.kv_caches[0].cpu(), c.kv_scales[0].cpu()))
+    assert torch.equal(runs[0][0], runs[1][0])
+    assert torch.equal(runs[0][1], runs[1][1]) and torch.equal(runs[0][2], runs[1][2])
