@@ -197,11 +197,11 @@ def bench_gla_prompt(sb, dev, S=16, L=8192, H=28, iters=3):
             "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 2), "frac_fp32_vector_peak_unpacked": round(flop / (ms * 1e-3) / 1e12 / 78.6, 4)}
 
 
-def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None):
+def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None, gla_state_dtype=torch.float32):
     """BASELINE config 5: the cache work of 128 consecutive decode steps of the 28-layer stack
     (14 GLA state layers + 14 paged SWA layers, one shared block table), B=256, every sequence at a
     logical context of 512k tokens (window-saturated), real appends, eviction and block recycling."""
-    c = sb.HybridDecodeCache(B, randomize=True, device=dev, kv_quant=kv_quant)
+    c = sb.HybridDecodeCache(B, randomize=True, device=dev, kv_quant=kv_quant, gla_state_dtype=gla_state_dtype)
     c.start(512 * 1024)
     g = torch.Generator(device=dev).manual_seed(1)
     q = torch.randn(B, HQ, D, device=dev, dtype=torch.bfloat16, generator=g)
@@ -243,7 +243,8 @@ def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None):
     by = c.bytes_per_step()
     gpu_ms = statistics.median(gpu)
     res = {"workload": f"BASELINE config 5: 28-layer hybrid decode step, B={B}, logical context 512k, "
-                       f"{steps} consecutive steps" + (", SWA K/V as per-row INT8" if kv_quant else ""),
+                       f"{steps} consecutive steps" + (", SWA K/V as per-row INT8" if kv_quant else "")
+                       + (", GLA state stored as bf16" if gla_state_dtype == torch.bfloat16 else ""),
            "bytes_per_step": by,
            "host_stepped": {"ms_per_step": round(ms, 3), "decode_tok_per_s": round(B / (ms * 1e-3)),
                             "GBps": round(by / (ms * 1e-3) / 1e9, 1),
@@ -282,7 +283,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
                                                     "28-layer hybrid decode step (config 5)")
-    ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "gla_prompt"), default=None,
+    ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "hybrid_lean", "gla_prompt"), default=None,
                     help="run just that section and print its JSON (short runs for profiling one kernel)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -304,6 +305,10 @@ def main():
         return
     if args.only == "hybrid":
         print(json.dumps({"hybrid_decode": bench_hybrid(sb, dev, steps=min(args.steps, 128))}))
+        return
+    if args.only == "hybrid_lean":
+        print(json.dumps({"hybrid_decode_int8_kv_bf16_state": bench_hybrid(
+            sb, dev, steps=min(args.steps, 128), kv_quant="int8", gla_state_dtype=torch.bfloat16)}))
         return
     if args.only == "hybrid_int8":
         print(json.dumps({"hybrid_decode_int8_kv": bench_hybrid(sb, dev, steps=min(args.steps, 128), kv_quant="int8")}))
@@ -418,6 +423,9 @@ def main():
         line["hybrid_decode"] = bench_hybrid(sb, dev)
         torch.cuda.empty_cache()
         line["hybrid_decode_int8_kv"] = bench_hybrid(sb, dev, kv_quant="int8")
+        torch.cuda.empty_cache()
+        # the storage formats of the reference's own variants: bf16 state cache (its serving path), INT8 K/V (W8ASpike)
+        line["hybrid_decode_int8_kv_bf16_state"] = bench_hybrid(sb, dev, kv_quant="int8", gla_state_dtype=torch.bfloat16)
         torch.cuda.empty_cache()
 
     if not args.no_cpu_baseline:

@@ -30,9 +30,14 @@ class HybridDecodeCache:
     def __init__(self, batch: int, *, num_layers: int = 28, num_heads: int = 28, num_kv_heads: int = 4,
                  head_size: int = 128, block_size: int = 16, window_left: int = 4096,
                  dtype: torch.dtype = torch.bfloat16, device="cuda:0", num_blocks: Optional[int] = None,
-                 randomize: bool = False, seed: int = 0, kv_quant: Optional[str] = None):
+                 randomize: bool = False, seed: int = 0, kv_quant: Optional[str] = None,
+                 gla_state_dtype: torch.dtype = torch.float32):
         """kv_quant="int8": the SWA layers keep their K/V as per-row INT8 codes + fp32 scales
-        (quantize_sym of W8ASpike/window_attention.py:227-237 applied once, at append time)."""
+        (quantize_sym of W8ASpike/window_attention.py:227-237 applied once, at append time).
+        gla_state_dtype: float32, or bfloat16 as the reference's serving path keeps its state cache
+        (vllm_hymeta/model_for_7B/modeling_gla_swa.py:361-364); the arithmetic is fp32 either way."""
+        if gla_state_dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError("gla_state_dtype must be float32 or bfloat16")
         if kv_quant not in (None, "int8"):
             raise ValueError(f"kv_quant {kv_quant!r} (None or 'int8')")
         self.kv_quant = kv_quant
@@ -65,7 +70,7 @@ class HybridDecodeCache:
         else:
             self.kv_caches: List[torch.Tensor] = [alloc(shape, dtype, 1.0) for _ in self.swa_layers]
         # [n_gla_layers, slots, H, D, D] fp32, as vllm_hymeta/model_for_7B/modeling_gla_swa.py:348-356
-        self.gla_state = alloc((len(self.gla_layers), batch, num_heads, head_size, head_size), torch.float32, 0.02)
+        self.gla_state = alloc((len(self.gla_layers), batch, num_heads, head_size, head_size), gla_state_dtype, 0.02)
         self.slot_idx = torch.arange(batch, dtype=torch.int32, device=self.device)
         self.impl = MetaAttentionImpl(num_heads, head_size, head_size ** -0.5, num_kv_heads, None, window_left + 1,
                                       "auto")
@@ -161,7 +166,8 @@ class HybridDecodeCache:
         else:
             swa = int(n_keys.sum()) * self.Hkv * self.D * 2 * e + self.batch * (2 * self.H * self.D * e
                                                                                + 4 * self.Hkv * self.D * e)
-        gla = self.batch * self.H * (2 * self.D * self.D * 4 + 3 * self.D * e + self.D * 4 + self.D * e)
+        gla = self.batch * self.H * (2 * self.D * self.D * self.gla_state.element_size() + 3 * self.D * e + self.D * 4
+                                     + self.D * e)
         return len(self.swa_layers) * swa + len(self.gla_layers) * gla
 
 
