@@ -18,14 +18,14 @@ from .decode_driver import HybridDecodeCache  # noqa: F401
 from .gla import (GLACacheManager, GLACacheParams, fused_chunk_gla, fused_recurrent_gla,  # noqa: F401
                   gla_prefill_packed, my_fused_recurrent_gla)
 from .hf_cache import Cache  # noqa: F401
-from .meta_attention import (AttentionType, MetaAttentionBackend, MetaAttentionImpl,  # noqa: F401
+from .meta_attention import (AttentionType, Int8KVCache, MetaAttentionBackend, MetaAttentionImpl,  # noqa: F401
                              MetaAttentionMetadata, MetaAttentionMetadataBuilder)
 from .runner import SwaCacheRunner  # noqa: F401
 from .window_attention import sliding_window_attention  # noqa: F401
 
 __all__ = [
     "Cache", "sliding_window_attention", "MetaAttentionBackend", "MetaAttentionImpl", "MetaAttentionMetadata",
-    "MetaAttentionMetadataBuilder", "AttentionType", "GLACacheManager", "GLACacheParams",
+    "MetaAttentionMetadataBuilder", "AttentionType", "Int8KVCache", "GLACacheManager", "GLACacheParams",
     "my_fused_recurrent_gla", "fused_recurrent_gla", "fused_chunk_gla", "gla_prefill_packed", "WindowBlockManager", "PAD_SLOT_ID",
     "compute_slot_mapping", "compute_slot_mapping_start_idx", "ops", "SwaCacheRunner", "HybridDecodeCache",
 ]

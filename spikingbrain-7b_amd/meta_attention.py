@@ -82,17 +82,50 @@ class MetaAttentionBackend:
         scr_to_dst is [n, 2] (source block, destination block). Block-granular async copies on
         the current stream, K half then V half (meta_attention.py:94-112)."""
         pairs = scr_to_dst.tolist()
-        for half in (0, 1):
-            src, dst = src_kv_cache[half], dst_kv_cache[half]
-            for s, d in pairs:
-                dst[d].copy_(src[s], non_blocking=True)
+        if isinstance(src_kv_cache, Int8KVCache):
+            tensors = ((src_kv_cache.codes, dst_kv_cache.codes), (src_kv_cache.scales, dst_kv_cache.scales))
+        else:
+            tensors = ((src_kv_cache, dst_kv_cache),)
+        for src_t, dst_t in tensors:
+            for half in (0, 1):
+                src, dst = src_t[half], dst_t[half]
+                for s, d in pairs:
+                    dst[d].copy_(src[s], non_blocking=True)
 
     @staticmethod
     def copy_blocks(kv_caches: List[torch.Tensor], src_to_dists: torch.Tensor) -> None:
         """Copy-on-write block copies inside every layer's cache (meta_attention.py:114-126)."""
         for kv_cache in kv_caches:
-            ops.copy_blocks(kv_cache[0], src_to_dists)
-            ops.copy_blocks(kv_cache[1], src_to_dists)
+            halves = (kv_cache.codes, kv_cache.scales) if isinstance(kv_cache, Int8KVCache) else (kv_cache,)
+            for t in halves:
+                ops.copy_blocks(t[0], src_to_dists)
+                ops.copy_blocks(t[1], src_to_dists)
+
+
+class Int8KVCache:
+    """One layer's paged K/V in per-row INT8 form: `codes` int8 [2, num_blocks, block_size, Hkv, D] and
+    `scales` fp32 [2, num_blocks, Hkv, block_size] (quantize_sym of W8ASpike/window_attention.py:227-237
+    applied once per row, at append time). Pass it where the bf16 `kv_cache` tensor goes."""
+
+    def __init__(self, codes: torch.Tensor, scales: torch.Tensor):
+        if codes.dtype != torch.int8 or codes.dim() != 5 or codes.shape[0] != 2:
+            raise ValueError("codes must be int8 [2, num_blocks, block_size, num_kv_heads, head_size]")
+        _, nb, bs, hkv, _ = codes.shape
+        if scales.dtype != torch.float32 or tuple(scales.shape) != (2, nb, hkv, bs):
+            raise ValueError("scales must be float32 [2, num_blocks, num_kv_heads, block_size]")
+        self.codes, self.scales = codes, scales
+
+    @classmethod
+    def allocate(cls, num_blocks: int, block_size: int, num_kv_heads: int, head_size: int, device) -> "Int8KVCache":
+        MetaAttentionBackend.get_kv_cache_shape(num_blocks, block_size, num_kv_heads, head_size)   # validates
+        return cls(*ops.alloc_int8_kv_cache(num_blocks, block_size, num_kv_heads, head_size, device))
+
+    def numel(self) -> int:
+        return self.codes.numel()
+
+    @property
+    def device(self):
+        return self.codes.device
 
 
 @dataclass
@@ -448,14 +481,20 @@ class MetaAttentionImpl:
         # A pure decode step (one new token per sequence, the hot loop) appends and attends in ONE
         # launch: the attention kernel takes the newest K/V row from `key`/`value` and stores it at
         # its slot. Every other step appends first, exactly as the reference does (:790-799).
-        fuse_append = (kv_cache.numel() > 0 and key is not None and value is not None
+        int8_kv = isinstance(kv_cache, Int8KVCache)
+        scales = dict(k_scale=kv_cache.scales[0], v_scale=kv_cache.scales[1]) if int8_kv else {}
+        fuse_append = (kv_cache.numel() > 0 and key is not None and value is not None and not int8_kv
                        and attn_metadata.num_prefill_tokens == 0 and attn_metadata.num_decode_tokens > 0
                        and (attn_metadata.max_decode_query_len or 1) == 1
                        and query.dtype in (torch.bfloat16, torch.float16)
                        and attn_metadata.slot_mapping is not None)
         if kv_cache.numel() > 0:
-            key_cache, value_cache = kv_cache[0], kv_cache[1]
-            if key is not None and value is not None and not fuse_append:
+            key_cache, value_cache = (kv_cache.codes[0], kv_cache.codes[1]) if int8_kv else (kv_cache[0], kv_cache[1])
+            if key is not None and value is not None and int8_kv:
+                # rows are quantised on their way in: 128 code bytes + one scale per (token, kv head)
+                ops.kv_append_int8(key, value, key_cache, value_cache, scales["k_scale"], scales["v_scale"],
+                                   attn_metadata.slot_mapping.flatten())
+            elif key is not None and value is not None and not fuse_append:
                 # all new K/V of the step (prefill and decode tokens) go in with one launch (:790-799)
                 ops.kv_append(key, value, key_cache, value_cache, attn_metadata.slot_mapping.flatten())
 
@@ -485,8 +524,11 @@ class MetaAttentionImpl:
         if prefill_meta := attn_metadata.prefill_metadata:
             if kv_cache.numel() == 0 or prefill_meta.block_tables is None or prefill_meta.block_tables.numel() == 0:
                 # plain prompt run: keys and values are the in-flight tensors (:835-884)
-                lse = self._varlen_inflight(query, key[:num_prefill_query_tokens], value[:num_prefill_query_tokens],
-                                            prefill_meta, prefill_output, window_left, return_lse=with_meta)
+                pk, pv = key[:num_prefill_query_tokens], value[:num_prefill_query_tokens]
+                if int8_kv:   # attend to what the cache will hold: the rows as quantize_sym returns them
+                    pk, pv = ops.quantize_sym(pk), ops.quantize_sym(pv)
+                lse = self._varlen_inflight(query, pk, pv, prefill_meta, prefill_output, window_left,
+                                            return_lse=with_meta)
             else:
                 # prefix hit / chunked prefill: keys and values come from the paged cache (:885-919)
                 assert prefill_meta.seq_lens is not None
@@ -494,7 +536,7 @@ class MetaAttentionImpl:
                 lse = self._varlen_paged(query, key_cache, value_cache, prefill_meta.query_start_loc,
                                          prefill_meta.seq_lens_tensor, prefill_meta.block_tables,
                                          max(prefill_meta.seq_lens), prefill_output, window_left,
-                                         meta=prefill_meta, return_lse=with_meta)
+                                         meta=prefill_meta, return_lse=with_meta, scales=scales)
             merge_meta(query, prefill_output, lse)
         if decode_meta := attn_metadata.decode_metadata:
             assert decode_meta.max_decode_query_len is not None
@@ -504,7 +546,7 @@ class MetaAttentionImpl:
                 lse = self._varlen_paged(decode_query, key_cache, value_cache, decode_meta.query_start_loc,
                                          decode_meta.seq_lens_tensor, decode_meta.block_tables,
                                          decode_meta.max_decode_seq_len, decode_output, window_left,
-                                         meta=decode_meta, return_lse=with_meta)
+                                         meta=decode_meta, return_lse=with_meta, scales=scales)
             else:
                 # one query token per sequence (:954-981); K/V were appended above, or are appended
                 # by this very launch when the step is a pure decode step
@@ -523,7 +565,8 @@ class MetaAttentionImpl:
                     decode_query, key_cache, value_cache, decode_meta.seq_lens_tensor[:n],
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
                     out=decode_output, return_lse=with_meta,
-                    max_seq_len=decode_meta.max_decode_seq_len or None, balanced=decode_meta._decode_balanced, **fused)
+                    max_seq_len=decode_meta.max_decode_seq_len or None,
+                    balanced=False if int8_kv else decode_meta._decode_balanced, **scales, **fused)
                 lse = res[1] if with_meta else None
             merge_meta(decode_query, decode_output, lse)
         return output
@@ -574,11 +617,14 @@ class MetaAttentionImpl:
         return res[1] if return_lse else None
 
     def _varlen_paged(self, q, key_cache, value_cache, query_start_loc, seq_lens_tensor, block_tables,
-                      max_seq_len, out, window_left, meta=None, return_lse=False):
+                      max_seq_len, out, window_left, meta=None, return_lse=False, scales=None):
+        """scales (k_scale, v_scale of an INT8 cache): every query token runs as one row of the
+        single-query kernel, the only one that reads that cache form."""
         T = q.shape[0]
         if T == 0:
             return None
-        plan = self._plan_for(meta, q) if meta is not None else None
+        scales = scales or {}
+        plan = self._plan_for(meta, q) if meta is not None and not scales else None
         if plan is not None and block_tables.shape[1] * key_cache.shape[1] >= plan.max_k:
             res = ops.swa_prefill_attention(q, key_cache, value_cache, plan=plan, block_table=block_tables,
                                             window_left=window_left, scale=self.scale, out=out, return_lse=return_lse)
@@ -589,5 +635,5 @@ class MetaAttentionImpl:
         res = ops.swa_decode_attention(
             q, key_cache, value_cache, seq_lens_row, block_table=block_tables, row_seq=row_seq.to(torch.int32),
             window_left=window_left, scale=self.scale, out=out, max_seq_len=max_seq_len or None,
-            return_lse=return_lse)
+            return_lse=return_lse, **scales)
         return res[1] if return_lse else None

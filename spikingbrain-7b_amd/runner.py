@@ -13,7 +13,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 from .block_manager import LogicalTable, WindowBlockManager
-from .meta_attention import MetaAttentionBackend, MetaAttentionMetadata, MetaAttentionMetadataBuilder
+from .meta_attention import Int8KVCache, MetaAttentionBackend, MetaAttentionMetadata, MetaAttentionMetadataBuilder
 
 
 @dataclass
@@ -71,12 +71,20 @@ class SwaCacheRunner:
     """Owns the block manager and the per-layer paged KV tensors; builds step metadata."""
 
     def __init__(self, num_layers: int, num_blocks: int, block_size: int, window_left: int, num_kv_heads: int,
-                 head_size: int, dtype: torch.dtype, device, max_seqs: int, max_chunk_tokens: int = 0):
+                 head_size: int, dtype: torch.dtype, device, max_seqs: int, max_chunk_tokens: int = 0,
+                 kv_quant: Optional[str] = None):
+        """kv_quant="int8": every layer's cache is an Int8KVCache (codes + per-row scales) instead of a `dtype` tensor."""
         self.device = torch.device(device)
         self.block_size, self.window_left = block_size, window_left
         self.manager = WindowBlockManager(num_blocks, block_size, window_left, max_seqs, max_chunk_tokens)
         shape = MetaAttentionBackend.get_kv_cache_shape(num_blocks, block_size, num_kv_heads, head_size)
-        self.kv_caches = [torch.zeros(shape, dtype=dtype, device=self.device) for _ in range(num_layers)]
+        if kv_quant == "int8":
+            self.kv_caches = [Int8KVCache.allocate(num_blocks, block_size, num_kv_heads, head_size, self.device)
+                              for _ in range(num_layers)]
+        elif kv_quant is None:
+            self.kv_caches = [torch.zeros(shape, dtype=dtype, device=self.device) for _ in range(num_layers)]
+        else:
+            raise ValueError(f"kv_quant {kv_quant!r} (None or 'int8')")
 
     def add_seq(self, seq_id) -> None:
         self.manager.add_seq(seq_id)

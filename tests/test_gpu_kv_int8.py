@@ -159,3 +159,64 @@ def test_hybrid_decode_driver_with_int8_kv(sb, dev):
         runs.append((torch.stack(outs), c.kv_caches[0].cpu(), c.kv_scales[0].cpu()))
     assert torch.equal(runs[0][0], runs[1][0])
     assert torch.equal(runs[0][1], runs[1][1]) and torch.equal(runs[0][2], runs[1][2])
+
+
+def test_backend_engine_with_int8_cache(sb, dev):
+    """Prompt step, chunked second prompt + decodes, decode steps with eviction, through
+    MetaAttentionImpl.forward on Int8KVCache layers: codes and scales bit-exact against the oracle's
+    quantised append at the oracle's slots; outputs within 2e-2 of attention over the rows as
+    quantize_sym returns them (what the W8ASpike layer attends to)."""
+    from oracle import paged as P
+    HQ, HKV, bs, wl, nb = 28, 4, 16, 40, 48
+    runner = sb.runner.SwaCacheRunner(1, nb, bs, wl, HKV, D, torch.bfloat16, dev, max_seqs=3, max_chunk_tokens=128,
+                                      kv_quant="int8")
+    impl = sb.MetaAttentionImpl(HQ, D, D ** -0.5, HKV, None, wl + 1, "auto")
+    model = P.WindowCacheModel(nb, bs, wl)
+    kc = np.zeros((nb, bs, HKV, D), np.int8); vc = np.zeros_like(kc)
+    ks = np.zeros((nb, HKV, bs), np.float32); vs = np.zeros_like(ks)
+    hist = {}
+    g = torch.Generator().manual_seed(11)
+
+    def step(prompts, decodes, chunked=False):
+        T = sum(n for _, n in prompts) + len(decodes)
+        q = torch.randn(T, HQ, D, generator=g).bfloat16()
+        k = torch.randn(T, HKV, D, generator=g).bfloat16()
+        v = torch.randn(T, HKV, D, generator=g).bfloat16()
+        meta = runner.build_step(prompts, decodes, chunked_prefill=chunked)
+        slots = []
+        for sid, n in prompts:
+            slots += model.append_tokens(sid, n, True, store_all=chunked)
+        for sid in decodes:
+            slots += model.append_tokens(sid, 1, False)
+        assert meta.slot_mapping.cpu().tolist() == slots
+        Q.kv_append_int8(k.float().numpy(), v.float().numpy(), kc, vc, ks, vs, slots)
+        out = torch.full((T, HQ, D), float("nan"), dtype=torch.bfloat16, device=dev)
+        impl.forward(None, q.to(dev), k.to(dev), v.to(dev), None, None, None, runner.kv_caches[0], meta, output=out)
+        cache = runner.kv_caches[0]
+        assert np.array_equal(cache.codes[0].cpu().numpy(), kc) and np.array_equal(cache.codes[1].cpu().numpy(), vc)
+        written = ks != 0
+        assert np.array_equal(cache.scales[0].cpu().numpy()[written], ks[written])
+        assert np.array_equal(cache.scales[1].cpu().numpy()[written], vs[written])
+        got = out.float().cpu().numpy()
+        t = 0
+        for sid, n in list(prompts) + [(s, 1) for s in decodes]:
+            hk, hv = hist.get(sid, (np.zeros((0, HKV, D), np.float32), np.zeros((0, HKV, D), np.float32)))
+            hk = np.concatenate([hk, Q.quantize_sym(k[t:t + n].float().numpy(), "bf16")])
+            hv = np.concatenate([hv, Q.quantize_sym(v[t:t + n].float().numpy(), "bf16")])
+            hist[sid] = (hk, hv)
+            ref = A.varlen_window_attention(q[t:t + n].float().numpy(), hk, hv, [0, n], [0, len(hk)], D ** -0.5, wl)
+            assert np.abs(got[t:t + n] - ref).max() <= 2e-2 + 2.0 ** -8 * np.abs(ref).max(), (sid, n)
+            t += n
+
+    for sid in (0, 1, 2):
+        runner.add_seq(sid); model.add_seq(sid)
+    step([(0, 25), (1, 90)], [])                       # plain prompts: attention over the quantised in-flight rows
+    step([(2, 50)], [0, 1], chunked=True)              # chunked prompt reads the INT8 paged cache + two decodes
+    for _ in range(bs + 3):
+        step([], [0, 1, 2])
+    # copy-on-write block copy moves codes and scales together
+    src = int(runner.kv_caches[0].scales[0].abs().sum((1, 2)).argmax())
+    dst = model.free[-1] if hasattr(model, "free") and model.free else (src + 1) % nb
+    before = runner.kv_caches[0].codes[:, src].clone(), runner.kv_caches[0].scales[:, src].clone()
+    sb.MetaAttentionBackend.copy_blocks(runner.kv_caches, torch.tensor([[src, dst]], dtype=torch.int64, device=dev))
+    assert torch.equal(runner.kv_caches[0].codes[:, dst], before[0]) and torch.equal(runner.kv_caches[0].scales[:, dst], before[1])
