@@ -195,6 +195,8 @@ int sb_swa_decode(const sb_swa_decode_args *args);
  *   state  [num_slots, H, 128, 128] dtype `state_dtype` (SB_F32 or SB_BF16)
  *   out    [B, H, T, 128] dtype `dtype`
  * ------------------------------------------------------------------------------------ */
+#define SB_GLA_VECTOR_ONLY 1
+
 typedef struct sb_gla_recurrent_args {
   const void *q, *k, *v, *g;
   void *state;
@@ -218,6 +220,11 @@ typedef struct sb_gla_recurrent_args {
    * q/k/v/g/out laid out [total_tokens, H, 128]; the *_stride_b fields are ignored, the *_stride_t
    * fields are the token strides, and seq_len is only an upper bound of the row lengths. */
   const int32_t *cu_seqlens;
+  /* SB_GLA_* bits. Calls of 32 steps or more, and every packed call, with bf16 q/k/v run the
+   * recurrence 16 tokens at a time on the matrix cores (its exact block form; fp32 state, gate
+   * scan and accumulation; bf16 operand rounding on the output path as in any bf16 GEMM).
+   * SB_GLA_VECTOR_ONLY keeps such calls on the step-by-step fp32 kernel. */
+  int32_t flags;
 } sb_gla_recurrent_args;
 
 int sb_gla_recurrent(const sb_gla_recurrent_args *args);

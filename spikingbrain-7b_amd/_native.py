@@ -19,6 +19,7 @@ SB_ERR_INVALID, SB_ERR_UNSUPPORTED, SB_ERR_WORKSPACE = -1, -2, -3
 SB_DECODE_FORCE_VALU = 1
 SB_DECODE_BALANCED = 2
 SB_KV_NONE, SB_KV_INT8 = 0, 1
+SB_GLA_VECTOR_ONLY = 1
 ABI_VERSION = 1
 
 _DTYPES = {torch.bfloat16: SB_BF16, torch.float16: SB_F16, torch.float32: SB_F32}
@@ -69,7 +70,7 @@ class GlaRecurrentArgs(C.Structure):
         ("g_stride_b", i64), ("g_stride_h", i64), ("g_stride_t", i64),
         ("out_stride_b", i64), ("out_stride_h", i64), ("out_stride_t", i64),
         ("state_stride_slot", i64), ("state_stride_head", i64),
-        ("num_slots", i64), ("stream", vp), ("cu_seqlens", vp),
+        ("num_slots", i64), ("stream", vp), ("cu_seqlens", vp), ("flags", i32),
     ]
 
 

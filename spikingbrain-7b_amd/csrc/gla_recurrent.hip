@@ -303,6 +303,13 @@ void launch_sequence(const GlaParams &p, dim3 grid, hipStream_t st) {
 
 }  // namespace
 
+namespace sb_host {
+void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups);
+}
+
+// Calls of this many steps or more (and every packed call) with bf16 q, k, v run on the matrix cores.
+constexpr int kChunkKernelMinSteps = 32;
+
 extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
   using namespace sb_host;
   if (!a) return fail(SB_ERR_INVALID, "sb_gla_recurrent: null args");
@@ -349,6 +356,11 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
                           quad_aligned(a->v, a->dtype, p.v_sb, p.v_sh, p.v_st) &&
                           quad_aligned(a->g, a->g_dtype, p.g_sb, p.g_sh, p.g_st) &&
                           quad_aligned(a->out, a->dtype, p.o_sb, p.o_sh, p.o_st);
+  if (a->dtype == SB_BF16 && !(a->flags & SB_GLA_VECTOR_ONLY) &&
+      (a->cu_seqlens || a->seq_len >= kChunkKernelMinSteps)) {
+    launch_gla_chunk(a, groups);
+    return check_launch("gla_chunk_kernel");
+  }
   if (a->cu_seqlens && !vectors_ok)
     return fail(SB_ERR_UNSUPPORTED,
                 "sb_gla_recurrent: the packed form needs pointers and strides of q, k, v, g, out aligned to 4 elements");

@@ -488,10 +488,13 @@ def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, sc
 
 def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
                   slot_idx: Optional[torch.Tensor] = None, scale: Optional[float] = None,
-                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  out: Optional[torch.Tensor] = None, vector_only: bool = False) -> torch.Tensor:
     """q, k, v, g [B, H, T, D] (any batch/head/time strides, contiguous D); state
     [slots, H, D, D] fp32 or bf16, updated in place; returns o [B, H, T, D] in q's dtype.
-    Rows with slot_idx == -1 are skipped (state and output untouched)."""
+    Rows with slot_idx == -1 are skipped (state and output untouched).
+    Calls of 32 steps or more with bf16 q/k/v run 16 tokens at a time on the matrix cores (state, gates
+    and accumulation in fp32, bf16 operand rounding on the output path); vector_only=True keeps them on
+    the step-by-step fp32 kernel."""
     dev = N.require_gpu(q, k, v, g, state, slot_idx, out)
     if q.dim() != 4 or k.shape != q.shape or v.shape != q.shape or g.shape != q.shape:
         raise ValueError(f"q, k, v, g must all be [B, H, T, D]; got {tuple(q.shape)}, {tuple(k.shape)}, "
@@ -529,7 +532,7 @@ def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
         g_stride_b=g.stride(0), g_stride_h=g.stride(1), g_stride_t=g.stride(2),
         out_stride_b=out.stride(0), out_stride_h=out.stride(1), out_stride_t=out.stride(2),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
-        num_slots=state.shape[0], stream=N.stream_ptr(dev))
+        num_slots=state.shape[0], stream=N.stream_ptr(dev), flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0)
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
 
@@ -537,7 +540,7 @@ def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
 def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
                          cu_seqlens: torch.Tensor, slot_idx: Optional[torch.Tensor] = None,
                          scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
-                         max_seq_len: Optional[int] = None) -> torch.Tensor:
+                         max_seq_len: Optional[int] = None, vector_only: bool = False) -> torch.Tensor:
     """The same recurrence over packed prompts: q, k, v, g [total_tokens, H, D] (token/head strides
     free, contiguous D), sequence b owning tokens cu_seqlens[b] .. cu_seqlens[b+1]-1 (int32 device
     vector [B+1]); its state is state[slot_idx[b]] (default b), advanced in place. One launch for
@@ -579,7 +582,8 @@ def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: t
         g_stride_b=0, g_stride_h=g.stride(1), g_stride_t=g.stride(0),
         out_stride_b=0, out_stride_h=out.stride(1), out_stride_t=out.stride(0),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
-        num_slots=state.shape[0], stream=N.stream_ptr(dev), cu_seqlens=N.ptr(cu_seqlens))
+        num_slots=state.shape[0], stream=N.stream_ptr(dev), cu_seqlens=N.ptr(cu_seqlens),
+        flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0)
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
 
