@@ -216,26 +216,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       vb[nt] = make_uint4(x.x, x.y, x.x, x.y);
     }
 
-    // ---- o = A v + (q exp B) S_0 ----------------------------------------------------------------------
+    // ---- o^T = v^T A^T + S_0^T (q exp B)^T: lane (g, c) ends up with token c, columns 4g..4g+3 of each tile:
+    // one 8-byte store per tile (the operand registers are the same either way round: a lane holds
+    // index c of the tile's outer dimension and 8g..8g+7 of the contraction in both operands)
     f32x4_t o[2];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
-      o[nt] = Mma<BF16>::run(pa, vb[nt], f32x4_t{0.f, 0.f, 0.f, 0.f});
+      o[nt] = Mma<BF16>::run(vb[nt], pa, f32x4_t{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
       for (int s4 = 0; s4 < 4; ++s4) {
         const f32x4_t &a = S[2 * s4][nt], &bb = S[2 * s4 + 1][nt];  // rows 32 s4 + 8g + {0..3}, {4..7}
         const uint4 sb16 = make_uint4(Mma<BF16>::pack(a[0], a[1]), Mma<BF16>::pack(a[2], a[3]),
                                       Mma<BF16>::pack(bb[0], bb[1]), Mma<BF16>::pack(bb[2], bb[3]));
-        o[nt] = Mma<BF16>::run(qa[s4], sb16, o[nt]);
+        o[nt] = Mma<BF16>::run(sb16, qa[s4], o[nt]);
       }
     }
+    if (t0 + c < T) {
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int t = t0 + 4 * g + i;
-        if (t < T) p.out[oo + (int64_t)t * p.o_st + 32 * w + 16 * nt + c] = f32_to_bf16(o[nt][i]);
-      }
+      for (int nt = 0; nt < 2; ++nt)
+        *reinterpret_cast<uint2 *>(p.out + oo + (int64_t)(t0 + c) * p.o_st + 32 * w + 16 * nt + 4 * g) =
+            make_uint2(Mma<BF16>::pack(o[nt][0], o[nt][1]), Mma<BF16>::pack(o[nt][2], o[nt][3]));
+    }
 
     // ---- S <- diag(exp B_16) S + k-hat^T v ------------------------------------------------------------
 #pragma unroll

@@ -356,7 +356,16 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
                           quad_aligned(a->v, a->dtype, p.v_sb, p.v_sh, p.v_st) &&
                           quad_aligned(a->g, a->g_dtype, p.g_sb, p.g_sh, p.g_st) &&
                           quad_aligned(a->out, a->dtype, p.o_sb, p.o_sh, p.o_st);
-  if (a->dtype == SB_BF16 && !(a->flags & SB_GLA_VECTOR_ONLY) &&
+  // the matrix-core kernel moves q, k, v, g as 16-byte pieces and out as 8-byte pieces
+  auto piece_aligned = [](const void *ptr, int64_t per16, int64_t sb_, int64_t sh, int64_t st) {
+    return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0 && sb_ % per16 == 0 && sh % per16 == 0 && st % per16 == 0;
+  };
+  const int64_t g_per16 = a->g_dtype == SB_F32 ? 4 : 8;
+  const bool pieces_ok = piece_aligned(a->q, 8, p.q_sb, p.q_sh, p.q_st) && piece_aligned(a->k, 8, p.k_sb, p.k_sh, p.k_st) &&
+                         piece_aligned(a->v, 8, p.v_sb, p.v_sh, p.v_st) &&
+                         piece_aligned(a->g, g_per16, p.g_sb, p.g_sh, p.g_st) &&
+                         piece_aligned(a->out, 8, p.o_sb, p.o_sh, p.o_st);
+  if (a->dtype == SB_BF16 && pieces_ok && !(a->flags & SB_GLA_VECTOR_ONLY) &&
       (a->cu_seqlens || a->seq_len >= kChunkKernelMinSteps)) {
     launch_gla_chunk(a, groups);
     return check_launch("gla_chunk_kernel");
