@@ -172,9 +172,8 @@ def bench_prefill(sb, dev, S=16, L=8192, iters=5):
 def bench_gla_prompt(sb, dev, S=16, L=8192, H=28, iters=3):
     """The GLA layers' share of BASELINE config 4 (16 prompts x 8192 tokens): one packed launch
     over token-major [tokens, H, D] projections, states read from and left in the slot cache.
-    The kernel is bound by fp32 vector issue: 3 vector operations (multiply, two multiply-adds)
-    per state element and token; the peak quoted is the unpacked fp32 vector rate (half of the
-    157.3 TFLOP/s that counts packed operations, which this build does not emit)."""
+    bf16 prompts run the recurrence 16 tokens at a time on the matrix cores; the step-by-step fp32
+    vector kernel is timed beside it. Bytes: q, k, v, out in bf16 and the fp32 gate, once each."""
     g = torch.Generator().manual_seed(0)
     tokens = S * L
     q, k, v = (torch.randn(tokens, H, D, generator=g).bfloat16().to(dev) for _ in range(3))
@@ -183,18 +182,22 @@ def bench_gla_prompt(sb, dev, S=16, L=8192, H=28, iters=3):
     cu = torch.arange(0, tokens + 1, L, dtype=torch.int32, device=dev)
     slots = torch.arange(S, dtype=torch.int32, device=dev)
     out = torch.empty_like(q)
-    sb.ops.gla_recurrent_packed(q, k, v, gate, cache, cu, slots, out=out, max_seq_len=L)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-    for a, b in evs:
-        a.record()
-        sb.ops.gla_recurrent_packed(q, k, v, gate, cache, cu, slots, out=out, max_seq_len=L)
-        b.record()
-    torch.cuda.synchronize()
-    ms = statistics.mean(a.elapsed_time(b) for a, b in evs)
-    flop = tokens * H * D * D * 5
+    times = {}
+    for name, vector_only in (("matrix_cores", False), ("vector_only", True)):
+        sb.ops.gla_recurrent_packed(q, k, v, gate, cache, cu, slots, out=out, max_seq_len=L, vector_only=vector_only)
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        for a, b in evs:
+            a.record()
+            sb.ops.gla_recurrent_packed(q, k, v, gate, cache, cu, slots, out=out, max_seq_len=L, vector_only=vector_only)
+            b.record()
+        torch.cuda.synchronize()
+        times[name] = statistics.mean(a.elapsed_time(b) for a, b in evs)
+    ms = times["matrix_cores"]
+    nbytes = tokens * H * D * (4 * 2 + 4) + 2 * S * H * D * D * 4
     return {"workload": f"GLA layer over BASELINE config 4's prompts: {S} x {L} tokens, H={H}, bf16 q/k/v, fp32 gate and state",
-            "kernel": "gla_sequence_kernel", "kernel_ms": round(ms, 3), "prompt_tokens_per_s_layer": round(tokens / (ms * 1e-3), 0),
-            "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 2), "frac_fp32_vector_peak_unpacked": round(flop / (ms * 1e-3) / 1e12 / 78.6, 4)}
+            "kernel": "gla_chunk_kernel", "kernel_ms": round(ms, 3), "prompt_tokens_per_s_layer": round(tokens / (ms * 1e-3), 0),
+            "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "vector_only_kernel_ms": round(times["vector_only"], 3)}
 
 
 def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None, gla_state_dtype=torch.float32):

@@ -68,7 +68,7 @@ __device__ __forceinline__ float load_gate(const void *p, int64_t i) {
 }
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t x) { return __uint_as_float((uint32_t)x << 16); }
-__device__ __forceinline__ uint16_t f32_to_bf16(float x) { return (uint16_t)f32_to_bf16_bits(x); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float x) { return __builtin_bit_cast(uint16_t, (__bf16)x); }  // v_cvt_pk_bf16_f32
 
 template <bool kStateF32, int GDT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gla_chunk_kernel(const GlaChunkParams p) {
@@ -117,15 +117,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // ---- block inputs in registers: gates and k for every thread, q (first half) or v (second half) ----
   float rg[kCB];
   uint16_t rk[kCB], rx[kCB];
+  // per-thread column pointers once; a token adds a wave-uniform multiple of the row stride
+  const char *gp = reinterpret_cast<const char *>(p.g) + (go + d) * (GDT == SB_F32 ? 4 : 2);
+  const uint16_t *kp = p.k + ko + d;
+  const uint16_t *xp = second ? p.v + vo + d : p.q + qo + d;
+  const int64_t xs = second ? p.v_st : p.q_st;
   auto fetch = [&](int t0) {
-    const uint16_t *xp = second ? p.v : p.q;
-    const int64_t xo = second ? vo : qo, xs = second ? p.v_st : p.q_st;
+    const int last = T - 1 - t0;  // rows past the end re-read the last token; they are zeroed when used
+    if (last >= kCB - 1) {
 #pragma unroll
-    for (int t = 0; t < kCB; ++t) {
-      const int64_t tt = min(t0 + t, T - 1);  // past the end: reads the last token, zeroed when used
-      rg[t] = load_gate<GDT>(p.g, go + tt * p.g_st + d);
-      rk[t] = p.k[ko + tt * p.k_st + d];
-      rx[t] = xp[xo + tt * xs + d];
+      for (int t = 0; t < kCB; ++t) {
+        rg[t] = load_gate<GDT>(gp, (t0 + t) * p.g_st);
+        rk[t] = kp[(t0 + t) * p.k_st];
+        rx[t] = xp[(t0 + t) * xs];
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < kCB; ++t) {
+        const int64_t tt = t0 + min(t, last);
+        rg[t] = load_gate<GDT>(gp, tt * p.g_st);
+        rk[t] = kp[tt * p.k_st];
+        rx[t] = xp[tt * xs];
+      }
     }
   };
 
