@@ -19,6 +19,13 @@ this path, so nothing here is pinned by a reference fixture):
   gla.*                       closed form S_T = sum_t diag(exp(sum_{u>t} g_u)) k_t^T v_t in
                               float64; g=0, k=0 and q=e_i special cases; slot -1 no-op
                               (tests/test_oracle_gla.py)
+  attention.metatoken_attention   the one-softmax statement equals window attention merged
+                              with the meta-token attention by lse_merge, per head and query;
+                              equal-score closed case (tests/test_oracle_attention.py)
+  quant.*                     hand-computed rows (ties to even, scale exactly 1), both scale
+                              clamps, code saturation, |x - code*scale| <= scale/2, symmetry and
+                              power-of-two invariance; bf16 rounding against torch's conversion
+                              (tests/test_oracle_quant.py)
   paged.*                     brute force over every position of small sequences: the set of
                               resident (block, offset) pairs equals the window; slots are
                               bt[pos//bs]*bs + pos%bs; dense<->paged equivalence
