@@ -6,7 +6,11 @@ these: they are a regression pin. If the oracle (or a kernel) later drifts, test
 fails against data that does not move with the code. Inputs are stored explicitly (bf16 tensors as
 their uint16 bit patterns), so nothing depends on a random-number generator at test time.
 
-    python tests/golden/make_fixtures.py        # rewrites the .npz (deterministic)
+cache_path_v2_ext.npz holds the same kind of vectors for the paths added later (per-row INT8 K/V,
+meta-token attention, GLA over a prompt, a ragged decode batch); it is a file of its own so that v1
+never changes.
+
+    python tests/golden/make_fixtures.py        # rewrites both .npz files (deterministic)
 """
 import os
 import sys
@@ -113,6 +117,60 @@ def main() -> None:
                gla_state_diag=np.diag(st[0, 0]).astype(np.float32))
 
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cache_path_v1.npz")
+    np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
+    write_extensions(np.random.default_rng(20240608))
+
+
+def write_extensions(rng) -> None:
+    """tests/golden/cache_path_v2_ext.npz: the paths added after v1 (its file stays byte-identical)."""
+    from oracle import quant as Q
+
+    out = {}
+    D = 128
+    # 6. per-row INT8: rows of different scales, an all-zero row, a tie row
+    x = (rng.standard_normal((6, 2, D)) * rng.uniform(0.05, 8, (6, 2, 1))).astype(np.float32)
+    x[1, 0] = 0
+    x[2, 1, :4] = [127.0, 63.5, 62.5, -62.5]; x[2, 1, 4:] = 0
+    xb = bf16_bits(x)
+    codes, scale = Q.quantize_rows(bf16_to_f32(xb))
+    out.update(i8_rows=xb, i8_codes=codes, i8_scales=scale, i8_dequant_bf16=Q.dequantize_rows(codes, scale, "bf16"))
+
+    # 7. meta-token attention: 5 queries at the end of 9 keys, window 6, 8 meta tokens, their own 8 queries
+    Hq, Hkv, M = 4, 2, 8
+    q1 = bf16_bits(rng.standard_normal((5, Hq, D)).astype(np.float32))
+    q2 = bf16_bits(rng.standard_normal((M, Hq, D)).astype(np.float32))
+    k1, v1 = (bf16_bits(rng.standard_normal((9, Hkv, D)).astype(np.float32)) for _ in range(2))
+    k2, v2 = (bf16_bits(rng.standard_normal((M, Hkv, D)).astype(np.float32)) for _ in range(2))
+    mo = A.metatoken_attention(*(bf16_to_f32(t) for t in (q1, q2, k1, k2, v1, v2)), D ** -0.5, 6)
+    out.update(mt_q1=q1, mt_q2=q2, mt_k1=k1, mt_v1=v1, mt_k2=k2, mt_v2=v2, mt_sliding_window=np.array(6),
+               mt_out=mo.astype(np.float32))
+
+    # 8. GLA over a 40-token prompt (one head): outputs and state summaries
+    T = 40
+    gq, gk, gv = (bf16_bits(np.maximum(rng.standard_normal((1, 1, T, D)), -0.5).astype(np.float32)) for _ in range(3))
+    gg = (-np.log1p(np.exp(-rng.standard_normal((1, 1, T, D)))) / 16).astype(np.float32)
+    s0 = (rng.standard_normal((1, 1, D, D)) * 0.02).astype(np.float32)
+    go, gs = G.gla_recurrent(bf16_to_f32(gq), bf16_to_f32(gk), bf16_to_f32(gv), gg, s0.astype(np.float64))
+    out.update(glp_q=gq, glp_k=gk, glp_v=gv, glp_g=gg, glp_state0=s0, glp_out=go.astype(np.float32),
+               glp_state_rowsum=gs[0, 0].sum(1).astype(np.float32), glp_state_diag=np.diag(gs[0, 0]).astype(np.float32),
+               glp_state_absmax=np.array(np.abs(gs).max(), np.float32))
+
+    # 9. ragged paged decode (rows of 3, 150 and 40 keys, no window): the case the balanced split is for
+    Hq, Hkv, bs = 4, 2, 16
+    lens = [3, 150, 40]
+    nblk = 16
+    kc = bf16_bits(rng.standard_normal((nblk, bs, Hkv, D)).astype(np.float32))
+    vc = bf16_bits(rng.standard_normal((nblk, bs, Hkv, D)).astype(np.float32))
+    q = bf16_bits(rng.standard_normal((3, Hq, D)).astype(np.float32))
+    tables = np.zeros((3, 10), np.int32)
+    tables[0, :1] = [9]; tables[1, :10] = [4, 0, 11, 7, 2, 15, 6, 1, 13, 8]; tables[2, :3] = [3, 12, 5]
+    o, lse = A.paged_decode_attention(bf16_to_f32(q), bf16_to_f32(kc), bf16_to_f32(vc), tables, lens, D ** -0.5, -1,
+                                      return_lse=True)
+    out.update(rag_q=q, rag_k_cache=kc, rag_v_cache=vc, rag_tables=tables, rag_lens=np.array(lens, np.int32),
+               rag_out=o.astype(np.float32), rag_lse=lse.astype(np.float32))
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cache_path_v2_ext.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
 
