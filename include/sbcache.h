@@ -108,6 +108,7 @@ int sb_kv_append(const sb_kv_append_args *args);
  * ------------------------------------------------------------------------------------ */
 #define SB_KV_NONE 0
 #define SB_KV_INT8 1
+#define SB_KV_FP8 2
 #define SB_DECODE_FORCE_VALU 1 /* bf16/fp16: use the vector-ALU split kernel instead of the matrix-core one */
 /* bf16/fp16, n_split > 1, up to 1024 rows: cut the chunks of ALL rows, laid end to end, into equal runs
  * (about one per CU) instead of cutting every row into n_split runs, so that rows of different
@@ -162,6 +163,10 @@ typedef struct sb_swa_decode_args {
   const float *k_scale;
   const float *v_scale;
   int32_t kv_quant;
+  /* fp8 cache (kv_quant = SB_KV_FP8): k_cache/v_cache hold e4m3fn codes [num_blocks, block_size, Hkv, 128]
+   * (kv strides in bytes), dequantised as code * k_scale_tensor / v_scale_tensor. Same restrictions as
+   * the INT8 cache. */
+  float k_scale_tensor, v_scale_tensor;
 } sb_swa_decode_args;
 
 /* Split count the auto rule (n_split = 0) would use for these shapes. */
@@ -353,6 +358,38 @@ typedef struct sb_quantize_sym_args {
 } sb_quantize_sym_args;
 
 int sb_quantize_sym(const sb_quantize_sym_args *args);
+
+/* ------------------------------------------------------------------------------------
+ * fp8 (OCP e4m3fn) K/V with per-tensor scales: the kv_cache_dtype = "fp8" branch of
+ *   vllm_hymeta/attention/meta_attention.py:790-812 (reshape_and_cache_flash with layer._k_scale /
+ *   layer._v_scale; the cache tensor viewed as float8_e4m3fn).
+ * code = e4m3fn(clamp(x / scale, -448, 448)), round to nearest even, NaN kept; value = code * scale.
+ * sb_kv_append_fp8: slot-mapped append into byte caches [num_blocks, block_size, num_kv_heads, 128]
+ *   (strides in bytes); same slot_mapping contract as sb_kv_append.
+ * sb_fp8_round: out = e4m3fn(clamp(in / scale)) * scale rounded to dtype, row by row (rows of
+ *   row_elems elements, a multiple of 8): what a tensor looks like after the fp8 round trip, for
+ *   queries (scaled_fp8_quant at :806-811) and for K/V attended to before they are cached (:853-869).
+ * sb_swa_decode reads such a cache with kv_quant = SB_KV_FP8 and k_scale_tensor / v_scale_tensor.
+ * ------------------------------------------------------------------------------------ */
+typedef struct sb_kv_append_fp8_args {
+  const void *key;
+  const void *value;
+  void *k_cache;
+  void *v_cache;
+  const int64_t *slot_mapping;
+  int64_t num_tokens;
+  int32_t num_kv_heads, head_size, block_size, dtype;
+  int64_t key_stride_token, key_stride_head;     /* elements */
+  int64_t value_stride_token, value_stride_head;
+  int64_t cache_stride_block, cache_stride_row, cache_stride_head; /* bytes */
+  float k_scale, v_scale;
+  void *stream;
+} sb_kv_append_fp8_args;
+
+int sb_kv_append_fp8(const sb_kv_append_fp8_args *args);
+
+int sb_fp8_round(const void *in, void *out, int64_t rows, int64_t row_elems, int64_t in_stride_row,
+                 int64_t out_stride_row, int32_t dtype, float scale, void *stream);
 
 /* ------------------------------------------------------------------------------------
  * Merge of two attention results over disjoint key sets by their log-sum-exps, in place:

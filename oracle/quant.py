@@ -60,3 +60,34 @@ def kv_append_int8(key: np.ndarray, value: np.ndarray, k_cache: np.ndarray, v_ca
         b, o = divmod(int(slot), bs)
         k_cache[b, o] = kc[t]; v_cache[b, o] = vc[t]
         k_scale[b, :, o] = ks[t]; v_scale[b, :, o] = vs[t]
+
+
+# ---- fp8 (OCP e4m3fn) with per-tensor scales ---------------------------------------------------------
+# The kv_cache_dtype="fp8" branch of reshape_and_cache_flash (vllm_hymeta/attention/meta_attention.py:790-799)
+# and scaled_fp8_quant (:806-811, :853-869). The kernels live in vllm 0.10.0, absent here: restated from
+# its published behaviour, code = e4m3fn(x / scale) with saturation at +-448 and round to nearest even.
+# The rounding itself is torch's own float8_e4m3fn cast (a library routine, checked code by code in
+# tests/test_oracle_quant.py); parity with vllm's kernel is unpinned.
+
+def fp8_codes(x: np.ndarray, scale: float) -> np.ndarray:
+    """uint8 e4m3fn codes of x / scale (float32 division, saturating, ties to even, NaN kept)."""
+    import torch
+    y = torch.from_numpy(np.ascontiguousarray(x, np.float32)) / np.float32(scale)
+    y = torch.where(torch.isnan(y), y, y.clamp(-448.0, 448.0))
+    return y.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+
+
+def fp8_values(codes: np.ndarray, scale: float) -> np.ndarray:
+    """float32 value of each code times scale."""
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(codes, np.uint8)).view(torch.float8_e4m3fn).float().numpy() * np.float32(scale)
+
+
+def fp8_round(x: np.ndarray, scale: float, dtype: str = "bf16") -> np.ndarray:
+    """x after the fp8 round trip, rounded to the tensor's dtype; returned as float32."""
+    y = fp8_values(fp8_codes(x, scale), scale)
+    if dtype == "bf16":
+        return round_to_bf16(y)
+    if dtype == "f16":
+        return y.astype(np.float16).astype(np.float32)
+    return y

@@ -18,7 +18,7 @@ SB_BF16, SB_F16, SB_F32 = 0, 1, 2
 SB_ERR_INVALID, SB_ERR_UNSUPPORTED, SB_ERR_WORKSPACE = -1, -2, -3
 SB_DECODE_FORCE_VALU = 1
 SB_DECODE_BALANCED = 2
-SB_KV_NONE, SB_KV_INT8 = 0, 1
+SB_KV_NONE, SB_KV_INT8, SB_KV_FP8 = 0, 1, 2
 SB_GLA_VECTOR_ONLY = 1
 ABI_VERSION = 1
 
@@ -56,6 +56,7 @@ class SwaDecodeArgs(C.Structure):
         ("new_key_stride_row", i64), ("new_key_stride_head", i64),
         ("new_value_stride_row", i64), ("new_value_stride_head", i64),
         ("stream", vp), ("k_scale", vp), ("v_scale", vp), ("kv_quant", i32),
+        ("k_scale_tensor", f32), ("v_scale_tensor", f32),
     ]
 
 
@@ -121,6 +122,18 @@ class KvAppendInt8Args(C.Structure):
     ]
 
 
+class KvAppendFp8Args(C.Structure):
+    _fields_ = [
+        ("key", vp), ("value", vp), ("k_cache", vp), ("v_cache", vp), ("slot_mapping", vp), ("num_tokens", i64),
+        ("num_kv_heads", i32), ("head_size", i32), ("block_size", i32), ("dtype", i32),
+        ("key_stride_token", i64), ("key_stride_head", i64),
+        ("value_stride_token", i64), ("value_stride_head", i64),
+        ("cache_stride_block", i64), ("cache_stride_row", i64), ("cache_stride_head", i64),
+        ("k_scale", f32), ("v_scale", f32),
+        ("stream", vp),
+    ]
+
+
 class QuantizeSymArgs(C.Structure):
     _fields_ = [
         ("in_", vp), ("out", vp), ("rows", i64), ("heads", i32), ("head_size", i32), ("dtype", i32),
@@ -156,6 +169,8 @@ EXPORTS = {
     "sb_lse_merge": (C.c_int, [C.POINTER(LseMergeArgs)]),
     "sb_kv_append_int8": (C.c_int, [C.POINTER(KvAppendInt8Args)]),
     "sb_quantize_sym": (C.c_int, [C.POINTER(QuantizeSymArgs)]),
+    "sb_kv_append_fp8": (C.c_int, [C.POINTER(KvAppendFp8Args)]),
+    "sb_fp8_round": (C.c_int, [vp, vp, i64, i64, i64, i64, i32, f32, vp]),
     "sb_stream_copy": (C.c_int, [vp, vp, i64, vp]),
 }
 

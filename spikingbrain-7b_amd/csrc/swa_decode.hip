@@ -20,7 +20,7 @@
 namespace sb_host {
 void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
                                   hipStream_t st, const sb::DecodeParams &p);
-void launch_swa_decode_split_i8(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, hipStream_t st,
+void launch_swa_decode_split_i8(int dtype, int kv_quant, int G, int Hkv, unsigned rows, unsigned n_split, hipStream_t st,
                                 const sb::DecodeParams &p);
 }
 
@@ -551,18 +551,21 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
     case SB_F32: esz = 4; break;
     default: return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: unknown dtype %d", a->dtype);
   }
-  const bool int8_kv = a->kv_quant == SB_KV_INT8;
+  const bool fp8_kv = a->kv_quant == SB_KV_FP8;
+  const bool int8_kv = a->kv_quant == SB_KV_INT8 || fp8_kv;   // byte codes: the same kernel family
   if (a->kv_quant != SB_KV_NONE && !int8_kv)
     return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: unknown kv_quant %d", a->kv_quant);
+  if (fp8_kv && (!(a->k_scale_tensor > 0.f) || !(a->v_scale_tensor > 0.f)))
+    return fail(SB_ERR_INVALID, "sb_swa_decode: the fp8 cache needs positive k_scale_tensor and v_scale_tensor");
   const int kv_esz = int8_kv ? 1 : esz;
   if (int8_kv) {
     if (a->dtype == SB_F32 || (a->flags & SB_DECODE_FORCE_VALU))
       return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: the INT8 cache needs bf16 or fp16 queries on the matrix-core path");
-    if (!a->block_table || !a->k_scale || !a->v_scale)
+    if (!a->block_table || (!fp8_kv && (!a->k_scale || !a->v_scale)))
       return fail(SB_ERR_INVALID, "sb_swa_decode: the INT8 cache needs paged mode and both scale tensors");
     if (a->new_key || a->new_value || a->new_slot_mapping)
       return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: no fused append into the INT8 cache (call sb_kv_append_int8 first)");
-    if ((reinterpret_cast<uintptr_t>(a->k_scale) | reinterpret_cast<uintptr_t>(a->v_scale)) & 15u)
+    if (!fp8_kv && ((reinterpret_cast<uintptr_t>(a->k_scale) | reinterpret_cast<uintptr_t>(a->v_scale)) & 15u))
       return fail(SB_ERR_INVALID, "sb_swa_decode: scale tensors not 16-byte aligned");
   }
   const int64_t es[] = {a->q_stride_row, a->q_stride_head};
@@ -608,6 +611,11 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   p.kv_sb = a->kv_stride_block * kv_esz; p.kv_sr = a->kv_stride_row * kv_esz; p.kv_sh = a->kv_stride_head * kv_esz;
   p.bt_stride = a->block_table_stride;
   p.k_scale = a->k_scale; p.v_scale = a->v_scale;
+  p.kv_out_scale = 1.f;
+  if (fp8_kv) {  // scores scale with the K tensor scale, the result with the V tensor scale
+    p.scale_log2 *= a->k_scale_tensor;
+    p.kv_out_scale = a->v_scale_tensor;
+  }
 
   const int G = a->num_q_heads / a->num_kv_heads;
   const dim3 grid((unsigned)a->num_rows, (unsigned)a->num_kv_heads, (unsigned)n_split);
@@ -663,7 +671,7 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   if (mfma && !int8_kv && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
     p.n_wg = (int)balanced_workgroups(a->num_rows, n_split);
   if (a->phases != 2) {
-    if (int8_kv) launch_swa_decode_split_i8(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p);
+    if (int8_kv) launch_swa_decode_split_i8(a->dtype, a->kv_quant, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p);
     else if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
                                            (a->flags >> 4) & 7, st, p);
     else if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);

@@ -32,33 +32,38 @@ struct ChunkI8 {
   float4 ks[2], vs[2];  // scales of keys 4g..4g+3 of tile 0 / tile 1
 };
 
-template <int B>
+// byte B of w as a float: a signed INT8 code, or an fp8 (OCP e4m3fn) code
+template <int Q, int B>
 __device__ __forceinline__ float code_to_float(uint32_t w) {
-  return (float)(int)(int8_t)(w >> (8 * B));
+  if constexpr (Q == SB_KV_INT8) return (float)(int)(int8_t)(w >> (8 * B));
+  else return __builtin_amdgcn_cvt_f32_fp8((int)w, B);
 }
 
 // 8 codes (two dwords) -> 8 elements of type E
-template <typename E>
+template <typename E, int Q>
 __device__ __forceinline__ uint4 widen8(uint32_t lo, uint32_t hi) {
-  return make_uint4(Mma<E>::pack(code_to_float<0>(lo), code_to_float<1>(lo)),
-                    Mma<E>::pack(code_to_float<2>(lo), code_to_float<3>(lo)),
-                    Mma<E>::pack(code_to_float<0>(hi), code_to_float<1>(hi)),
-                    Mma<E>::pack(code_to_float<2>(hi), code_to_float<3>(hi)));
+  return make_uint4(Mma<E>::pack(code_to_float<Q, 0>(lo), code_to_float<Q, 1>(lo)),
+                    Mma<E>::pack(code_to_float<Q, 2>(lo), code_to_float<Q, 3>(lo)),
+                    Mma<E>::pack(code_to_float<Q, 0>(hi), code_to_float<Q, 1>(hi)),
+                    Mma<E>::pack(code_to_float<Q, 2>(hi), code_to_float<Q, 3>(hi)));
 }
 
 __device__ __forceinline__ uint32_t word2(const uint2 &v, int i) { return i == 0 ? v.x : v.y; }
 
-template <typename E, int B>
+template <typename E, int Q, int B>
 __device__ __forceinline__ uint4 v_column(const uint2 (&v)[8], int w) {
-  return make_uint4(Mma<E>::pack(code_to_float<B>(word2(v[0], w)), code_to_float<B>(word2(v[1], w))),
-                    Mma<E>::pack(code_to_float<B>(word2(v[2], w)), code_to_float<B>(word2(v[3], w))),
-                    Mma<E>::pack(code_to_float<B>(word2(v[4], w)), code_to_float<B>(word2(v[5], w))),
-                    Mma<E>::pack(code_to_float<B>(word2(v[6], w)), code_to_float<B>(word2(v[7], w))));
+  return make_uint4(Mma<E>::pack(code_to_float<Q, B>(word2(v[0], w)), code_to_float<Q, B>(word2(v[1], w))),
+                    Mma<E>::pack(code_to_float<Q, B>(word2(v[2], w)), code_to_float<Q, B>(word2(v[3], w))),
+                    Mma<E>::pack(code_to_float<Q, B>(word2(v[4], w)), code_to_float<Q, B>(word2(v[5], w))),
+                    Mma<E>::pack(code_to_float<Q, B>(word2(v[6], w)), code_to_float<Q, B>(word2(v[7], w))));
 }
 
 // 256 registers per wavefront (two per SIMD): the matrix-core results then live in ordinary registers
 // and the rescale inside the loop costs no accumulator-register traffic.
-template <typename E>
+// Q = SB_KV_FP8: the codes are fp8 with one scale per tensor: the K scale is folded into the softmax
+// scale and the V scale into the result on the host side of the launch, nothing per key; an fp8 byte
+// CAN be a NaN, so the V codes of masked keys are zeroed before they meet their zero probability.
+template <typename E, int Q>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void swa_decode_split_i8_kernel(const DecodeParams p, const int G, const int Hkv) {
   const int64_t r = blockIdx.x;
   const int split = blockIdx.z;
@@ -120,9 +125,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const unsigned long long w = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(vp + voff[j]));
         ck.v[4 * t + j] = make_uint2((uint32_t)w, (uint32_t)(w >> 32));
       }
-      const int64_t sbase = (blk * Hkv + kvh) * p.block_size + row + 4 * g;
-      ck.ks[t] = *reinterpret_cast<const float4 *>(p.k_scale + sbase);
-      ck.vs[t] = *reinterpret_cast<const float4 *>(p.v_scale + sbase);
+      if constexpr (Q == SB_KV_INT8) {
+        const int64_t sbase = (blk * Hkv + kvh) * p.block_size + row + 4 * g;
+        ck.ks[t] = *reinterpret_cast<const float4 *>(p.k_scale + sbase);
+        ck.vs[t] = *reinterpret_cast<const float4 *>(p.v_scale + sbase);
+      }
     }
   };
 
@@ -131,12 +138,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const uint4 &a = ck.k[0][s >> 1], &b = ck.k[1][s >> 1];
-      s0 = Mma<E>::run((s & 1) ? widen8<E>(a.z, a.w) : widen8<E>(a.x, a.y), qb[s], s0);
-      s1 = Mma<E>::run((s & 1) ? widen8<E>(b.z, b.w) : widen8<E>(b.x, b.y), qb[s], s1);
+      s0 = Mma<E>::run((s & 1) ? widen8<E, Q>(a.z, a.w) : widen8<E, Q>(a.x, a.y), qb[s], s0);
+      s1 = Mma<E>::run((s & 1) ? widen8<E, Q>(b.z, b.w) : widen8<E, Q>(b.x, b.y), qb[s], s1);
     }
-    float sc[8] = {s0[0] * ck.ks[0].x, s0[1] * ck.ks[0].y, s0[2] * ck.ks[0].z, s0[3] * ck.ks[0].w,
-                   s1[0] * ck.ks[1].x, s1[1] * ck.ks[1].y, s1[2] * ck.ks[1].z, s1[3] * ck.ks[1].w};
-    const float vsc[8] = {ck.vs[0].x, ck.vs[0].y, ck.vs[0].z, ck.vs[0].w, ck.vs[1].x, ck.vs[1].y, ck.vs[1].z, ck.vs[1].w};
+    float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+    float vsc[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
+    if constexpr (Q == SB_KV_INT8) {
+      const float ksc[8] = {ck.ks[0].x, ck.ks[0].y, ck.ks[0].z, ck.ks[0].w, ck.ks[1].x, ck.ks[1].y, ck.ks[1].z, ck.ks[1].w};
+      const float vs8[8] = {ck.vs[0].x, ck.vs[0].y, ck.vs[0].z, ck.vs[0].w, ck.vs[1].x, ck.vs[1].y, ck.vs[1].z, ck.vs[1].w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        sc[j] *= ksc[j];
+        vsc[j] = vs8[j];
+      }
+    }
     bool vis[8];
     const int i0 = ch << 5;
 #pragma unroll
@@ -160,6 +175,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       psum += e;
       pv[j] = vis[j] ? e * vsc[j] : 0.f;
     }
+    uint2 vq[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) vq[j] = (Q == SB_KV_FP8 && !vis[j]) ? make_uint2(0u, 0u) : ck.v[j];
     l = fmaf(l, alpha, psum);
     if (__builtin_amdgcn_ballot_w64(grew) != 0) {
 #pragma unroll
@@ -167,14 +185,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     const uint4 pb = make_uint4(Mma<E>::pack(pv[0], pv[1]), Mma<E>::pack(pv[2], pv[3]),
                                 Mma<E>::pack(pv[4], pv[5]), Mma<E>::pack(pv[6], pv[7]));
-    acc[0] = Mma<E>::run(v_column<E, 0>(ck.v, 0), pb, acc[0]);
-    acc[1] = Mma<E>::run(v_column<E, 1>(ck.v, 0), pb, acc[1]);
-    acc[2] = Mma<E>::run(v_column<E, 2>(ck.v, 0), pb, acc[2]);
-    acc[3] = Mma<E>::run(v_column<E, 3>(ck.v, 0), pb, acc[3]);
-    acc[4] = Mma<E>::run(v_column<E, 0>(ck.v, 1), pb, acc[4]);
-    acc[5] = Mma<E>::run(v_column<E, 1>(ck.v, 1), pb, acc[5]);
-    acc[6] = Mma<E>::run(v_column<E, 2>(ck.v, 1), pb, acc[6]);
-    acc[7] = Mma<E>::run(v_column<E, 3>(ck.v, 1), pb, acc[7]);
+    acc[0] = Mma<E>::run(v_column<E, Q, 0>(vq, 0), pb, acc[0]);
+    acc[1] = Mma<E>::run(v_column<E, Q, 1>(vq, 0), pb, acc[1]);
+    acc[2] = Mma<E>::run(v_column<E, Q, 2>(vq, 0), pb, acc[2]);
+    acc[3] = Mma<E>::run(v_column<E, Q, 3>(vq, 0), pb, acc[3]);
+    acc[4] = Mma<E>::run(v_column<E, Q, 0>(vq, 1), pb, acc[4]);
+    acc[5] = Mma<E>::run(v_column<E, Q, 1>(vq, 1), pb, acc[5]);
+    acc[6] = Mma<E>::run(v_column<E, Q, 2>(vq, 1), pb, acc[6]);
+    acc[7] = Mma<E>::run(v_column<E, Q, 3>(vq, 1), pb, acc[7]);
   };
 
   // one chunk of loads in flight behind the one being computed; two register sets, the loop
@@ -200,7 +218,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if (c < G) {
     const int hq = kvh * G + c;
     if (p.n_split == 1) {
-      const float inv = l > 0.f ? 1.f / l : 0.f;
+      const float inv = l > 0.f ? p.kv_out_scale / l : 0.f;
       char *dst = p.out + (r * p.o_sr + (int64_t)hq * p.o_sh + 32 * g) * 2;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -215,10 +233,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     } else {
       const int64_t part = (r * p.Hq + hq) * p.n_split + split;
       float *dst = p.ws_acc + part * 128 + 32 * g;
+      const float os = p.kv_out_scale;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        reinterpret_cast<float4 *>(dst + 8 * i)[0] = make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]);
-        reinterpret_cast<float4 *>(dst + 8 * i)[1] = make_float4(acc[4][i], acc[5][i], acc[6][i], acc[7][i]);
+        reinterpret_cast<float4 *>(dst + 8 * i)[0] = make_float4(acc[0][i] * os, acc[1][i] * os, acc[2][i] * os, acc[3][i] * os);
+        reinterpret_cast<float4 *>(dst + 8 * i)[1] = make_float4(acc[4][i] * os, acc[5][i] * os, acc[6][i] * os, acc[7][i] * os);
       }
       if (g == 0) {
         p.ws_ml[part * 2] = m;
@@ -232,13 +251,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 namespace sb_host {
 
-// Launches the INT8-cache split kernel (query dtype bf16 or fp16, group size <= 16, paged mode).
-void launch_swa_decode_split_i8(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, hipStream_t st,
+// Launches the split kernel over an INT8 or fp8 cache (query dtype bf16 or fp16, group size <= 16, paged mode).
+void launch_swa_decode_split_i8(int dtype, int kv_quant, int G, int Hkv, unsigned rows, unsigned n_split, hipStream_t st,
                                 const sb::DecodeParams &p) {
   const int waves = Hkv < 4 ? Hkv : 4;
   const dim3 grid(rows, (unsigned)((Hkv + waves - 1) / waves), n_split), block(64 * waves);
-  if (dtype == SB_BF16) hipLaunchKernelGGL((swa_decode_split_i8_kernel<sb::BF16>), grid, block, 0, st, p, G, Hkv);
-  else hipLaunchKernelGGL((swa_decode_split_i8_kernel<sb::F16>), grid, block, 0, st, p, G, Hkv);
+  if (kv_quant == SB_KV_INT8) {
+    if (dtype == SB_BF16) hipLaunchKernelGGL((swa_decode_split_i8_kernel<sb::BF16, SB_KV_INT8>), grid, block, 0, st, p, G, Hkv);
+    else hipLaunchKernelGGL((swa_decode_split_i8_kernel<sb::F16, SB_KV_INT8>), grid, block, 0, st, p, G, Hkv);
+  } else {
+    if (dtype == SB_BF16) hipLaunchKernelGGL((swa_decode_split_i8_kernel<sb::BF16, SB_KV_FP8>), grid, block, 0, st, p, G, Hkv);
+    else hipLaunchKernelGGL((swa_decode_split_i8_kernel<sb::F16, SB_KV_FP8>), grid, block, 0, st, p, G, Hkv);
+  }
 }
 
 }  // namespace sb_host

@@ -31,6 +31,7 @@ struct DecodeParams {
   // INT8 cache: per-row scales [num_blocks, Hkv, block_size]
   const float *k_scale;
   const float *v_scale;
+  float kv_out_scale;  // multiplies the result (fp8 cache: the V tensor scale; else 1)
 };
 
 }  // namespace sb

@@ -96,6 +96,7 @@ def swa_decode_attention(
     host_seq_lens=None,
     k_scale: Optional[torch.Tensor] = None,
     v_scale: Optional[torch.Tensor] = None,
+    fp8_scales: Optional[Tuple[float, float]] = None,
     pipeline_depth: int = 0,
     new_key: Optional[torch.Tensor] = None,
     new_value: Optional[torch.Tensor] = None,
@@ -123,19 +124,30 @@ def swa_decode_attention(
     a lot, a little slower when they do not. Default: decided from host_seq_lens (the same numbers
     as seq_lens, as Python ints) when the caller has them, else off.
     k_scale, v_scale (fp32 [num_blocks, Hkv, block_size]): the caches are per-row INT8 codes as
-    kv_append_int8 wrote them (paged mode, bf16/fp16 queries, append not fused)."""
+    kv_append_int8 wrote them (paged mode, bf16/fp16 queries, append not fused).
+    fp8_scales (k_scale, v_scale floats): the caches are fp8 (e4m3fn) codes as kv_append_fp8 wrote them
+    (float8_e4m3fn or uint8 tensors), dequantised as code * scale; same restrictions."""
     dev = N.require_gpu(q, key_cache, value_cache, seq_lens, block_table, kv_start, row_seq, key_lo, out)
     if q.dim() != 3:
         raise ValueError(f"q must be [rows, num_heads, head_size], got {tuple(q.shape)}")
     R, Hq, D = q.shape
     _inner_contiguous(q, "q")
-    int8_kv = k_scale is not None or v_scale is not None
+    fp8_kv = fp8_scales is not None
+    int8_kv = k_scale is not None or v_scale is not None or fp8_kv     # byte-code caches
+    if fp8_kv:
+        if k_scale is not None or v_scale is not None or block_table is None:
+            raise ValueError("the fp8 cache needs paged mode and takes fp8_scales instead of k_scale/v_scale")
+        if key_cache.dtype not in (torch.float8_e4m3fn, torch.uint8) or value_cache.dtype != key_cache.dtype:
+            raise ValueError("with fp8_scales the caches must be float8_e4m3fn (or uint8) tensors")
+        if key_cache.dtype != torch.uint8:
+            key_cache, value_cache = key_cache.view(torch.uint8), value_cache.view(torch.uint8)
     if int8_kv:
-        N.require_gpu(q, k_scale, v_scale)
-        if k_scale is None or v_scale is None or block_table is None:
-            raise ValueError("the INT8 cache needs k_scale, v_scale and paged mode")
-        if key_cache.dtype != torch.int8 or value_cache.dtype != torch.int8:
-            raise ValueError("with k_scale/v_scale the caches must be int8")
+        if not fp8_kv:
+            N.require_gpu(q, k_scale, v_scale)
+            if k_scale is None or v_scale is None or block_table is None:
+                raise ValueError("the INT8 cache needs k_scale, v_scale and paged mode")
+            if key_cache.dtype != torch.int8 or value_cache.dtype != torch.int8:
+                raise ValueError("with k_scale/v_scale the caches must be int8")
         if q.dtype not in (torch.bfloat16, torch.float16) or force_valu:
             raise NotImplementedError("the INT8 cache needs bf16 or fp16 queries on the matrix-core path")
         if new_key is not None or new_value is not None or new_slot_mapping is not None:
@@ -154,7 +166,7 @@ def swa_decode_attention(
             raise ValueError("block_table must be a 2-D int32 tensor with contiguous rows")
         bt_stride = block_table.stride(0)
         bound = block_table.shape[1] * bs
-        if int8_kv:
+        if int8_kv and not fp8_kv:
             for t, name in ((k_scale, "k_scale"), (v_scale, "v_scale")):
                 if t.shape != (nb, Hkv, bs) or t.dtype != torch.float32 or not t.is_contiguous():
                     raise ValueError(f"{name} must be a contiguous float32 [num_blocks, num_kv_heads, block_size] tensor")
@@ -222,7 +234,10 @@ def swa_decode_attention(
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
         kv_stride_block=kv_strides[0], kv_stride_row=kv_strides[1], kv_stride_head=kv_strides[2],
         block_table_stride=bt_stride, stream=N.stream_ptr(dev),
-        k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale), kv_quant=N.SB_KV_INT8 if int8_kv else N.SB_KV_NONE, **fused)
+        k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale),
+        kv_quant=N.SB_KV_FP8 if fp8_kv else (N.SB_KV_INT8 if int8_kv else N.SB_KV_NONE),
+        k_scale_tensor=float(fp8_scales[0]) if fp8_kv else 0.0, v_scale_tensor=float(fp8_scales[1]) if fp8_kv else 0.0,
+        **fused)
     N.check(L.sb_swa_decode(C.byref(a)), "swa_decode")
     return (out, lse) if return_lse else out
 
@@ -265,6 +280,53 @@ def kv_append_int8(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor
         cache_stride_block=k_cache.stride(0), cache_stride_row=k_cache.stride(1), cache_stride_head=k_cache.stride(2),
         stream=N.stream_ptr(dev))
     N.check(N.lib().sb_kv_append_int8(C.byref(a)), "kv_append_int8")
+
+
+def kv_append_fp8(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  slot_mapping: torch.Tensor, k_scale: float = 1.0, v_scale: float = 1.0) -> None:
+    """Store this step's K/V rows as fp8 (e4m3fn) codes of x / scale (saturating at +-448) at their slots;
+    slots < 0 are skipped. Caches float8_e4m3fn or uint8 [nb, bs, Hkv, 128]."""
+    dev = N.require_gpu(key, value, k_cache, v_cache, slot_mapping)
+    if key.dim() != 3 or value.shape != key.shape or value.dtype != key.dtype:
+        raise ValueError("key and value must be [tokens, num_kv_heads, head_size] of one dtype")
+    T, Hkv, D = key.shape
+    if k_cache.dtype not in (torch.float8_e4m3fn, torch.uint8) or v_cache.dtype != k_cache.dtype or k_cache.dim() != 4 \
+            or v_cache.shape != k_cache.shape or k_cache.stride() != v_cache.stride():
+        raise ValueError("k_cache and v_cache must be float8_e4m3fn/uint8 [num_blocks, block_size, num_kv_heads, head_size] "
+                         "with equal strides")
+    if k_cache.shape[2:] != (Hkv, D) or k_cache.stride(3) != 1:
+        raise ValueError(f"cache rows must be [{Hkv}, {D}] with a contiguous head dimension")
+    _inner_contiguous(key, "key")
+    _inner_contiguous(value, "value")
+    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous() or slot_mapping.numel() < T:
+        raise ValueError("slot_mapping must be a contiguous int64 vector with one entry per token")
+    a = N.KvAppendFp8Args(
+        key=N.ptr(key), value=N.ptr(value), k_cache=N.ptr(k_cache), v_cache=N.ptr(v_cache),
+        slot_mapping=N.ptr(slot_mapping), num_tokens=T, num_kv_heads=Hkv, head_size=D, block_size=k_cache.shape[1],
+        dtype=N.dtype_code(key.dtype), key_stride_token=key.stride(0), key_stride_head=key.stride(1),
+        value_stride_token=value.stride(0), value_stride_head=value.stride(1),
+        cache_stride_block=k_cache.stride(0), cache_stride_row=k_cache.stride(1), cache_stride_head=k_cache.stride(2),
+        k_scale=float(k_scale), v_scale=float(v_scale), stream=N.stream_ptr(dev))
+    N.check(N.lib().sb_kv_append_fp8(C.byref(a)), "kv_append_fp8")
+
+
+def fp8_round(x: torch.Tensor, scale: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x after a round trip through fp8: e4m3fn(clamp(x / scale, -448, 448)) * scale in x's dtype (what
+    scaled_fp8_quant followed by the kernel's descale makes of a query, meta_attention.py:806-811).
+    x: any shape with a contiguous last dimension that is a multiple of 8; out may be x."""
+    dev = N.require_gpu(x, out)
+    if x.dim() < 1 or x.stride(-1) != 1 or x.shape[-1] % 8 != 0:
+        raise ValueError("x needs a contiguous last dimension that is a multiple of 8")
+    x2 = x.reshape(-1, x.shape[-1]) if x.is_contiguous() else None
+    if x2 is None:
+        raise ValueError("x must be contiguous")
+    if out is None:
+        out = torch.empty_like(x)
+    elif out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous():
+        raise ValueError("out must be contiguous and match x in shape and dtype")
+    N.check(N.lib().sb_fp8_round(N.ptr(x), N.ptr(out), x2.shape[0], x2.shape[1], x2.stride(0), x2.stride(0),
+                                 N.dtype_code(x.dtype), float(scale), N.stream_ptr(dev)), "fp8_round")
+    return out
 
 
 def quantize_sym(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:

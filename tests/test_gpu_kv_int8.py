@@ -220,3 +220,70 @@ def test_backend_engine_with_int8_cache(sb, dev):
     before = runner.kv_caches[0].codes[:, src].clone(), runner.kv_caches[0].scales[:, src].clone()
     sb.MetaAttentionBackend.copy_blocks(runner.kv_caches, torch.tensor([[src, dst]], dtype=torch.int64, device=dev))
     assert torch.equal(runner.kv_caches[0].codes[:, dst], before[0]) and torch.equal(runner.kv_caches[0].scales[:, dst], before[1])
+
+
+# ---------------------------------------------------------------- fp8 (e4m3fn) cache
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("scales", [(1.0, 1.0), (0.5, 0.03125)])
+def test_append_fp8_and_round_bit_exact(sb, dev, dtype, scales):
+    nb, bs, T, H = 6, 16, 30, 4
+    g = torch.Generator().manual_seed(21)
+    k = (torch.randn(T, H, D, generator=g) * 10 ** torch.empty(T, H, 1).uniform_(-3, 2.5, generator=g)).to(dtype)
+    v = (torch.randn(T, H, D, generator=g) * 3).to(dtype)
+    k[0, 0, :6] = torch.tensor([448.0, 464.0, 1000.0, -3000.0, 2.0 ** -9, 1.5 * 2.0 ** -9]).to(dtype)   # saturation, subnormals, a tie
+    slots = torch.randperm(nb * bs, generator=g)[:T]
+    slots[3] = -1
+    kc = torch.full((2, nb, bs, H, D), 0x11, dtype=torch.uint8, device=dev)
+    ref = kc.cpu().numpy().copy()
+    codes_k = Q.fp8_codes(k.float().numpy(), scales[0]); codes_v = Q.fp8_codes(v.float().numpy(), scales[1])
+    for t, s in enumerate(slots.tolist()):
+        if s >= 0:
+            ref[0, s // bs, s % bs] = codes_k[t]; ref[1, s // bs, s % bs] = codes_v[t]
+    cache = kc.view(torch.float8_e4m3fn)
+    sb.ops.kv_append_fp8(k.to(dev), v.to(dev), cache[0], cache[1], slots.to(dev), *scales)
+    assert np.array_equal(kc.cpu().numpy(), ref)
+    name = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}[dtype]
+    got = sb.ops.fp8_round(k.to(dev), scales[0]).float().cpu().numpy()
+    assert np.array_equal(got, Q.fp8_round(k.float().numpy(), scales[0], name))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Hq,Hkv", [(28, 4), (16, 2)])
+@pytest.mark.parametrize("wl,n_split,scales", [(64, 1, (1.0, 1.0)), (100, 3, (0.25, 0.5)), (-1, 2, (1.0, 1.0))])
+def test_decode_over_fp8_cache_vs_oracle(sb, dev, dtype, Hq, Hkv, wl, n_split, scales):
+    bs = 16
+    lens = [1, 17, 64, 65, 300, 0, 129]
+    g = torch.Generator().manual_seed(Hq + wl)
+    need = [(n + bs - 1) // bs for n in lens]
+    nb = sum(need) + 3
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(len(lens), max(need), dtype=torch.int32)
+    p = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[p:p + n]; p += n
+    T = sum(lens)
+    k = torch.randn(T, Hkv, D, generator=g).to(dtype)
+    v = (torch.randn(T, Hkv, D, generator=g) * 1.5).to(dtype)
+    slots = torch.cat([torch.tensor([int(tables[b, i // bs]) * bs + i % bs for i in range(n)], dtype=torch.int64)
+                       for b, n in enumerate(lens)])
+    raw = torch.full((2, nb, bs, Hkv, D), 0x7F, dtype=torch.uint8, device=dev)      # every unwritten byte is a NaN code
+    cache = raw.view(torch.float8_e4m3fn)
+    sb.ops.kv_append_fp8(k.to(dev), v.to(dev), cache[0], cache[1], slots.to(dev), *scales)
+    kc = np.zeros((nb, bs, Hkv, D)); vc = np.zeros((nb, bs, Hkv, D))
+    kd = Q.fp8_values(Q.fp8_codes(k.float().numpy(), scales[0]), scales[0])
+    vd = Q.fp8_values(Q.fp8_codes(v.float().numpy(), scales[1]), scales[1])
+    for t, s in enumerate(slots.tolist()):
+        kc[s // bs, s % bs] = kd[t]; vc[s // bs, s % bs] = vd[t]
+    q = torch.randn(len(lens), Hq, D, generator=g).to(dtype)
+    scale = D ** -0.5
+    ref, ref_lse = A.paged_decode_attention(q.float().numpy(), kc, vc, tables.numpy(), lens, scale, wl, return_lse=True)
+    out, lse = sb.ops.swa_decode_attention(q.to(dev), cache[0], cache[1], torch.tensor(lens, dtype=torch.int32, device=dev),
+                                           block_table=tables.to(dev), window_left=wl, scale=scale, n_split=n_split,
+                                           fp8_scales=scales, return_lse=True)
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    live = [b for b, n in enumerate(lens) if n > 0]
+    ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+    assert (np.abs(got[live] - ref[live]) <= 2e-2 + ulp * np.abs(ref[live])).all()
+    assert np.abs(lse.cpu().numpy()[live] - ref_lse[live]).max() <= 2e-3
+    assert (got[5] == 0).all()

@@ -59,3 +59,18 @@ def test_append_layout():
     np.testing.assert_array_equal(kc[1, 1], c[0]); np.testing.assert_array_equal(ks[1, :, 1], s[0])
     np.testing.assert_array_equal(kc[3, 15], c[2]); np.testing.assert_array_equal(ks[3, :, 15], s[2])
     assert np.count_nonzero(ks) == 2 * H and np.count_nonzero(vs) == 2 * H
+
+
+def test_fp8_codes_known_values():
+    """e4m3fn by hand: 1 sign, 4 exponent (bias 7), 3 mantissa bits; largest finite 448 = 0x7e; subnormal
+    step 2^-9; ties to even; saturation instead of NaN beyond 464."""
+    x = np.array([0.0, 1.0, -1.0, 448.0, 1000.0, -1e9, 2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -9, 1.0625, 1.1875, 17.0, 0.1],
+                 np.float32)
+    codes = Q.fp8_codes(x, 1.0)
+    #                 0     1     -1    448   sat   -sat  min subnormal, tie->0, tie->2*2^-9, 1.0625->1.0, 1.1875->1.25, 17->16, 0.1
+    assert codes.tolist() == [0x00, 0x38, 0xB8, 0x7E, 0x7E, 0xFE, 0x01, 0x00, 0x02, 0x38, 0x3A, 0x58, 0x1D]
+    np.testing.assert_array_equal(Q.fp8_values(np.array([0x38, 0x7E, 0x01, 0x58], np.uint8), 2.0), [2.0, 896.0, 2.0 ** -8, 32.0])
+    # scale: codes of x / scale; the round trip is idempotent
+    y = Q.fp8_round(np.linspace(-30, 30, 64, dtype=np.float32), 0.25, "f32")
+    np.testing.assert_array_equal(Q.fp8_round(y, 0.25, "f32"), y)
+    assert np.isnan(Q.fp8_values(Q.fp8_codes(np.array([np.nan], np.float32), 1.0), 1.0)).all()
