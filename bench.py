@@ -246,7 +246,7 @@ def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None, gla_state_d
     by = c.bytes_per_step()
     gpu_ms = statistics.median(gpu)
     res = {"workload": f"BASELINE config 5: 28-layer hybrid decode step, B={B}, logical context 512k, "
-                       f"{steps} consecutive steps" + (", SWA K/V as per-row INT8" if kv_quant else "")
+                       f"{steps} consecutive steps" + ({"int8": ", SWA K/V as per-row INT8", "fp8": ", SWA K/V as fp8 (e4m3fn)"}.get(kv_quant, ""))
                        + (", GLA state stored as bf16" if gla_state_dtype == torch.bfloat16 else ""),
            "bytes_per_step": by,
            "host_stepped": {"ms_per_step": round(ms, 3), "decode_tok_per_s": round(B / (ms * 1e-3)),
@@ -286,7 +286,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
                                                     "28-layer hybrid decode step (config 5)")
-    ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "hybrid_lean", "gla_prompt"), default=None,
+    ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "hybrid_fp8", "hybrid_lean", "gla_prompt"), default=None,
                     help="run just that section and print its JSON (short runs for profiling one kernel)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -312,6 +312,9 @@ def main():
     if args.only == "hybrid_lean":
         print(json.dumps({"hybrid_decode_int8_kv_bf16_state": bench_hybrid(
             sb, dev, steps=min(args.steps, 128), kv_quant="int8", gla_state_dtype=torch.bfloat16)}))
+        return
+    if args.only == "hybrid_fp8":
+        print(json.dumps({"hybrid_decode_fp8_kv": bench_hybrid(sb, dev, steps=min(args.steps, 128), kv_quant="fp8")}))
         return
     if args.only == "hybrid_int8":
         print(json.dumps({"hybrid_decode_int8_kv": bench_hybrid(sb, dev, steps=min(args.steps, 128), kv_quant="int8")}))
@@ -426,6 +429,8 @@ def main():
         line["hybrid_decode"] = bench_hybrid(sb, dev)
         torch.cuda.empty_cache()
         line["hybrid_decode_int8_kv"] = bench_hybrid(sb, dev, kv_quant="int8")
+        torch.cuda.empty_cache()
+        line["hybrid_decode_fp8_kv"] = bench_hybrid(sb, dev, kv_quant="fp8")
         torch.cuda.empty_cache()
         # the storage formats of the reference's own variants: bf16 state cache (its serving path), INT8 K/V (W8ASpike)
         line["hybrid_decode_int8_kv_bf16_state"] = bench_hybrid(sb, dev, kv_quant="int8", gla_state_dtype=torch.bfloat16)

@@ -33,13 +33,15 @@ class HybridDecodeCache:
                  randomize: bool = False, seed: int = 0, kv_quant: Optional[str] = None,
                  gla_state_dtype: torch.dtype = torch.float32):
         """kv_quant="int8": the SWA layers keep their K/V as per-row INT8 codes + fp32 scales
-        (quantize_sym of W8ASpike/window_attention.py:227-237 applied once, at append time).
+        (quantize_sym of W8ASpike/window_attention.py:227-237 applied once, at append time);
+        kv_quant="fp8": as e4m3fn codes with per-tensor scales of 1 (the kv_cache_dtype="fp8" branch of
+        vllm_hymeta/attention/meta_attention.py:790-812).
         gla_state_dtype: float32, or bfloat16 as the reference's serving path keeps its state cache
         (vllm_hymeta/model_for_7B/modeling_gla_swa.py:361-364); the arithmetic is fp32 either way."""
         if gla_state_dtype not in (torch.float32, torch.bfloat16):
             raise ValueError("gla_state_dtype must be float32 or bfloat16")
-        if kv_quant not in (None, "int8"):
-            raise ValueError(f"kv_quant {kv_quant!r} (None or 'int8')")
+        if kv_quant not in (None, "int8", "fp8"):
+            raise ValueError(f"kv_quant {kv_quant!r} (None, 'int8' or 'fp8')")
         self.kv_quant = kv_quant
         self.device = torch.device(device)
         self.batch, self.num_layers = batch, num_layers
@@ -67,6 +69,13 @@ class HybridDecodeCache:
                     scales.uniform_(0.005, 0.03, generator=g)
                 self.kv_caches.append(codes)
                 self.kv_scales.append(scales)
+        elif kv_quant == "fp8":
+            self.kv_caches = []
+            for _ in self.swa_layers:
+                codes = torch.zeros(shape, dtype=torch.uint8, device=self.device)
+                if randomize:   # finite codes only: 0x7f / 0xff are NaN
+                    codes.random_(0, 0x7F, generator=g)
+                self.kv_caches.append(codes)
         else:
             self.kv_caches: List[torch.Tensor] = [alloc(shape, dtype, 1.0) for _ in self.swa_layers]
         # [n_gla_layers, slots, H, D, D] fp32, as vllm_hymeta/model_for_7B/modeling_gla_swa.py:348-356
@@ -154,13 +163,23 @@ class HybridDecodeCache:
                 q, codes[0], codes[1], meta.seq_lens_tensor[:n], block_table=meta.block_tables, window_left=self.wl,
                 scale=self.D ** -0.5, out=out, max_seq_len=meta.max_decode_seq_len or None,
                 k_scale=scales[0], v_scale=scales[1])
+        if self.kv_quant == "fp8":
+            codes = self.kv_caches[layer_idx // 2]
+            n = q.shape[0]
+            ops.kv_append_fp8(k, v, codes[0], codes[1], meta.slot_mapping.flatten()[:n], 1.0, 1.0)
+            return ops.swa_decode_attention(
+                q, codes[0], codes[1], meta.seq_lens_tensor[:n], block_table=meta.block_tables, window_left=self.wl,
+                scale=self.D ** -0.5, out=out, max_seq_len=meta.max_decode_seq_len or None, fp8_scales=(1.0, 1.0))
         return self.impl.forward(self._layer, q, k, v, None, None, None, self.kv_caches[layer_idx // 2], meta, out)
 
     def bytes_per_step(self) -> int:
         """Algorithmic HBM bytes of one decode step over all layers (window-saturated sequences)."""
         e = self._gla_out.element_size()
         n_keys = np.minimum(self.manager.n_tokens[:self.batch], self.wl + 1)
-        if self.kv_quant == "int8":     # per key and kv head: 2 x 128 code bytes + 2 fp32 scales; new row read in e, written as codes
+        if self.kv_quant == "fp8":      # per key and kv head: 2 x 128 code bytes
+            swa = int(n_keys.sum()) * self.Hkv * 2 * self.D + self.batch * (
+                2 * self.H * self.D * e + 2 * self.Hkv * self.D * e + self.Hkv * 2 * self.D)
+        elif self.kv_quant == "int8":   # per key and kv head: 2 x 128 code bytes + 2 fp32 scales; new row read in e, written as codes
             swa = int(n_keys.sum()) * self.Hkv * (2 * self.D + 8) + self.batch * (
                 2 * self.H * self.D * e + 2 * self.Hkv * self.D * e + self.Hkv * (2 * self.D + 8))
         else:

@@ -411,10 +411,14 @@ class MetaAttentionImpl:
         self.sliding_window = ((sliding_window - 1, 0) if sliding_window is not None else (-1, -1))
         self.kv_cache_dtype = kv_cache_dtype
         self.num_meta_tokens = num_meta_tokens
-        if kv_cache_dtype in _QUANTIZED_KV or kv_cache_dtype.startswith("fp8"):
+        # "fp8" / "fp8_e4m3": the cache tensor holds e4m3fn codes (uint8 or float8_e4m3fn, as the reference
+        # views it at :801-803) with the layer's per-tensor scales. (An INT8 cache is not a dtype string
+        # but an Int8KVCache object passed as kv_cache.)
+        if kv_cache_dtype in ("fp8_e5m2", "int8") or (kv_cache_dtype.startswith("fp8")
+                                                       and kv_cache_dtype not in ("fp8", "fp8_e4m3")):
             raise NotImplementedError(
                 f"MetaAttention does not support {self.kv_cache_dtype} kv-cache on this device "
-                "(FA supports fp8 = False).")
+                "(fp8 means e4m3fn here).")
         if logits_soft_cap is None:
             logits_soft_cap = 0
         if logits_soft_cap != 0:
@@ -446,8 +450,10 @@ class MetaAttentionImpl:
         assert output is not None, "Output tensor must be provided."
         if output_scale is not None:
             raise NotImplementedError("fused output quantization is not supported in MetaAttention.")
-        assert (getattr(layer, "_k_scale_float", 1.0) == 1.0 and getattr(layer, "_v_scale_float", 1.0) == 1.0), (
-            "key/v_scale is only supported in FlashAttention 3 with base dtype bfloat16")
+        fp8_kv = self.kv_cache_dtype.startswith("fp8")
+        k_scale_f, v_scale_f = float(getattr(layer, "_k_scale_float", 1.0)), float(getattr(layer, "_v_scale_float", 1.0))
+        assert fp8_kv or (k_scale_f == 1.0 and v_scale_f == 1.0), (
+            "key/v_scale is only supported with an fp8 kv-cache")
         attn_type = self.attn_type
         if attn_type == AttentionType.ENCODER and not attn_metadata.is_all_encoder_attn_metadata_set:
             raise AttributeError("Encoder attention requires setting encoder metadata attributes.")
@@ -483,14 +489,26 @@ class MetaAttentionImpl:
         # its slot. Every other step appends first, exactly as the reference does (:790-799).
         int8_kv = isinstance(kv_cache, Int8KVCache)
         scales = dict(k_scale=kv_cache.scales[0], v_scale=kv_cache.scales[1]) if int8_kv else {}
-        fuse_append = (kv_cache.numel() > 0 and key is not None and value is not None and not int8_kv
+        if fp8_kv:
+            if int8_kv:
+                raise ValueError("kv_cache_dtype says fp8 but the cache is an Int8KVCache")
+            scales = dict(fp8_scales=(k_scale_f, v_scale_f))
+            # queries take the fp8 round trip as well (scaled_fp8_quant with layer._q_scale, :806-811)
+            query = ops.fp8_round(query.contiguous(), float(getattr(layer, "_q_scale_float", 1.0)))
+        byte_kv = int8_kv or fp8_kv
+        fuse_append = (kv_cache.numel() > 0 and key is not None and value is not None and not byte_kv
                        and attn_metadata.num_prefill_tokens == 0 and attn_metadata.num_decode_tokens > 0
                        and (attn_metadata.max_decode_query_len or 1) == 1
                        and query.dtype in (torch.bfloat16, torch.float16)
                        and attn_metadata.slot_mapping is not None)
         if kv_cache.numel() > 0:
             key_cache, value_cache = (kv_cache.codes[0], kv_cache.codes[1]) if int8_kv else (kv_cache[0], kv_cache[1])
-            if key is not None and value is not None and int8_kv:
+            if fp8_kv and key_cache.dtype not in (torch.uint8, torch.float8_e4m3fn):
+                raise ValueError(f"an fp8 kv-cache must be a uint8 or float8_e4m3fn tensor, got {key_cache.dtype}")
+            if key is not None and value is not None and fp8_kv:
+                ops.kv_append_fp8(key, value, key_cache, value_cache, attn_metadata.slot_mapping.flatten(),
+                                  k_scale_f, v_scale_f)
+            elif key is not None and value is not None and int8_kv:
                 # rows are quantised on their way in: 128 code bytes + one scale per (token, kv head)
                 ops.kv_append_int8(key, value, key_cache, value_cache, scales["k_scale"], scales["v_scale"],
                                    attn_metadata.slot_mapping.flatten())
@@ -527,6 +545,8 @@ class MetaAttentionImpl:
                 pk, pv = key[:num_prefill_query_tokens], value[:num_prefill_query_tokens]
                 if int8_kv:   # attend to what the cache will hold: the rows as quantize_sym returns them
                     pk, pv = ops.quantize_sym(pk), ops.quantize_sym(pv)
+                elif fp8_kv:  # scaled_fp8_quant of the prompt's keys and values (:853-869)
+                    pk, pv = ops.fp8_round(pk.contiguous(), k_scale_f), ops.fp8_round(pv.contiguous(), v_scale_f)
                 lse = self._varlen_inflight(query, pk, pv, prefill_meta, prefill_output, window_left,
                                             return_lse=with_meta)
             else:
@@ -566,7 +586,7 @@ class MetaAttentionImpl:
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
                     out=decode_output, return_lse=with_meta,
                     max_seq_len=decode_meta.max_decode_seq_len or None,
-                    balanced=False if int8_kv else decode_meta._decode_balanced, **scales, **fused)
+                    balanced=False if byte_kv else decode_meta._decode_balanced, **scales, **fused)
                 lse = res[1] if with_meta else None
             merge_meta(decode_query, decode_output, lse)
         return output

@@ -182,4 +182,4 @@ def test_profile_run_and_errors(sb, dev):
     with pytest.raises(NotImplementedError, match="KV sharing"):
         sb.MetaAttentionImpl(HQ, D, 1.0, HKV, None, 65, "auto", kv_sharing_target_layer_name="x")
     with pytest.raises(NotImplementedError, match="kv-cache"):
-        sb.MetaAttentionImpl(HQ, D, 1.0, HKV, None, 65, "fp8")
+        sb.MetaAttentionImpl(HQ, D, 1.0, HKV, None, 65, "fp8_e5m2")

@@ -287,3 +287,61 @@ def test_decode_over_fp8_cache_vs_oracle(sb, dev, dtype, Hq, Hkv, wl, n_split, s
     assert (np.abs(got[live] - ref[live]) <= 2e-2 + ulp * np.abs(ref[live])).all()
     assert np.abs(lse.cpu().numpy()[live] - ref_lse[live]).max() <= 2e-3
     assert (got[5] == 0).all()
+
+
+def test_backend_engine_with_fp8_cache(sb, dev):
+    """kv_cache_dtype="fp8" through MetaAttentionImpl.forward with layer scales: codes bit-exact against
+    the oracle's fp8 append at the oracle's slots; outputs within 2e-2 of attention computed from the
+    query, keys and values after their fp8 round trips (the reference quantises all three)."""
+    from oracle import paged as P
+    HQ, HKV, bs, wl, nb = 28, 4, 16, 40, 48
+    runner = sb.runner.SwaCacheRunner(1, nb, bs, wl, HKV, D, torch.uint8, dev, max_seqs=3, max_chunk_tokens=128)
+    impl = sb.MetaAttentionImpl(HQ, D, D ** -0.5, HKV, None, wl + 1, "fp8")
+
+    class Layer:
+        _k_scale_float, _v_scale_float, _q_scale_float = 0.5, 0.25, 0.125
+
+    ks, vs, qs = Layer._k_scale_float, Layer._v_scale_float, Layer._q_scale_float
+    model = P.WindowCacheModel(nb, bs, wl)
+    kc = np.zeros((nb, bs, HKV, D), np.uint8); vc = np.zeros_like(kc)
+    hist = {}
+    g = torch.Generator().manual_seed(12)
+
+    def step(prompts, decodes, chunked=False):
+        T = sum(n for _, n in prompts) + len(decodes)
+        q = torch.randn(T, HQ, D, generator=g).bfloat16()
+        k = torch.randn(T, HKV, D, generator=g).bfloat16()
+        v = torch.randn(T, HKV, D, generator=g).bfloat16()
+        meta = runner.build_step(prompts, decodes, chunked_prefill=chunked)
+        slots = []
+        for sid, n in prompts:
+            slots += model.append_tokens(sid, n, True, store_all=chunked)
+        for sid in decodes:
+            slots += model.append_tokens(sid, 1, False)
+        ck, cv = Q.fp8_codes(k.float().numpy(), ks), Q.fp8_codes(v.float().numpy(), vs)
+        for t, s in enumerate(slots):
+            if s >= 0:
+                kc[s // bs, s % bs] = ck[t]; vc[s // bs, s % bs] = cv[t]
+        out = torch.full((T, HQ, D), float("nan"), dtype=torch.bfloat16, device=dev)
+        impl.forward(Layer(), q.to(dev), k.to(dev), v.to(dev), None, None, None, runner.kv_caches[0], meta, output=out)
+        assert np.array_equal(runner.kv_caches[0][0].cpu().numpy(), kc) and np.array_equal(runner.kv_caches[0][1].cpu().numpy(), vc)
+        got = out.float().cpu().numpy()
+        qr = Q.fp8_round(q.float().numpy(), qs, "bf16")
+        t = 0
+        for sid, n in list(prompts) + [(s, 1) for s in decodes]:
+            hk, hv = hist.get(sid, (np.zeros((0, HKV, D), np.float32), np.zeros((0, HKV, D), np.float32)))
+            hk = np.concatenate([hk, Q.fp8_round(k[t:t + n].float().numpy(), ks, "f32")])
+            hv = np.concatenate([hv, Q.fp8_round(v[t:t + n].float().numpy(), vs, "f32")])
+            hist[sid] = (hk, hv)
+            ref = A.varlen_window_attention(qr[t:t + n], hk, hv, [0, n], [0, len(hk)], D ** -0.5, wl)
+            assert np.abs(got[t:t + n] - ref).max() <= 2e-2 + 2.0 ** -8 * np.abs(ref).max(), (sid, n)
+            t += n
+
+    for sid in (0, 1, 2):
+        runner.add_seq(sid); model.add_seq(sid)
+    step([(0, 25), (1, 90)], [])
+    step([(2, 50)], [0, 1], chunked=True)
+    for _ in range(bs + 3):
+        step([], [0, 1, 2])
+    with pytest.raises(NotImplementedError):
+        sb.MetaAttentionImpl(HQ, D, D ** -0.5, HKV, None, wl + 1, "fp8_e5m2")
