@@ -309,6 +309,13 @@ typedef struct sb_swa_prefill_args {
   void *stream;
   float *lse;      /* optional, fp32 [total_q, Hq], natural log: log-sum-exp of each query's scaled scores,
                       the second result of _flash_attn_varlen_forward that fa_kernel_metatoken.py:254-257 merges on */
+  /* byte-code paged caches, as for sb_swa_decode: kv_quant = SB_KV_INT8 with k_scale / v_scale, or
+   * SB_KV_FP8 with k_scale_tensor / v_scale_tensor; k/v then hold codes and the kv strides are bytes.
+   * Rows are dequantised (code * scale, rounded to dtype) on their way into the kernel's LDS stage. */
+  const float *k_scale;
+  const float *v_scale;
+  int32_t kv_quant;
+  float k_scale_tensor, v_scale_tensor;
 } sb_swa_prefill_args;
 
 int sb_swa_prefill(const sb_swa_prefill_args *args);

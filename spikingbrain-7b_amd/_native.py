@@ -96,7 +96,8 @@ class SwaPrefillArgs(C.Structure):
         ("out_stride_row", i64), ("out_stride_head", i64),
         ("kv_stride_block", i64), ("kv_stride_row", i64), ("kv_stride_head", i64),
         ("block_table_stride", i64),
-        ("stream", vp), ("lse", vp),
+        ("stream", vp), ("lse", vp), ("k_scale", vp), ("v_scale", vp), ("kv_quant", i32),
+        ("k_scale_tensor", f32), ("v_scale_tensor", f32),
     ]
 
 

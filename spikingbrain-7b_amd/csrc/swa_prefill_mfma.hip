@@ -41,6 +41,11 @@ struct PrefillParams {
   const char *v;
   char *out;
   float *lse;                 // [total_q, Hq] natural-log log-sum-exp, or null
+  // byte-code caches (paged): per-row INT8 scales [nb, Hkv, bs], or one fp8 scale per tensor
+  const float *k_scale;
+  const float *v_scale;
+  float k_scale_tensor, v_scale_tensor;
+  int Hkv;
   const int32_t *block_table;
   const int64_t *kv_start;
   const int32_t *key_lo;      // [S] first visible key of each sequence, or null
@@ -74,7 +79,38 @@ struct Shape {
   static constexpr int kLoads = 8 / kFetchWaves;                // 4-row loads per fetching lane, per K and per V
 };
 
-template <typename E, int NHEADS>
+// The registers a fetching lane carries a chunk in: 16-byte pieces of K and V rows, or, for a byte-code
+// cache (KVQ = SB_KV_INT8 / SB_KV_FP8), the 8 codes that become such a piece plus (INT8) their row's scales.
+template <int KVQ, int N>
+struct StageSet {
+  uint4 k[N], v[N];
+};
+template <int N>
+struct StageSet<SB_KV_INT8, N> {
+  uint2 k[N], v[N];
+  float ks[N], vs[N];
+};
+template <int N>
+struct StageSet<SB_KV_FP8, N> {
+  uint2 k[N], v[N];
+};
+
+template <int Q, int B>
+__device__ __forceinline__ float code_value(uint32_t w) {
+  if constexpr (Q == SB_KV_INT8) return (float)(int)(int8_t)(w >> (8 * B));
+  else return __builtin_amdgcn_cvt_f32_fp8((int)w, B);
+}
+// 8 codes times their scale, rounded to E: the values the reference attends to after its own
+// quantise-dequantise (code * scale cast back to the tensor's dtype)
+template <typename E, int Q>
+__device__ __forceinline__ uint4 dequant8(uint2 w, float s) {
+  return make_uint4(Mma<E>::pack(code_value<Q, 0>(w.x) * s, code_value<Q, 1>(w.x) * s),
+                    Mma<E>::pack(code_value<Q, 2>(w.x) * s, code_value<Q, 3>(w.x) * s),
+                    Mma<E>::pack(code_value<Q, 0>(w.y) * s, code_value<Q, 1>(w.y) * s),
+                    Mma<E>::pack(code_value<Q, 2>(w.y) * s, code_value<Q, 3>(w.y) * s));
+}
+
+template <typename E, int NHEADS, int KVQ>
 __global__ __attribute__((amdgpu_flat_work_group_size(64 * Shape<NHEADS>::kWaves, 64 * Shape<NHEADS>::kWaves),
                           amdgpu_waves_per_eu(2, 2)))
 void swa_prefill_kernel(const PrefillParams p) {
@@ -152,11 +188,13 @@ void swa_prefill_kernel(const PrefillParams p) {
   const bool paged = p.block_table != nullptr;
   const int64_t dense_row0 = (!paged && p.kv_start) ? p.kv_start[seq] : 0;
   const int64_t head_off = (int64_t)kvh * p.kv_sh;
+  int64_t scale_base = 0;  // INT8: index of the tile's first row in the scale tensors (set by tile_base)
   auto tile_base = [&](int t) -> int64_t {  // t inside [first_tile, last_tile], wave-uniform
     const int i0 = t << 4;
     if (paged) {
       const int bi = i0 / p.block_size;
       const int64_t blk = p.block_table[(int64_t)seq * p.bt_stride + bi];
+      if constexpr (KVQ == SB_KV_INT8) scale_base = (blk * p.Hkv + kvh) * p.block_size + (i0 - bi * p.block_size);
       return blk * p.kv_sb + (int64_t)(i0 - bi * p.block_size) * p.kv_sr + head_off;
     }
     return (dense_row0 + i0) * p.kv_sr + head_off;
@@ -168,25 +206,49 @@ void swa_prefill_kernel(const PrefillParams p) {
   const bool fetcher = wave < S::kFetchWaves;
   const int rows_per_wave = 32 / S::kFetchWaves;                         // 8 or 16
   const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the 16-key tile, +4 per load
-  uint4 stage_k[2][S::kLoads], stage_v[2][S::kLoads];  // chunk x travels in set (x - ch_begin) & 1
-  auto fetch = [&](int ch, uint4 (&sk_)[S::kLoads], uint4 (&sv_)[S::kLoads]) {
+  using Set = StageSet<KVQ, S::kLoads>;
+  Set stage[2];  // chunk x travels in set (x - ch_begin) & 1
+  auto fetch = [&](int ch, Set &st) {
     const int t = min(max(2 * ch + (wave * rows_per_wave) / 16, first_tile), last_tile);
     const int64_t base = tile_base(t);
 #pragma unroll
     for (int u = 0; u < S::kLoads; ++u) {
       const int row = min(max((t << 4) + lrow + 4 * u, wg_lo), wg_hi - 1) - (t << 4);
-      const int64_t off = base + (int64_t)row * p.kv_sr + c * 16;
-      sk_[u] = load_stream16(p.k + off);
-      sv_[u] = load_stream16(p.v + off);
+      if constexpr (KVQ == SB_KV_NONE) {
+        const int64_t off = base + (int64_t)row * p.kv_sr + c * 16;
+        st.k[u] = load_stream16(p.k + off);
+        st.v[u] = load_stream16(p.v + off);
+      } else {  // a row is 128 code bytes: 8 per lane
+        const int64_t off = base + (int64_t)row * p.kv_sr + c * 8;
+        const unsigned long long wk = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(p.k + off));
+        const unsigned long long wv = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(p.v + off));
+        st.k[u] = make_uint2((uint32_t)wk, (uint32_t)(wk >> 32));
+        st.v[u] = make_uint2((uint32_t)wv, (uint32_t)(wv >> 32));
+        if constexpr (KVQ == SB_KV_INT8) {
+          st.ks[u] = p.k_scale[scale_base + row];
+          st.vs[u] = p.v_scale[scale_base + row];
+        }
+      }
     }
   };
-  auto stash = [&](int buf, const uint4 (&sk_)[S::kLoads], const uint4 (&sv_)[S::kLoads]) {
+  auto stash = [&](int buf, const Set &st) {
     char *sk = smem + buf * 2 * kStage, *sv = sk + kStage;
 #pragma unroll
     for (int u = 0; u < S::kLoads; ++u) {
       const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
-      *reinterpret_cast<uint4 *>(sk + kk * kRowPad + c * 16) = sk_[u];
-      *reinterpret_cast<uint4 *>(sv + kk * kRowPad + c * 16) = sv_[u];
+      uint4 kq, vq;
+      if constexpr (KVQ == SB_KV_NONE) {
+        kq = st.k[u];
+        vq = st.v[u];
+      } else if constexpr (KVQ == SB_KV_INT8) {
+        kq = dequant8<E, KVQ>(st.k[u], st.ks[u]);
+        vq = dequant8<E, KVQ>(st.v[u], st.vs[u]);
+      } else {
+        kq = dequant8<E, KVQ>(st.k[u], p.k_scale_tensor);
+        vq = dequant8<E, KVQ>(st.v[u], p.v_scale_tensor);
+      }
+      *reinterpret_cast<uint4 *>(sk + kk * kRowPad + c * 16) = kq;
+      *reinterpret_cast<uint4 *>(sv + kk * kRowPad + c * 16) = vq;
     }
   };
 
@@ -291,16 +353,16 @@ void swa_prefill_kernel(const PrefillParams p) {
   // counts exactly the loads that may still be in flight.
   auto body = [&](int x, auto par) {
     constexpr int P = decltype(par)::value;
-    if (fetcher) fetch(x + 2, stage_k[P], stage_v[P]);
+    if (fetcher) fetch(x + 2, stage[P]);
     if (scores(x, P)) rescale();
     accumulate(P);
-    if (fetcher) stash(P ^ 1, stage_k[P ^ 1], stage_v[P ^ 1]);
+    if (fetcher) stash(P ^ 1, stage[P ^ 1]);
     __syncthreads();
   };
   if (fetcher) {
-    fetch(ch_begin, stage_k[0], stage_v[0]);
-    fetch(ch_begin + 1, stage_k[1], stage_v[1]);
-    stash(0, stage_k[0], stage_v[0]);
+    fetch(ch_begin, stage[0]);
+    fetch(ch_begin + 1, stage[1]);
+    stash(0, stage[0]);
   }
   __syncthreads();
   int ch = ch_begin;
@@ -336,14 +398,20 @@ void swa_prefill_kernel(const PrefillParams p) {
   }
 }
 
-template <typename E>
-void launch_prefill(int nh, dim3 grid, hipStream_t st, const PrefillParams &p) {
+template <typename E, int KVQ>
+void launch_prefill_q(int nh, dim3 grid, hipStream_t st, const PrefillParams &p) {
   switch (nh) {
-    case 1: hipLaunchKernelGGL((swa_prefill_kernel<E, 1>), grid, dim3(64 * Shape<1>::kWaves), 0, st, p); break;
-    case 2: hipLaunchKernelGGL((swa_prefill_kernel<E, 2>), grid, dim3(64 * Shape<2>::kWaves), 0, st, p); break;
-    case 3: hipLaunchKernelGGL((swa_prefill_kernel<E, 3>), grid, dim3(64 * Shape<3>::kWaves), 0, st, p); break;
-    default: hipLaunchKernelGGL((swa_prefill_kernel<E, 4>), grid, dim3(64 * Shape<4>::kWaves), 0, st, p); break;
+    case 1: hipLaunchKernelGGL((swa_prefill_kernel<E, 1, KVQ>), grid, dim3(64 * Shape<1>::kWaves), 0, st, p); break;
+    case 2: hipLaunchKernelGGL((swa_prefill_kernel<E, 2, KVQ>), grid, dim3(64 * Shape<2>::kWaves), 0, st, p); break;
+    case 3: hipLaunchKernelGGL((swa_prefill_kernel<E, 3, KVQ>), grid, dim3(64 * Shape<3>::kWaves), 0, st, p); break;
+    default: hipLaunchKernelGGL((swa_prefill_kernel<E, 4, KVQ>), grid, dim3(64 * Shape<4>::kWaves), 0, st, p); break;
   }
+}
+template <typename E>
+void launch_prefill(int kv_quant, int nh, dim3 grid, hipStream_t st, const PrefillParams &p) {
+  if (kv_quant == SB_KV_INT8) launch_prefill_q<E, SB_KV_INT8>(nh, grid, st, p);
+  else if (kv_quant == SB_KV_FP8) launch_prefill_q<E, SB_KV_FP8>(nh, grid, st, p);
+  else launch_prefill_q<E, SB_KV_NONE>(nh, grid, st, p);
 }
 
 }  // namespace
@@ -366,11 +434,23 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
     return fail(SB_ERR_INVALID, "sb_swa_prefill: block_size %d must be a multiple of 16", a->block_size);
   if (a->num_tiles > 0x7ffffff0LL || a->num_kv_heads > 65535)
     return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: grid too large");
-  const int64_t es[] = {a->q_stride_row, a->q_stride_head, a->out_stride_row, a->out_stride_head,
-                        a->kv_stride_block, a->kv_stride_row, a->kv_stride_head};
+  const bool codes = a->kv_quant == SB_KV_INT8 || a->kv_quant == SB_KV_FP8;
+  if (a->kv_quant != SB_KV_NONE && !codes)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: unknown kv_quant %d", a->kv_quant);
+  if (codes && !a->block_table) return fail(SB_ERR_INVALID, "sb_swa_prefill: a byte-code cache needs paged mode");
+  if (a->kv_quant == SB_KV_INT8 && (!a->k_scale || !a->v_scale))
+    return fail(SB_ERR_INVALID, "sb_swa_prefill: the INT8 cache needs both scale tensors");
+  if (a->kv_quant == SB_KV_FP8 && (!(a->k_scale_tensor > 0.f) || !(a->v_scale_tensor > 0.f)))
+    return fail(SB_ERR_INVALID, "sb_swa_prefill: the fp8 cache needs positive k_scale_tensor and v_scale_tensor");
+  const int kv_esz = codes ? 1 : 2;
+  const int64_t es[] = {a->q_stride_row, a->q_stride_head, a->out_stride_row, a->out_stride_head};
   for (int64_t s : es)
     if ((s * 2) % 16 != 0)
       return fail(SB_ERR_INVALID, "sb_swa_prefill: stride %lld elements is not 16-byte aligned", (long long)s);
+  const int64_t kes[] = {a->kv_stride_block, a->kv_stride_row, a->kv_stride_head};
+  for (int64_t s : kes)
+    if ((s * kv_esz) % 16 != 0)
+      return fail(SB_ERR_INVALID, "sb_swa_prefill: cache stride %lld elements is not 16-byte aligned", (long long)s);
   if ((reinterpret_cast<uintptr_t>(a->q) | reinterpret_cast<uintptr_t>(a->k) | reinterpret_cast<uintptr_t>(a->v) |
        reinterpret_cast<uintptr_t>(a->out)) & 15u)
     return fail(SB_ERR_INVALID, "sb_swa_prefill: q/k/v/out base not 16-byte aligned");
@@ -384,7 +464,9 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   p.block_size = a->block_size > 0 ? a->block_size : 16; p.window_left = a->window_left;
   p.scale_log2 = a->scale * sb::kLog2e;
   p.q_sr = a->q_stride_row; p.q_sh = a->q_stride_head; p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
-  p.kv_sb = a->kv_stride_block * 2; p.kv_sr = a->kv_stride_row * 2; p.kv_sh = a->kv_stride_head * 2;
+  p.kv_sb = a->kv_stride_block * kv_esz; p.kv_sr = a->kv_stride_row * kv_esz; p.kv_sh = a->kv_stride_head * kv_esz;
+  p.k_scale = a->k_scale; p.v_scale = a->v_scale;
+  p.k_scale_tensor = a->k_scale_tensor; p.v_scale_tensor = a->v_scale_tensor; p.Hkv = a->num_kv_heads;
   p.bt_stride = a->block_table_stride;
   p.num_tiles = (int)a->num_tiles;
 
@@ -392,8 +474,8 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   for (int h0 = 0; h0 < p.G; h0 += 4) {  // a GQA group is covered 4 heads at a time
     p.head_begin = h0;
     const int nh = p.G - h0 < 4 ? p.G - h0 : 4;
-    if (a->dtype == SB_BF16) launch_prefill<BF16>(nh, grid, (hipStream_t)a->stream, p);
-    else launch_prefill<F16>(nh, grid, (hipStream_t)a->stream, p);
+    if (a->dtype == SB_BF16) launch_prefill<BF16>(a->kv_quant, nh, grid, (hipStream_t)a->stream, p);
+    else launch_prefill<F16>(a->kv_quant, nh, grid, (hipStream_t)a->stream, p);
     const int rc = check_launch("swa_prefill_kernel");
     if (rc != SB_OK) return rc;
   }

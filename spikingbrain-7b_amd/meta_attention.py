@@ -638,16 +638,17 @@ class MetaAttentionImpl:
 
     def _varlen_paged(self, q, key_cache, value_cache, query_start_loc, seq_lens_tensor, block_tables,
                       max_seq_len, out, window_left, meta=None, return_lse=False, scales=None):
-        """scales (k_scale, v_scale of an INT8 cache): every query token runs as one row of the
-        single-query kernel, the only one that reads that cache form."""
+        """scales: k_scale/v_scale of an INT8 cache or fp8_scales of an fp8 cache, passed on to whichever
+        kernel takes the step."""
         T = q.shape[0]
         if T == 0:
             return None
         scales = scales or {}
-        plan = self._plan_for(meta, q) if meta is not None and not scales else None
+        plan = self._plan_for(meta, q) if meta is not None else None
         if plan is not None and block_tables.shape[1] * key_cache.shape[1] >= plan.max_k:
             res = ops.swa_prefill_attention(q, key_cache, value_cache, plan=plan, block_table=block_tables,
-                                            window_left=window_left, scale=self.scale, out=out, return_lse=return_lse)
+                                            window_left=window_left, scale=self.scale, out=out, return_lse=return_lse,
+                                            **scales)
             return res[1] if return_lse else None
         row_seq, j, lens = self._rows(query_start_loc, T)
         # query j of a run of n queries in a sequence of L keys sits at key index L - n + j

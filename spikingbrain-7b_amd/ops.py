@@ -416,6 +416,9 @@ def swa_prefill_attention(
     scale: Optional[float] = None,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = False,
+    k_scale: Optional[torch.Tensor] = None,
+    v_scale: Optional[torch.Tensor] = None,
+    fp8_scales: Optional[Tuple[float, float]] = None,
 ):
     """Causal sliding-window attention for q [total_q, Hq, D] packed sequence after sequence.
     With return_lse also the fp32 [total_q, Hq] natural-log log-sum-exp of each query's scores.
@@ -428,13 +431,26 @@ def swa_prefill_attention(
     With kv_strides = (row, head) in elements (and num_kv_heads), k/v may be any tensors whose
     element offset for (sequence s, key i, head h) is (kv_start[s] + i)*row + h*head.
     key_lo [S] int32: keys below key_lo[s] are invisible (left padding); a query that sees no key
-    gets zeros."""
-    dev = N.require_gpu(q, k, v, block_table, kv_start, key_lo, out)
+    gets zeros.
+    k_scale/v_scale (INT8 codes) or fp8_scales (e4m3fn codes): the paged caches are byte codes as
+    kv_append_int8 / kv_append_fp8 wrote them; rows are dequantised on their way into the kernel."""
+    dev = N.require_gpu(q, k, v, block_table, kv_start, key_lo, out, k_scale, v_scale)
+    kv_quant = N.SB_KV_NONE
+    if fp8_scales is not None:
+        if block_table is None or k.dtype not in (torch.float8_e4m3fn, torch.uint8) or v.dtype != k.dtype:
+            raise ValueError("fp8_scales needs paged float8_e4m3fn (or uint8) caches")
+        if k.dtype != torch.uint8:
+            k, v = k.view(torch.uint8), v.view(torch.uint8)
+        kv_quant = N.SB_KV_FP8
+    elif k_scale is not None or v_scale is not None:
+        if k_scale is None or v_scale is None or block_table is None or k.dtype != torch.int8 or v.dtype != torch.int8:
+            raise ValueError("k_scale and v_scale go together, with paged int8 caches")
+        kv_quant = N.SB_KV_INT8
     if q.dim() != 3:
         raise ValueError(f"q must be [total_q, num_heads, head_size], got {tuple(q.shape)}")
     Tq, Hq, D = q.shape
     _inner_contiguous(q, "q")
-    if k.dtype != q.dtype or v.dtype != q.dtype:
+    if kv_quant == N.SB_KV_NONE and (k.dtype != q.dtype or v.dtype != q.dtype):
         raise ValueError("q, k and v must share one dtype")
     if plan is None:
         if query_lens is None:
@@ -455,6 +471,10 @@ def swa_prefill_attention(
             raise ValueError("block_table must be a 2-D int32 tensor with contiguous rows, one per sequence")
         if block_table.shape[1] * bs < plan.max_k:
             raise ValueError(f"block_table rows hold {block_table.shape[1] * bs} keys, a sequence has {plan.max_k}")
+        if kv_quant == N.SB_KV_INT8:
+            for t, name in ((k_scale, "k_scale"), (v_scale, "v_scale")):
+                if t.shape != (nb, Hkv, bs) or t.dtype != torch.float32 or not t.is_contiguous():
+                    raise ValueError(f"{name} must be a contiguous float32 [num_blocks, num_kv_heads, block_size] tensor")
         bt_stride = block_table.stride(0)
     else:
         bs, bt_stride = 16, 0
@@ -502,7 +522,10 @@ def swa_prefill_attention(
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
         kv_stride_block=strides[0], kv_stride_row=strides[1], kv_stride_head=strides[2],
-        block_table_stride=bt_stride, stream=N.stream_ptr(dev), lse=N.ptr(lse))
+        block_table_stride=bt_stride, stream=N.stream_ptr(dev), lse=N.ptr(lse),
+        k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale), kv_quant=kv_quant,
+        k_scale_tensor=float(fp8_scales[0]) if fp8_scales is not None else 0.0,
+        v_scale_tensor=float(fp8_scales[1]) if fp8_scales is not None else 0.0)
     N.check(N.lib().sb_swa_prefill(C.byref(a)), "swa_prefill")
     return (out, lse) if return_lse else out
 

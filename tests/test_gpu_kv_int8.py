@@ -345,3 +345,46 @@ def test_backend_engine_with_fp8_cache(sb, dev):
         step([], [0, 1, 2])
     with pytest.raises(NotImplementedError):
         sb.MetaAttentionImpl(HQ, D, D ** -0.5, HKV, None, wl + 1, "fp8_e5m2")
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+@pytest.mark.parametrize("Hq,Hkv", [(28, 4), (8, 8)])
+def test_prefill_kernel_over_byte_code_caches(sb, dev, kind, Hq, Hkv):
+    """Chunked prefill reading an INT8 / fp8 paged cache with the many-query kernel: rows are
+    dequantised into the kernel's LDS stage; compared with the oracle's attention over the rows as the
+    reference's quantise-dequantise leaves them (code * scale rounded to bf16)."""
+    bs, wl = 16, 70
+    qlens, klens = [40, 5, 130], [100, 5, 230]           # second and third chunks of prompts, one whole short prompt
+    g = torch.Generator().manual_seed(31)
+    need = [(n + bs - 1) // bs for n in klens]
+    nb = sum(need) + 2
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(len(klens), max(need), dtype=torch.int32)
+    p = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[p:p + n]; p += n
+    Tk, Tq = sum(klens), sum(qlens)
+    k = (torch.randn(Tk, Hkv, D, generator=g) * (0.5 + torch.rand(Tk, Hkv, 1, generator=g))).bfloat16()
+    v = (torch.randn(Tk, Hkv, D, generator=g) * (1 + torch.rand(Tk, Hkv, 1, generator=g))).bfloat16()
+    q = torch.randn(Tq, Hq, D, generator=g).bfloat16()
+    slots = torch.cat([torch.tensor([int(tables[b, i // bs]) * bs + i % bs for i in range(n)], dtype=torch.int64)
+                       for b, n in enumerate(klens)])
+    if kind == "int8":
+        kv, sc = sb.ops.alloc_int8_kv_cache(nb, bs, Hkv, D, dev)
+        sc.fill_(float("nan"))
+        sb.ops.kv_append_int8(k.to(dev), v.to(dev), kv[0], kv[1], sc[0], sc[1], slots.to(dev))
+        kw = dict(k_scale=sc[0], v_scale=sc[1])
+        kd, vd = Q.quantize_sym(k.float().numpy(), "bf16"), Q.quantize_sym(v.float().numpy(), "bf16")
+    else:
+        raw = torch.full((2, nb, bs, Hkv, D), 0x7F, dtype=torch.uint8, device=dev)
+        kv = raw.view(torch.float8_e4m3fn)
+        sb.ops.kv_append_fp8(k.to(dev), v.to(dev), kv[0], kv[1], slots.to(dev), 0.5, 0.25)
+        kw = dict(fp8_scales=(0.5, 0.25))
+        kd, vd = Q.fp8_round(k.float().numpy(), 0.5, "bf16"), Q.fp8_round(v.float().numpy(), 0.25, "bf16")
+    out, lse = sb.ops.swa_prefill_attention(q.to(dev), kv[0], kv[1], query_lens=qlens, seq_lens_k=klens,
+                                            block_table=tables.to(dev), window_left=wl, return_lse=True, **kw)
+    cu_q = np.concatenate([[0], np.cumsum(qlens)]); cu_k = np.concatenate([[0], np.cumsum(klens)])
+    ref = A.varlen_window_attention(q.float().numpy(), kd, vd, cu_q, cu_k, D ** -0.5, wl)
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any() and not torch.isnan(lse).any()
+    assert (np.abs(got - ref) <= 2e-2 + 2.0 ** -8 * np.abs(ref)).all()
