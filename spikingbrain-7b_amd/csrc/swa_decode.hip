@@ -307,17 +307,35 @@ __global__ __launch_bounds__(128) void swa_decode_merge_kernel(const DecodeParam
   const int hq = (int)(rh - r * p.Hq);
   const int d = threadIdx.x;
   const float *ml = p.ws_ml + rh * p.n_split * 2;
-  float M = kNegInf;
-  for (int s = 0; s < p.n_split; ++s) M = fmaxf(M, ml[2 * s]);
-  float tot = 0.f, L = 0.f;
-  if (M != kNegInf) {
-    const float *acc = p.ws_acc + rh * p.n_split * 128 + d;
-    for (int s = 0; s < p.n_split; ++s) {
-      const float ms = ml[2 * s];
-      const float f = (ms == kNegInf) ? 0.f : fast_exp2(ms - M);
-      tot = fmaf(acc[(int64_t)s * 128], f, tot);
-      L = fmaf(ml[2 * s + 1], f, L);
+  const float *acc = p.ws_acc + rh * p.n_split * 128 + d;
+  // Four splits per trip, every load of a trip issued before any is used: with the usual split counts
+  // the kernel is one round trip to memory. Across trips the running sums are rescaled to the new maximum.
+  float tot = 0.f, L = 0.f, M = kNegInf;
+  for (int s0 = 0; s0 < p.n_split; s0 += 4) {
+    float ms[4], ls[4], av[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int s = min(s0 + j, p.n_split - 1);
+      ms[j] = ml[2 * s];
+      ls[j] = ml[2 * s + 1];
+      av[j] = acc[(int64_t)s * 128];
     }
+    float Mn = M;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (s0 + j < p.n_split) Mn = fmaxf(Mn, ms[j]);
+    if (Mn != kNegInf) {
+      const float keep = (M == kNegInf) ? 0.f : fast_exp2(M - Mn);
+      tot *= keep;
+      L *= keep;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float f = (s0 + j >= p.n_split || ms[j] == kNegInf) ? 0.f : fast_exp2(ms[j] - Mn);
+        tot = fmaf(av[j], f, tot);
+        L = fmaf(ls[j], f, L);
+      }
+    }
+    M = Mn;
   }
   store_out<E>(p.out, r * p.o_sr + (int64_t)hq * p.o_sh + d, L > 0.f ? tot / L : 0.f);
   if (d == 0 && p.lse) p.lse[rh] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
