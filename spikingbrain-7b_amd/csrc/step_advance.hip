@@ -41,6 +41,8 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
   __shared__ int s_alloc[kRowsPerPass];      // logical block it allocates, -1 = none
   __shared__ int s_newid[kRowsPerPass];      // physical id that block got
   __shared__ int s_cache[kTopCache];         // stack entries [cache_base, cache_base + cache_n)
+  __shared__ int s_work[kRowsPerPass];       // rows of this pass that evict or allocate, in row order
+  __shared__ int s_wave_work[kRowsPerPass / 64];
   __shared__ int s_top, s_cache_base, s_cache_n, s_status;
 
   const int tid = threadIdx.x;
@@ -57,6 +59,7 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
     const int r = r0 + tid;
     int64_t p0 = 0;
     int lo = 0, hi = -1;
+    bool has_work = false;
     // ---- per row: eviction range and allocation need (block_manager policy) ------------------
     if (r < p.B) {
       p0 = p.n_tokens[r];
@@ -65,6 +68,7 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
       const int64_t lo_new64 = (p0 - wl) / bs;
       const int lo_new = p0 - wl > 0 ? (int)lo_new64 : 0;
       const int ev_end = min(lo_new, hi + 1);
+      const int lo_old = lo;
       s_evict_lo[tid] = lo;
       s_evict_n[tid] = max(0, ev_end - lo);
       if (ev_end > lo) s_evict_id[tid] = p.ring[(int64_t)r * R + lo % R];
@@ -81,13 +85,29 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
       } else {
         s_alloc[tid] = -1;
       }
+      has_work = ev_end > lo_old || s_alloc[tid] >= 0;
+    }
+    // Most rows of a decode step neither evict nor allocate (one in block_size does): list the ones that
+    // do, still in row order, so that the serial replay below walks only those.
+    const unsigned long long work_mask = __ballot(has_work);
+    if ((tid & 63) == 0) s_wave_work[tid >> 6] = __popcll(work_mask);
+    __syncthreads();
+    int n_work = 0;
+    {
+      int before = 0;
+      for (int w = 0; w < kRowsPerPass / 64; ++w) {
+        const int c = s_wave_work[w];
+        before += w < (tid >> 6) ? c : 0;
+        n_work += c;
+      }
+      if (has_work) s_work[before + __popcll(work_mask & ((1ull << (tid & 63)) - 1))] = tid;
     }
     __syncthreads();
     // ---- one thread replays pushes and pops in row order ---------------------------------------
     if (tid == 0) {
-      const int rows = min(kRowsPerPass, p.B - r0);
       int top = s_top, base = s_cache_base, n = s_cache_n;
-      for (int i = 0; i < rows; ++i) {
+      for (int w = 0; w < n_work; ++w) {
+        const int i = s_work[w];
         const int en = s_evict_n[i];
         for (int k = 0; k < en; ++k) {
           const int id = k == 0 ? s_evict_id[i] : p.ring[(int64_t)(r0 + i) * R + (s_evict_lo[i] + k) % R];
