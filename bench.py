@@ -200,18 +200,22 @@ def bench_gla_prompt(sb, dev, S=16, L=8192, H=28, iters=3):
             "vector_only_kernel_ms": round(times["vector_only"], 3)}
 
 
-def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None, gla_state_dtype=torch.float32):
+def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None, gla_state_dtype=torch.float32,
+                 gla_shared_states=False):
     """BASELINE config 5: the cache work of 128 consecutive decode steps of the 28-layer stack
     (14 GLA state layers + 14 paged SWA layers, one shared block table), B=256, every sequence at a
     logical context of 512k tokens (window-saturated), real appends, eviction and block recycling."""
-    c = sb.HybridDecodeCache(B, randomize=True, device=dev, kv_quant=kv_quant, gla_state_dtype=gla_state_dtype)
+    c = sb.HybridDecodeCache(B, randomize=True, device=dev, kv_quant=kv_quant, gla_state_dtype=gla_state_dtype,
+                             gla_shared_states=gla_shared_states)
     c.start(512 * 1024)
     g = torch.Generator(device=dev).manual_seed(1)
     q = torch.randn(B, HQ, D, device=dev, dtype=torch.bfloat16, generator=g)
     k = torch.randn(B, HKV, D, device=dev, dtype=torch.bfloat16, generator=g)
     v = torch.randn(B, HKV, D, device=dev, dtype=torch.bfloat16, generator=g)
-    gq, gk, gv = (torch.randn(B, HQ, 1, D, device=dev, dtype=torch.bfloat16, generator=g) for _ in range(3))
-    gg = torch.nn.functional.logsigmoid(torch.randn(B, HQ, 1, D, device=dev, generator=g)) / 16
+    gh = c.gla_state_heads  # heads of the GLA k, v, gate: all 28, or the 4 kv heads with shared states
+    gq = torch.randn(B, HQ, 1, D, device=dev, dtype=torch.bfloat16, generator=g)
+    gk, gv = (torch.randn(B, gh, 1, D, device=dev, dtype=torch.bfloat16, generator=g) for _ in range(2))
+    gg = torch.nn.functional.logsigmoid(torch.randn(B, gh, 1, D, device=dev, generator=g)) / 16
     out = torch.empty(B, HQ, D, device=dev, dtype=torch.bfloat16)
 
     def layers(meta):
@@ -247,7 +251,8 @@ def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None, gla_state_d
     gpu_ms = statistics.median(gpu)
     res = {"workload": f"BASELINE config 5: 28-layer hybrid decode step, B={B}, logical context 512k, "
                        f"{steps} consecutive steps" + ({"int8": ", SWA K/V as per-row INT8", "fp8": ", SWA K/V as fp8 (e4m3fn)"}.get(kv_quant, ""))
-                       + (", GLA state stored as bf16" if gla_state_dtype == torch.bfloat16 else ""),
+                       + (", GLA state stored as bf16" if gla_state_dtype == torch.bfloat16 else "")
+                       + (", one GLA state per kv head" if gla_shared_states else ""),
            "bytes_per_step": by,
            "host_stepped": {"ms_per_step": round(ms, 3), "decode_tok_per_s": round(B / (ms * 1e-3)),
                             "GBps": round(by / (ms * 1e-3) / 1e9, 1),
@@ -286,7 +291,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
                                                     "28-layer hybrid decode step (config 5)")
-    ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "hybrid_fp8", "hybrid_lean", "gla_prompt"), default=None,
+    ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "hybrid_fp8", "hybrid_lean", "hybrid_shared",
+                                       "hybrid_leanest", "gla_prompt"), default=None,
                     help="run just that section and print its JSON (short runs for profiling one kernel)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -312,6 +318,14 @@ def main():
     if args.only == "hybrid_lean":
         print(json.dumps({"hybrid_decode_int8_kv_bf16_state": bench_hybrid(
             sb, dev, steps=min(args.steps, 128), kv_quant="int8", gla_state_dtype=torch.bfloat16)}))
+        return
+    if args.only == "hybrid_shared":
+        print(json.dumps({"hybrid_decode_shared_gla_states": bench_hybrid(
+            sb, dev, steps=min(args.steps, 128), gla_shared_states=True)}))
+        return
+    if args.only == "hybrid_leanest":
+        print(json.dumps({"hybrid_decode_fp8_kv_shared_gla_states": bench_hybrid(
+            sb, dev, steps=min(args.steps, 128), kv_quant="fp8", gla_shared_states=True)}))
         return
     if args.only == "hybrid_fp8":
         print(json.dumps({"hybrid_decode_fp8_kv": bench_hybrid(sb, dev, steps=min(args.steps, 128), kv_quant="fp8")}))
@@ -434,6 +448,11 @@ def main():
         torch.cuda.empty_cache()
         # the storage formats of the reference's own variants: bf16 state cache (its serving path), INT8 K/V (W8ASpike)
         line["hybrid_decode_int8_kv_bf16_state"] = bench_hybrid(sb, dev, kv_quant="int8", gla_state_dtype=torch.bfloat16)
+        torch.cuda.empty_cache()
+        # one GLA state per kv head (same outputs, a seventh of the state traffic), alone and with fp8 K/V
+        line["hybrid_decode_shared_gla_states"] = bench_hybrid(sb, dev, gla_shared_states=True)
+        torch.cuda.empty_cache()
+        line["hybrid_decode_fp8_kv_shared_gla_states"] = bench_hybrid(sb, dev, kv_quant="fp8", gla_shared_states=True)
         torch.cuda.empty_cache()
 
     if not args.no_cpu_baseline:

@@ -230,6 +230,15 @@ typedef struct sb_gla_recurrent_args {
    * scan and accumulation; bf16 operand rounding on the output path as in any bf16 GEMM).
    * SB_GLA_VECTOR_ONLY keeps such calls on the step-by-step fp32 kernel. */
   int32_t flags;
+  /* Shared states, 0 or 1 = off. The reference computes k, v and the gate for the 4 kv heads and
+   * repeats them to the 28 query heads (hf_7B_model/gla_attention.py:147-149,
+   * vllm_hymeta/model_for_7B/gla_attention.py:264-267), so the q_heads_per_state = 7 query heads of
+   * a group carry bit-identical states as long as they start identical (they do: zeros). With
+   * q_heads_per_state = G > 1, k, v, g and state have num_heads / G heads (query head h uses head
+   * h / G of them), q and out keep num_heads heads, and every state is read and written once per
+   * step for its whole group: the state traffic of a decode step drops G-fold, results unchanged.
+   * num_heads must be a multiple of G, G <= 8. */
+  int32_t q_heads_per_state;
 } sb_gla_recurrent_args;
 
 int sb_gla_recurrent(const sb_gla_recurrent_args *args);

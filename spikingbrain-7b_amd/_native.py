@@ -71,7 +71,7 @@ class GlaRecurrentArgs(C.Structure):
         ("g_stride_b", i64), ("g_stride_h", i64), ("g_stride_t", i64),
         ("out_stride_b", i64), ("out_stride_h", i64), ("out_stride_t", i64),
         ("state_stride_slot", i64), ("state_stride_head", i64),
-        ("num_slots", i64), ("stream", vp), ("cu_seqlens", vp), ("flags", i32),
+        ("num_slots", i64), ("stream", vp), ("cu_seqlens", vp), ("flags", i32), ("q_heads_per_state", i32),
     ]
 
 

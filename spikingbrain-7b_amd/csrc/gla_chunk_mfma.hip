@@ -44,6 +44,10 @@ struct GlaChunkParams {
   float scale;
   int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, v_sb, v_sh, v_st, g_sb, g_sh, g_st, o_sb, o_sh, o_st;
   int64_t s_slot, s_head;
+  // Shared states: G query heads per head of k, v, g and state; head index hh of this launch (H of them)
+  // stands for state head hh / jn and query head (hh / jn) * G + j0 + hh % jn; write_state: store the
+  // final state. One state per head: G = jn = 1, j0 = 0, write_state = 1.
+  int G, jn, j0, write_state;
 };
 
 constexpr int kCB = 16;      // tokens per block
@@ -73,7 +77,9 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) { return __builtin_bit_
 template <bool kStateF32, int GDT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gla_chunk_kernel(const GlaChunkParams p) {
   const int b = blockIdx.x / p.H;
-  const int h = blockIdx.x - b * p.H;
+  const int hh = blockIdx.x - b * p.H;
+  const int hk = hh / p.jn;
+  const int h = hk * p.G + p.j0 + (hh - hk * p.jn);
   const int64_t slot = p.slot_idx ? (int64_t)p.slot_idx[b] : (int64_t)b;
   if (slot < 0) return;
   int T = p.T;
@@ -86,7 +92,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     qo = b * p.q_sb; ko = b * p.k_sb; vo = b * p.v_sb; go = b * p.g_sb; oo = b * p.o_sb;
   }
   if (T <= 0) return;
-  qo += h * p.q_sh; ko += h * p.k_sh; vo += h * p.v_sh; go += h * p.g_sh; oo += h * p.o_sh;
+  qo += h * p.q_sh; ko += hk * p.k_sh; vo += hk * p.v_sh; go += hk * p.g_sh; oo += h * p.o_sh;
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -98,7 +104,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   __shared__ __attribute__((aligned(16))) Stage stage[2];
 
   // ---- state: 8 row tiles x 2 column tiles of this wavefront's 32 columns -------------------------
-  char *sbase = reinterpret_cast<char *>(p.state) + (slot * p.s_slot + (int64_t)h * p.s_head) * (kStateF32 ? 4 : 2);
+  char *sbase = reinterpret_cast<char *>(p.state) + (slot * p.s_slot + (int64_t)hk * p.s_head) * (kStateF32 ? 4 : 2);
   f32x4_t S[8][2];
   auto state_index = [&](int rt, int nt, int i) {
     return (32 * (rt >> 1) + 8 * g + 4 * (rt & 1) + i) * 128 + 32 * w + 16 * nt + c;
@@ -268,6 +274,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
   }
 
+  if (!p.write_state) return;
 #pragma unroll
   for (int rt = 0; rt < 8; ++rt)
 #pragma unroll
@@ -285,11 +292,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 namespace sb_host {
 
 // Launch for bf16 q/k/v/out; g of any built type. Grid: one workgroup per (row, head).
-void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups) {
+void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads, int G, int jn, int j0, int write_state) {
   GlaChunkParams p;
   p.q = (const uint16_t *)a->q; p.k = (const uint16_t *)a->k; p.v = (const uint16_t *)a->v; p.g = a->g;
   p.state = a->state; p.out = (uint16_t *)a->out; p.slot_idx = a->slot_idx; p.cu = a->cu_seqlens;
-  p.H = a->num_heads; p.T = a->seq_len; p.scale = a->scale;
+  p.H = heads; p.T = a->seq_len; p.scale = a->scale;
+  p.G = G; p.jn = jn; p.j0 = j0; p.write_state = write_state;
   p.q_sb = a->q_stride_b; p.q_sh = a->q_stride_h; p.q_st = a->q_stride_t;
   p.k_sb = a->k_stride_b; p.k_sh = a->k_stride_h; p.k_st = a->k_stride_t;
   p.v_sb = a->v_stride_b; p.v_sh = a->v_stride_h; p.v_st = a->v_stride_t;

@@ -25,7 +25,17 @@ struct GlaParams {
   int64_t o_sb, o_sh, o_st;
   int64_t s_slot, s_head;
   const int32_t *cu;  // packed form: tokens of row b are cu[b] .. cu[b+1]-1, or null
+  // Shared states: G query heads per head of k, v, g and state. H counts the heads of THIS launch: head
+  // index hh of the grid stands for state head hk = hh / jn and query head hk * G + j0 + hh % jn, and the
+  // final state is stored only if write_state. One state per head: G = jn = 1, j0 = 0, write_state = 1.
+  int G, jn, j0, write_state;
 };
+
+// (state head, query head) of head index hh of the launch
+__device__ __forceinline__ void launch_heads(const GlaParams &p, int hh, int &hk, int &h) {
+  hk = hh / p.jn;
+  h = hk * p.G + p.j0 + (hh - hk * p.jn);
+}
 
 __device__ __forceinline__ float load_scalar(const void *p, int64_t i, int dtype) {
   if (dtype == SB_F32) return reinterpret_cast<const float *>(p)[i];
@@ -127,6 +137,83 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(const GlaParams p) {
   for (int i = 0; i < 16; ++i) store_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4, S[i]);
 }
 
+// ---- shared states: one state per kv head, G query heads read it -----------------------------------
+// Same thread layout, update and summation order as the kernel above (a group's state and each of its
+// heads' outputs come out bit-identical to what that kernel gives on repeated k, v, g), but the state
+// crosses HBM once per group instead of once per query head.
+constexpr int kMaxGroup = 8;
+
+template <bool kStateF32>
+__global__ __launch_bounds__(256) void gla_recurrent_grouped_kernel(const GlaParams p) {
+  const int Hk = p.H / p.G;
+  const int b = blockIdx.x / Hk;
+  const int hk = blockIdx.x - b * Hk;
+  const int64_t slot = p.slot_idx ? (int64_t)p.slot_idx[b] : (int64_t)b;
+  if (slot < 0) return;
+
+  const int tid = threadIdx.x;
+  const int col4 = tid & 31;
+  const int rg = tid >> 5;
+  const int G = p.G;
+
+  __shared__ float s_q[kMaxGroup][128], s_k[128], s_eg[128];
+  __shared__ __attribute__((aligned(16))) float s_v[128];
+  __shared__ __attribute__((aligned(16))) float s_o[kMaxGroup][8][128];
+
+  char *sbase = reinterpret_cast<char *>(p.state) +
+                (slot * p.s_slot + (int64_t)hk * p.s_head) * (kStateF32 ? 4 : 2);
+
+  float4 S[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) S[i] = load_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4);
+
+  for (int t = 0; t < p.T; ++t) {
+    for (int idx = tid; idx < G * 128; idx += 256) {
+      const int j = idx >> 7, e = idx & 127;
+      s_q[j][e] = load_scalar(p.q, b * p.q_sb + (hk * G + j) * p.q_sh + t * p.q_st + e, p.dtype) * p.scale;
+    }
+    if (tid < 128) {
+      s_k[tid] = load_scalar(p.k, b * p.k_sb + hk * p.k_sh + t * p.k_st + tid, p.dtype);
+      s_v[tid] = load_scalar(p.v, b * p.v_sb + hk * p.v_sh + t * p.v_st + tid, p.dtype);
+      s_eg[tid] = expf(load_scalar(p.g, b * p.g_sb + hk * p.g_sh + t * p.g_st + tid, p.g_dtype));
+    }
+    __syncthreads();
+    const float4 vv = reinterpret_cast<const float4 *>(s_v)[col4];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = i * 8 + rg;
+      const float kk = s_k[row], eg = s_eg[row];
+      S[i].x = fmaf(kk, vv.x, eg * S[i].x);
+      S[i].y = fmaf(kk, vv.y, eg * S[i].y);
+      S[i].z = fmaf(kk, vv.z, eg * S[i].z);
+      S[i].w = fmaf(kk, vv.w, eg * S[i].w);
+    }
+    for (int j = 0; j < G; ++j) {
+      float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float qq = s_q[j][i * 8 + rg];
+        o.x = fmaf(qq, S[i].x, o.x);
+        o.y = fmaf(qq, S[i].y, o.y);
+        o.z = fmaf(qq, S[i].z, o.z);
+        o.w = fmaf(qq, S[i].w, o.w);
+      }
+      reinterpret_cast<float4 *>(s_o[j][rg])[col4] = o;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < G * 128; idx += 256) {
+      const int j = idx >> 7, e = idx & 127;
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) acc += s_o[j][r][e];
+      store_scalar(p.out, b * p.o_sb + (hk * G + j) * p.o_sh + t * p.o_st + e, p.dtype, acc);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < 16; ++i) store_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4, S[i]);
+}
+
 // ---- many steps per call (prompts) ---------------------------------------------------------
 // The one-workgroup kernel above pays a global-memory round trip and two barriers per step. For
 // prompts the state is cut into four 32-column blocks, one single-wavefront workgroup each (no
@@ -157,7 +244,10 @@ struct Quad {
   static __device__ __forceinline__ float4 widen(Raw w) {
     if (DT == SB_BF16) return make_float4(sb::bf16_lo(w.x), sb::bf16_hi(w.x), sb::bf16_lo(w.y), sb::bf16_hi(w.y));
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    const h2 a = __builtin_bit_cast(h2, w.x), b = __builtin_bit_cast(h2, w.y);
+    // (through scalars: a bit cast taken directly from an element of the vector reads element 0 whichever
+    // element is named)
+    const unsigned int wx = w.x, wy = w.y;
+    const h2 a = __builtin_bit_cast(h2, wx), b = __builtin_bit_cast(h2, wy);
     return make_float4((float)a.x, (float)a.y, (float)b.x, (float)b.y);
   }
   static __device__ __forceinline__ void store(void *p, int64_t i, float4 o) {
@@ -194,7 +284,8 @@ __global__ __launch_bounds__(64) void gla_sequence_kernel(const GlaParams p) {
   const int cb = blockIdx.x & 3;
   const int bh = blockIdx.x >> 2;
   const int b = bh / p.H;
-  const int h = bh - b * p.H;
+  int hk, h;
+  launch_heads(p, bh - b * p.H, hk, h);
   const int64_t slot = p.slot_idx ? (int64_t)p.slot_idx[b] : (int64_t)b;
   if (slot < 0) return;
   int T = p.T;
@@ -212,8 +303,8 @@ __global__ __launch_bounds__(64) void gla_sequence_kernel(const GlaParams p) {
   // loads: q, k, g as (step parity lane / 32, elements 4*(lane % 32) ..), v as (step lane / 8,
   // columns 4*(lane % 8) .. of this block)
   const int lstep = lane >> 5, lcol = (lane & 31) * 4;
-  qo += h * p.q_sh + lcol; ko += h * p.k_sh + lcol; go += h * p.g_sh + lcol;
-  vo += h * p.v_sh + cb * 32 + rg * 4;
+  qo += h * p.q_sh + lcol; ko += hk * p.k_sh + lcol; go += hk * p.g_sh + lcol;
+  vo += hk * p.v_sh + cb * 32 + rg * 4;
   oo += h * p.o_sh + cb * 32 + cq * 4;
 
   __shared__ __attribute__((aligned(16))) float s_q[kSeqBlock][128];
@@ -222,7 +313,7 @@ __global__ __launch_bounds__(64) void gla_sequence_kernel(const GlaParams p) {
   __shared__ __attribute__((aligned(16))) float s_v[kSeqBlock][32];
 
   char *sbase = reinterpret_cast<char *>(p.state) +
-                (slot * p.s_slot + (int64_t)h * p.s_head) * (kStateF32 ? 4 : 2);
+                (slot * p.s_slot + (int64_t)hk * p.s_head) * (kStateF32 ? 4 : 2);
   float4 S[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) S[i] = load_state4<kStateF32>(sbase, (rg * 16 + i) * 32 + cb * 8 + cq);
@@ -284,6 +375,7 @@ __global__ __launch_bounds__(64) void gla_sequence_kernel(const GlaParams p) {
     const int steps = min(kSeqBlock, T - t0);
     for (int s = 0; s < steps; ++s) step(s);
   }
+  if (!p.write_state) return;
 #pragma unroll
   for (int i = 0; i < 16; ++i) store_state4<kStateF32>(sbase, (rg * 16 + i) * 32 + cb * 8 + cq, S[i]);
 }
@@ -304,7 +396,7 @@ void launch_sequence(const GlaParams &p, dim3 grid, hipStream_t st) {
 }  // namespace
 
 namespace sb_host {
-void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups);
+void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads, int G, int jn, int j0, int write_state);
 }
 
 // Calls of this many steps or more (and every packed call) with bf16 q, k, v run on the matrix cores.
@@ -331,6 +423,11 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
     return fail(SB_ERR_INVALID, "sb_gla_recurrent: state rows must be 16-byte aligned");
   const int64_t groups = a->batch * (int64_t)a->num_heads;
   if (groups > 0x7fffffffLL) return fail(SB_ERR_UNSUPPORTED, "sb_gla_recurrent: batch*heads too large");
+  const int G = a->q_heads_per_state > 1 ? a->q_heads_per_state : 1;
+  if (a->q_heads_per_state < 0 || G > kMaxGroup || a->num_heads % G)
+    return fail(SB_ERR_INVALID, "sb_gla_recurrent: q_heads_per_state %d must be 0..%d and divide num_heads %d",
+                a->q_heads_per_state, kMaxGroup, a->num_heads);
+  const int Hk = a->num_heads / G;
 
   GlaParams p;
   p.q = a->q; p.k = a->k; p.v = a->v; p.g = a->g;
@@ -345,6 +442,7 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
   p.s_slot = a->state_stride_slot; p.s_head = a->state_stride_head;
 
   p.cu = a->cu_seqlens;
+  p.G = G; p.jn = 1; p.j0 = 0; p.write_state = 1;
 
   // the prompt kernel moves q, k, v, g, out as 4-element vectors
   auto quad_aligned = [](const void *ptr, int dt, int64_t sb_, int64_t sh, int64_t st) {
@@ -367,7 +465,13 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
                          piece_aligned(a->out, 8, p.o_sb, p.o_sh, p.o_st);
   if (a->dtype == SB_BF16 && pieces_ok && !(a->flags & SB_GLA_VECTOR_ONLY) &&
       (a->cu_seqlens || a->seq_len >= kChunkKernelMinSteps)) {
-    launch_gla_chunk(a, groups);
+    // Shared states: the heads of a group each carry the recurrence for their own outputs (that keeps
+    // one workgroup per query head busy), all reading the group's state. The group's first head stores
+    // the final state, in a launch of its own behind the others so that no head reads a state already
+    // advanced.
+    if (G > 1) launch_gla_chunk(a, a->batch * (int64_t)Hk * (G - 1), Hk * (G - 1), G, G - 1, 1, 0);
+    if (G > 1) launch_gla_chunk(a, a->batch * (int64_t)Hk, Hk, G, 1, 0, 1);
+    else launch_gla_chunk(a, groups, a->num_heads, 1, 1, 0, 1);
     return check_launch("gla_chunk_kernel");
   }
   if (a->cu_seqlens && !vectors_ok)
@@ -376,12 +480,28 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
   if (a->cu_seqlens || (a->seq_len >= kSeqKernelMinSteps && vectors_ok)) {
     // prompts: one wavefront per (row, head, 32-column block of the state), inputs staged ahead
     if (groups * 4 > 0x7fffffffLL) return fail(SB_ERR_UNSUPPORTED, "sb_gla_recurrent: batch*heads too large");
-    const dim3 sgrid((unsigned)(groups * 4));
-    if (a->state_dtype == SB_F32)
-      launch_sequence<true>(p, sgrid, (hipStream_t)a->stream);
-    else
-      launch_sequence<false>(p, sgrid, (hipStream_t)a->stream);
+    for (int pass = G > 1 ? 0 : 1; pass < 2; ++pass) {  // shared states: see the matrix-core launches above
+      if (G > 1) {
+        p.jn = pass == 0 ? G - 1 : 1;
+        p.j0 = pass == 0 ? 1 : 0;
+        p.write_state = pass;
+        p.H = Hk * p.jn;
+      }
+      const dim3 sgrid((unsigned)(a->batch * p.H * 4));
+      if (a->state_dtype == SB_F32)
+        launch_sequence<true>(p, sgrid, (hipStream_t)a->stream);
+      else
+        launch_sequence<false>(p, sgrid, (hipStream_t)a->stream);
+    }
     return check_launch("gla_sequence_kernel");
+  }
+  if (G > 1) {  // decode with shared states: one workgroup per (row, state head)
+    const dim3 ggrid((unsigned)(a->batch * Hk));
+    if (a->state_dtype == SB_F32)
+      hipLaunchKernelGGL(gla_recurrent_grouped_kernel<true>, ggrid, dim3(256), 0, (hipStream_t)a->stream, p);
+    else
+      hipLaunchKernelGGL(gla_recurrent_grouped_kernel<false>, ggrid, dim3(256), 0, (hipStream_t)a->stream, p);
+    return check_launch("gla_recurrent_grouped_kernel");
   }
   const dim3 grid((unsigned)groups), block(256);
   if (a->state_dtype == SB_F32)

@@ -31,13 +31,16 @@ class HybridDecodeCache:
                  head_size: int = 128, block_size: int = 16, window_left: int = 4096,
                  dtype: torch.dtype = torch.bfloat16, device="cuda:0", num_blocks: Optional[int] = None,
                  randomize: bool = False, seed: int = 0, kv_quant: Optional[str] = None,
-                 gla_state_dtype: torch.dtype = torch.float32):
+                 gla_state_dtype: torch.dtype = torch.float32, gla_shared_states: bool = False):
         """kv_quant="int8": the SWA layers keep their K/V as per-row INT8 codes + fp32 scales
         (quantize_sym of W8ASpike/window_attention.py:227-237 applied once, at append time);
         kv_quant="fp8": as e4m3fn codes with per-tensor scales of 1 (the kv_cache_dtype="fp8" branch of
         vllm_hymeta/attention/meta_attention.py:790-812).
         gla_state_dtype: float32, or bfloat16 as the reference's serving path keeps its state cache
-        (vllm_hymeta/model_for_7B/modeling_gla_swa.py:361-364); the arithmetic is fp32 either way."""
+        (vllm_hymeta/model_for_7B/modeling_gla_swa.py:361-364); the arithmetic is fp32 either way.
+        gla_shared_states: keep one GLA state per kv head instead of one per query head; the layers then
+        take k, v, g with num_kv_heads heads, before the model's repeat_kv
+        (vllm_hymeta/model_for_7B/gla_attention.py:264-267), and give the same outputs."""
         if gla_state_dtype not in (torch.float32, torch.bfloat16):
             raise ValueError("gla_state_dtype must be float32 or bfloat16")
         if kv_quant not in (None, "int8", "fp8"):
@@ -79,7 +82,9 @@ class HybridDecodeCache:
         else:
             self.kv_caches: List[torch.Tensor] = [alloc(shape, dtype, 1.0) for _ in self.swa_layers]
         # [n_gla_layers, slots, H, D, D] fp32, as vllm_hymeta/model_for_7B/modeling_gla_swa.py:348-356
-        self.gla_state = alloc((len(self.gla_layers), batch, num_heads, head_size, head_size), gla_state_dtype, 0.02)
+        self.gla_state_heads = num_kv_heads if gla_shared_states else num_heads
+        self.gla_state = alloc((len(self.gla_layers), batch, self.gla_state_heads, head_size, head_size),
+                               gla_state_dtype, 0.02)
         self.slot_idx = torch.arange(batch, dtype=torch.int32, device=self.device)
         self.impl = MetaAttentionImpl(num_heads, head_size, head_size ** -0.5, num_kv_heads, None, window_left + 1,
                                       "auto")
@@ -148,7 +153,8 @@ class HybridDecodeCache:
         return graph
 
     def gla_layer(self, layer_idx: int, q, k, v, g, out=None) -> torch.Tensor:
-        """q, k, v, g [B, H, 1, D]; the layer's state is advanced in place. Returns o [B, H, 1, D]."""
+        """q [B, H, 1, D]; k, v, g [B, H, 1, D], or [B, Hkv, 1, D] with shared states; the layer's state is
+        advanced in place. Returns o [B, H, 1, D]."""
         out = self._gla_out if out is None else out
         ops.gla_recurrent(q, k, v, g, self.gla_state[layer_idx // 2], self.slot_idx, self.D ** -0.5, out)
         return out
@@ -185,8 +191,10 @@ class HybridDecodeCache:
         else:
             swa = int(n_keys.sum()) * self.Hkv * self.D * 2 * e + self.batch * (2 * self.H * self.D * e
                                                                                + 4 * self.Hkv * self.D * e)
-        gla = self.batch * self.H * (2 * self.D * self.D * self.gla_state.element_size() + 3 * self.D * e + self.D * 4
-                                     + self.D * e)
+        # per state: read + write, and its k, v (e bytes) and gate (fp32) rows; per query head: q in, o out
+        Hs = self.gla_state_heads
+        gla = self.batch * (Hs * (2 * self.D * self.D * self.gla_state.element_size() + 2 * self.D * e + self.D * 4)
+                            + self.H * 2 * self.D * e)
         return len(self.swa_layers) * swa + len(self.gla_layers) * gla
 
 

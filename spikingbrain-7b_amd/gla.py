@@ -37,12 +37,16 @@ def my_fused_recurrent_gla(
     Returns o [B, H, D] (my_fused_recurrent.py:117-119). `initial_state`, `output_final_state`
     and `reverse` are accepted and ignored, as in the reference (:88-119 never reads them).
     Rows whose slot is -1 keep whatever the output buffer held (the reference leaves them
-    uninitialised); here the buffer starts zeroed."""
+    uninitialised); here the buffer starts zeroed.
+
+    Shared states (not in the reference, which repeats k, v and the gate to all query heads before this
+    call, gla_attention.py:264-267): k, v, g [B, Hkv, 1, D] and kv_caches [slots, Hkv, D, D] with H a
+    multiple of Hkv give the same outputs from one state per kv head."""
     if q.dim() != 4 or q.shape[2] != 1:
         raise AssertionError(f"decode expects q of shape [B, H, 1, D], got {tuple(q.shape)}")
     B, H, _, D = q.shape
-    assert k.shape == (B, H, 1, D)
-    assert v.shape == (B, H, 1, D)
+    assert k.dim() == 4 and (k.shape[0], k.shape[2], k.shape[3]) == (B, 1, D) and H % k.shape[1] == 0
+    assert v.shape == k.shape
     if scale is None:
         scale = D ** -0.5
     if slot_idx is not None and slot_idx.dtype != torch.int32:
@@ -66,10 +70,11 @@ def fused_recurrent_gla(
     hf_7B_model/gla_attention.py:153: returns (o [B, H, T, D], final_state [B, H, D, D] fp32 or None).
     The state crosses HBM once in each direction whatever T is. With inplace_state=True an fp32
     `initial_state` is advanced in place and returned (the cache replaces it by reference anyway,
-    hf_7B_model/cache.py:92-93), saving the copy."""
+    hf_7B_model/cache.py:92-93), saving the copy. With k, v, gk of Hkv < H heads the state is
+    [B, Hkv, D, D], shared by each group of H / Hkv query heads."""
     B, H, T, D = q.shape
     if initial_state is None:
-        state = torch.zeros((B, H, D, D), dtype=torch.float32, device=q.device)
+        state = torch.zeros((B, k.shape[1], D, D), dtype=torch.float32, device=q.device)
     elif inplace_state and initial_state.dtype == torch.float32 and initial_state.is_contiguous():
         state = initial_state
     else:

@@ -579,16 +579,22 @@ def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
     Rows with slot_idx == -1 are skipped (state and output untouched).
     Calls of 32 steps or more with bf16 q/k/v run 16 tokens at a time on the matrix cores (state, gates
     and accumulation in fp32, bf16 operand rounding on the output path); vector_only=True keeps them on
-    the step-by-step fp32 kernel."""
+    the step-by-step fp32 kernel.
+    Shared states: k, v, g may come with Hkv < H heads (H a multiple of Hkv, up to 8 query heads per kv
+    head) and state as [slots, Hkv, D, D]: query head h then works on head h // (H // Hkv) of them, which is
+    the reference's repeat_kv of k, v and the gate (hf_7B_model/gla_attention.py:147-149) without the
+    copies, and every state crosses HBM once per step for its whole group."""
     dev = N.require_gpu(q, k, v, g, state, slot_idx, out)
-    if q.dim() != 4 or k.shape != q.shape or v.shape != q.shape or g.shape != q.shape:
-        raise ValueError(f"q, k, v, g must all be [B, H, T, D]; got {tuple(q.shape)}, {tuple(k.shape)}, "
-                         f"{tuple(v.shape)}, {tuple(g.shape)}")
+    if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape or g.shape != k.shape or \
+            (k.shape[0], k.shape[2], k.shape[3]) != (q.shape[0], q.shape[2], q.shape[3]):
+        raise ValueError(f"q [B, H, T, D] and k, v, g [B, H or Hkv, T, D] expected; got {tuple(q.shape)}, "
+                         f"{tuple(k.shape)}, {tuple(v.shape)}, {tuple(g.shape)}")
     B, H, T, D = q.shape
+    Hk = _state_heads(H, k.shape[1])
     if not (k.dtype == q.dtype and v.dtype == q.dtype):
         raise ValueError("q, k, v must share one dtype")
-    if state.dim() != 4 or state.shape[1:] != (H, D, D):
-        raise ValueError(f"state must be [slots, {H}, {D}, {D}], got {tuple(state.shape)}")
+    if state.dim() != 4 or state.shape[1:] != (Hk, D, D):
+        raise ValueError(f"state must be [slots, {Hk}, {D}, {D}], got {tuple(state.shape)}")
     if state.stride(3) != 1 or state.stride(2) != D:
         raise ValueError("each [dk, dv] state matrix must be contiguous")
     for t, n in ((q, "q"), (k, "k"), (v, "v"), (g, "g")):
@@ -617,9 +623,18 @@ def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
         g_stride_b=g.stride(0), g_stride_h=g.stride(1), g_stride_t=g.stride(2),
         out_stride_b=out.stride(0), out_stride_h=out.stride(1), out_stride_t=out.stride(2),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
-        num_slots=state.shape[0], stream=N.stream_ptr(dev), flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0)
+        num_slots=state.shape[0], stream=N.stream_ptr(dev), flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0,
+        q_heads_per_state=H // Hk)
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
+
+
+def _state_heads(num_q_heads: int, num_k_heads: int) -> int:
+    """Heads of k, v, g and of the state: all of them, or one per group of up to 8 query heads."""
+    if num_k_heads <= 0 or num_q_heads % num_k_heads or num_q_heads // num_k_heads > 8:
+        raise ValueError(f"{num_q_heads} query heads over {num_k_heads} heads of k, v, g: need a whole number of "
+                         "query heads per head, at most 8")
+    return num_k_heads
 
 
 def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
@@ -629,15 +644,18 @@ def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: t
     """The same recurrence over packed prompts: q, k, v, g [total_tokens, H, D] (token/head strides
     free, contiguous D), sequence b owning tokens cu_seqlens[b] .. cu_seqlens[b+1]-1 (int32 device
     vector [B+1]); its state is state[slot_idx[b]] (default b), advanced in place. One launch for
-    all sequences. Returns o [total_tokens, H, D]."""
+    all sequences. Returns o [total_tokens, H, D]. Shared states as in gla_recurrent: k, v, g
+    [total_tokens, Hkv, D] with state [slots, Hkv, D, D]."""
     dev = N.require_gpu(q, k, v, g, state, cu_seqlens, slot_idx, out)
-    if q.dim() != 3 or k.shape != q.shape or v.shape != q.shape or g.shape != q.shape:
-        raise ValueError("q, k, v, g must all be [total_tokens, H, D]")
+    if q.dim() != 3 or k.dim() != 3 or v.shape != k.shape or g.shape != k.shape or \
+            (k.shape[0], k.shape[2]) != (q.shape[0], q.shape[2]):
+        raise ValueError("q [total_tokens, H, D] and k, v, g [total_tokens, H or Hkv, D] expected")
     Tt, H, D = q.shape
+    Hk = _state_heads(H, k.shape[1])
     if not (k.dtype == q.dtype and v.dtype == q.dtype):
         raise ValueError("q, k, v must share one dtype")
-    if state.dim() != 4 or state.shape[1:] != (H, D, D) or state.stride(3) != 1 or state.stride(2) != D:
-        raise ValueError(f"state must be [slots, {H}, {D}, {D}] with contiguous matrices")
+    if state.dim() != 4 or state.shape[1:] != (Hk, D, D) or state.stride(3) != 1 or state.stride(2) != D:
+        raise ValueError(f"state must be [slots, {Hk}, {D}, {D}] with contiguous matrices")
     if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2 or not cu_seqlens.is_contiguous():
         raise ValueError("cu_seqlens must be a contiguous int32 vector [B+1]")
     B = cu_seqlens.numel() - 1
@@ -668,7 +686,7 @@ def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: t
         out_stride_b=0, out_stride_h=out.stride(1), out_stride_t=out.stride(0),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
         num_slots=state.shape[0], stream=N.stream_ptr(dev), cu_seqlens=N.ptr(cu_seqlens),
-        flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0)
+        flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0, q_heads_per_state=H // Hk)
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
 

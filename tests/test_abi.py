@@ -58,6 +58,12 @@ def test_bad_shapes_rejected_before_launch(sb):
     assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_WORKSPACE
     g = N.GlaRecurrentArgs(q=16, k=16, v=16, g=16, state=16, out=16, batch=1, num_heads=1, seq_len=1, head_dim=64)
     assert L.sb_gla_recurrent(C.byref(g)) == N.SB_ERR_UNSUPPORTED
+    # shared states: the group size must divide the query heads and stay within 8
+    g = N.GlaRecurrentArgs(q=16, k=16, v=16, g=16, state=16, out=16, batch=1, num_heads=28, seq_len=1, head_dim=128,
+                           state_dtype=N.SB_F32, state_stride_slot=4 * 16384, state_stride_head=16384)
+    for bad in (3, 14, -1):
+        g.q_heads_per_state = bad
+        assert L.sb_gla_recurrent(C.byref(g)) == N.SB_ERR_INVALID
 
 
 def test_auto_split_and_workspace(sb):

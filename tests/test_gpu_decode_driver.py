@@ -147,3 +147,32 @@ def test_captured_graph_replays_whole_steps(sb, dev):
             assert np.array_equal(drv.kv_caches[j][0].float().cpu().numpy(), kc[j])
     drv.device_state.download()
     assert drv.manager.free_stack() == model.free
+
+
+def test_shared_gla_states_give_the_same_outputs(sb, dev):
+    """One GLA state per kv head: the driver takes k, v and the gate before the model's repeat_kv
+    (vllm_hymeta/model_for_7B/gla_attention.py:264-267) and must give, bit for bit, what the 28-state
+    driver gives on the repeated tensors; bytes_per_step counts the smaller state traffic."""
+    B, L, H, HKV, D = 5, 4, 28, 4, 128
+    kw = dict(num_layers=L, num_heads=H, num_kv_heads=HKV, head_size=D, window_left=40, device=dev)
+    shared = sb.HybridDecodeCache(B, randomize=True, seed=9, gla_shared_states=True, **kw)
+    full = sb.HybridDecodeCache(B, **kw)
+    assert shared.gla_state.shape == (L // 2, B, HKV, D, D) and full.gla_state.shape == (L // 2, B, H, D, D)
+    full.gla_state.copy_(shared.gla_state.repeat_interleave(H // HKV, dim=2))
+    g = torch.Generator().manual_seed(0)
+    for step in range(4):
+        for li in (0, 2):
+            q = torch.randn(B, H, 1, D, generator=g).bfloat16().to(dev)
+            k, v = (torch.randn(B, HKV, 1, D, generator=g).bfloat16().to(dev) for _ in range(2))
+            gate = (torch.nn.functional.logsigmoid(torch.randn(B, HKV, 1, D, generator=g)) / 16).to(dev)
+            o = shared.gla_layer(li, q, k, v, gate).clone()
+            r = H // HKV
+            o_full = full.gla_layer(li, q, k.repeat_interleave(r, 1), v.repeat_interleave(r, 1),
+                                    gate.repeat_interleave(r, 1))
+            assert torch.equal(o, o_full), (step, li)
+    assert torch.equal(shared.gla_state, full.gla_state[:, :, ::H // HKV])
+    shared.start(100)
+    full.start(100)
+    e = 2
+    per_layer_saving = B * (H - HKV) * (2 * D * D * 4 + 2 * D * e + D * 4)
+    assert full.bytes_per_step() - shared.bytes_per_step() == (L // 2) * per_layer_saving

@@ -282,3 +282,24 @@ def test_block_form_strong_gates_and_gate_dtypes(sb, dev, gdtype):
     o, S = sb.fused_recurrent_gla(qd, kd, vd, gate.to(dev), output_final_state=True)
     assert rel(S.double().cpu().numpy(), ref_S) <= STATE_RTOL
     assert out_close(o.float().cpu().numpy(), ref_o)
+
+
+@pytest.mark.parametrize("gdtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T", [4, 9, 24])
+def test_step_by_step_prompt_kernel_every_element_type(sb, dev, dtype, gdtype, T):
+    """The many-step vector kernel is compiled once per (q/k/v type, gate type): each of them against the
+    oracle, on calls short enough (or of a type) that the matrix-core block form does not take."""
+    B, H, D = 2, 3, 128
+    q, k, v, gate = make(B, H, T, D, 7 * T, dtype, relu=True)
+    gate = gate.to(gdtype)
+    S0 = torch.randn(B, H, D, D, generator=torch.Generator().manual_seed(T)) * 0.02
+    ref_o, ref_S = G.gla_recurrent(q.float().numpy(), k.float().numpy(), v.float().numpy(), gate.float().numpy(),
+                                   S0.double().numpy())
+    st = S0.clone().to(dev)
+    o = sb.ops.gla_recurrent(q.to(dev), k.to(dev), v.to(dev), gate.to(dev), st)
+    assert rel(st.double().cpu().numpy(), ref_S) <= STATE_RTOL
+    if dtype == torch.float32:
+        assert np.abs(o.double().cpu().numpy() - ref_o).max() <= 1e-4 * max(1.0, np.abs(ref_o).max())
+    else:
+        assert out_close(o.float().cpu().numpy(), ref_o, dtype)
