@@ -167,6 +167,19 @@ typedef struct sb_swa_decode_args {
    * (kv strides in bytes), dequantised as code * k_scale_tensor / v_scale_tensor. Same restrictions as
    * the INT8 cache. */
   float k_scale_tensor, v_scale_tensor;
+  /* Meta (sink) tokens, the query2/key2/value2 path of vllm_hymeta/attention/fa_kernel_metatoken.py:
+   * 110-194: every query row also attends, without mask or window, to the meta_len rows of meta_k /
+   * meta_v ([meta_len, num_kv_heads, 128] of dtype, strides in elements), the same rows for every
+   * sequence. The reference runs a second attention and merges the two results by their log-sum-exp;
+   * here the 32-row chunks of the meta rows are dealt round robin to the splits of each query row's
+   * window and enter the same online softmax, so out and lse are those of ONE softmax over window
+   * and meta keys (a row with an empty window attends to the meta rows alone). meta_len = 0 = off.
+   * bf16/fp16 matrix-core kernel with the fixed split only (rejected with SB_DECODE_BALANCED,
+   * SB_DECODE_FORCE_VALU, fp32 or a byte-code cache). */
+  const void *meta_k;
+  const void *meta_v;
+  int32_t meta_len;
+  int64_t meta_stride_row, meta_stride_head;
 } sb_swa_decode_args;
 
 /* Split count the auto rule (n_split = 0) would use for these shapes. */

@@ -57,6 +57,7 @@ class SwaDecodeArgs(C.Structure):
         ("new_value_stride_row", i64), ("new_value_stride_head", i64),
         ("stream", vp), ("k_scale", vp), ("v_scale", vp), ("kv_quant", i32),
         ("k_scale_tensor", f32), ("v_scale_tensor", f32),
+        ("meta_k", vp), ("meta_v", vp), ("meta_len", i32), ("meta_stride_row", i64), ("meta_stride_head", i64),
     ]
 
 

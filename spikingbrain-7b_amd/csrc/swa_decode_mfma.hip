@@ -63,12 +63,15 @@ __device__ __forceinline__ int row_chunks(const DecodeParams &p, const int32_t *
 // with an online softmax of its own, result written as the row's output (`direct`) or as the
 // fp32 partial number part_base + head * part_hs. kDepth = chunks in flight besides the one being
 // computed. `owns_newest`: this range ends the row's window (with a fused append it stores the
-// step's K/V row into the cache).
+// step's K/V row into the cache). Meta tokens: the call also takes chunks meta_first,
+// meta_first + meta_step, ... of the p.meta_len shared meta rows into the same softmax (meta_step 0:
+// none); the first of them is fetched before the window is walked and computed after it.
 template <typename E, int kDepth>
 __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32_t *block_table, const int G,
                                               const int kvh, const int lane, const int64_t r, const int lo,
                                               const int hi, const int cb, const int ce, const bool owns_newest,
-                                              const bool direct, const int64_t part_base, const int part_hs) {
+                                              const bool direct, const int64_t part_base, const int part_hs,
+                                              const int meta_first, const int meta_step) {
   const int g = lane >> 4;
   const int c = lane & 15;
   const int64_t seq = p.row_seq ? (int64_t)p.row_seq[r] : r;
@@ -165,9 +168,28 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
     }
   };
 
+  // Meta chunk cc: rows 32cc .. 32cc+31 of the dense meta tensors, clamped to the last row (masked by
+  // their true index in the scores). Ordinary loads: every workgroup of the launch reads these rows.
+  auto load_meta = [&](int cc, Chunk &ck) {
+    const char *mk = p.meta_k + (int64_t)kvh * p.meta_sh, *mv = p.meta_v + (int64_t)kvh * p.meta_sh;
+    const int last = p.meta_len - 1, i0 = cc << 5;
+    const char *pk0 = mk + (int64_t)min(i0 + c, last) * p.meta_sr + g * 16;
+    const char *pk1 = mk + (int64_t)min(i0 + 16 + c, last) * p.meta_sr + g * 16;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      ck.k0[s] = *reinterpret_cast<const uint4 *>(pk0 + s * 64);
+      ck.k1[s] = *reinterpret_cast<const uint4 *>(pk1 + s * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      ck.v[j] = *reinterpret_cast<const uint4 *>(mv + (int64_t)min(i0 + 4 * g + j, last) * p.meta_sr + c * 16);
+      ck.v[4 + j] = *reinterpret_cast<const uint4 *>(mv + (int64_t)min(i0 + 16 + 4 * g + j, last) * p.meta_sr + c * 16);
+    }
+  };
+
   // One chunk of work: S^T = K Q^T, online softmax, O^T += V^T P^T. kMask = edge chunk (keys outside
-  // [lo, hi) are masked by their true index).
-  auto compute_chunk = [&](int ch, const Chunk &ck, auto mask_tag) {
+  // [mlo, mhi) are masked by their true index).
+  auto compute_chunk = [&](int ch, const Chunk &ck, auto mask_tag, const int mlo, const int mhi) {
     constexpr bool kMask = decltype(mask_tag)::value;
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -181,7 +203,7 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int i = i0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-        if (i < lo || i >= hi) sc[j] = kNegInf;
+        if (i < mlo || i >= mhi) sc[j] = kNegInf;
       }
     }
     float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
@@ -231,6 +253,11 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
   // Interior chunks lie wholly inside [lo, hi), so the unclamped interior loader (and the block
   // table lookups made for it) never leave the sequence; when a split has no interior chunk the
   // loop and its prologue are skipped altogether.
+  const int meta_chunks = (p.meta_len + 31) >> 5;
+  const bool has_meta = meta_step > 0 && meta_first < meta_chunks;
+  Chunk metac;
+  if (has_meta) load_meta(meta_first, metac);
+
   if (cb < ce) {
     // with a fused append the chunk holding the newest key is an edge chunk even when it is full:
     // that row is not in the cache yet and only the edge loader reads it from the step inputs
@@ -262,14 +289,14 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
       // edge loads go behind the prologue: by the time they have landed so has the prologue
       load_edge(cb, head);
       load_edge(ce - 1, tail);
-      if (e_head) compute_chunk(cb, head, kMasked);
+      if (e_head) compute_chunk(cb, head, kMasked, lo, hi);
       bool more = true;
       while (more) {
 #pragma unroll
         for (int u = 0; u <= kDepth; ++u) {
           if (more) {
             issue(ch + kDepth, ring[(u + kDepth) % (kDepth + 1)]);
-            compute_chunk(ch, ring[u], kUnmasked);
+            compute_chunk(ch, ring[u], kUnmasked, lo, hi);
             ++ch;
             more = ch < ie;
           }
@@ -278,9 +305,17 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
     } else {
       load_edge(cb, head);
       load_edge(ce - 1, tail);
-      if (e_head) compute_chunk(cb, head, kMasked);
+      if (e_head) compute_chunk(cb, head, kMasked, lo, hi);
     }
-    if (e_tail) compute_chunk(ce - 1, tail, kMasked);
+    if (e_tail) compute_chunk(ce - 1, tail, kMasked, lo, hi);
+  }
+
+  if (has_meta) {
+    compute_chunk(meta_first, metac, kMasked, 0, p.meta_len);
+    for (int cc = meta_first + meta_step; cc < meta_chunks; cc += meta_step) {
+      load_meta(cc, metac);
+      compute_chunk(cc, metac, kMasked, 0, p.meta_len);
+    }
   }
 
   // ---- fused append: store the newest K/V row at its slot ---------------------------------
@@ -349,7 +384,8 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
   const int cb = first_chunk + split * cps;
   const int ce = min(cb + cps, first_chunk + n_chunks);
   split_segment<E, kDepth>(p, p.block_table, G, kvh, tid & 63, r, lo, hi, cb, ce, ce == first_chunk + n_chunks,
-                           p.n_split == 1, r * p.Hq * p.n_split + split, p.n_split);
+                           p.n_split == 1, r * p.Hq * p.n_split + split, p.n_split,
+                           split, p.meta_len > 0 ? p.n_split : 0);  // meta chunks dealt round robin to the splits
 }
 
 __device__ __forceinline__ int wave_sum(int x) {
@@ -409,7 +445,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_balanced_mfma_kerne
       const int rn = row_chunks(p, seq_lens, r, rlo, rhi, rfc);  // uniform: scalar loads
       const int cb = rfc + max(c0 - r_start, 0), ce = rfc + min(c1 - r_start, rn);
       split_segment<E, kDepth>(p, block_table, G, kvh, lane, r, rlo, rhi, cb, ce, ce == rfc + rn, false,
-                               (int64_t)(w + r) * p.Hq, 1);
+                               (int64_t)(w + r) * p.Hq, 1, 0, 0);
     }
     before += __builtin_amdgcn_readlane(incl, 63);
   }

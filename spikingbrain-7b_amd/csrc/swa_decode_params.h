@@ -32,6 +32,12 @@ struct DecodeParams {
   const float *k_scale;
   const float *v_scale;
   float kv_out_scale;  // multiplies the result (fp8 cache: the V tensor scale; else 1)
+  // Meta tokens (matrix-core fixed split only): meta_len rows [meta_len, Hkv, 128] every query row also
+  // attends to, without mask; meta_len = 0 = none
+  const char *meta_k;
+  const char *meta_v;
+  int meta_len;
+  int64_t meta_sr, meta_sh;  // bytes
 };
 
 }  // namespace sb

@@ -581,12 +581,19 @@ class MetaAttentionImpl:
                         host_lens is not None and len(host_lens) >= n and
                         ops.plan_decode_split(n, self.num_kv_heads, decode_meta.max_decode_seq_len or max(host_lens[:n]),
                                               window_left, host_lens[:n]))
+                # meta tokens ride in the same launch (their chunks join each split's softmax) when the
+                # cache holds bf16/fp16 rows; over a byte-code cache they stay a second attention + merge
+                meta_inside = with_meta and not byte_kv and decode_query.dtype in (torch.bfloat16, torch.float16)
+                if meta_inside:
+                    fused.update(meta_k=key2, meta_v=value2)
                 res = ops.swa_decode_attention(
                     decode_query, key_cache, value_cache, decode_meta.seq_lens_tensor[:n],
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
-                    out=decode_output, return_lse=with_meta,
+                    out=decode_output, return_lse=with_meta and not meta_inside,
                     max_seq_len=decode_meta.max_decode_seq_len or None,
                     balanced=False if byte_kv else decode_meta._decode_balanced, **scales, **fused)
+                if meta_inside:
+                    return output
                 lse = res[1] if with_meta else None
             merge_meta(decode_query, decode_output, lse)
         return output

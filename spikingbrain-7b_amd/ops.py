@@ -101,8 +101,14 @@ def swa_decode_attention(
     new_key: Optional[torch.Tensor] = None,
     new_value: Optional[torch.Tensor] = None,
     new_slot_mapping: Optional[torch.Tensor] = None,
+    meta_k: Optional[torch.Tensor] = None,
+    meta_v: Optional[torch.Tensor] = None,
 ):
     """Single-query window attention for each row of q [R, Hq, D].
+
+    meta_k/meta_v [M, Hkv, D]: meta (sink) tokens every row also attends to, unmasked, inside the same
+    softmax (key2/value2 of vllm_hymeta/attention/fa_kernel_metatoken.py:110-194, there a second
+    attention merged by log-sum-exp). bf16/fp16 caches with the fixed split only.
 
     new_key/new_value [R, Hkv, D] + new_slot_mapping [R] int64 (all three or none): the newest key
     of each row (index seq_lens[r]-1) is taken from these tensors and stored into the paged cache
@@ -208,6 +214,21 @@ def swa_decode_attention(
         fused = dict(new_key=N.ptr(new_key), new_value=N.ptr(new_value), new_slot_mapping=N.ptr(new_slot_mapping),
                      new_key_stride_row=new_key.stride(0), new_key_stride_head=new_key.stride(1),
                      new_value_stride_row=new_value.stride(0), new_value_stride_head=new_value.stride(1))
+    if meta_k is not None or meta_v is not None:
+        if meta_k is None or meta_v is None:
+            raise ValueError("meta_k and meta_v go together")
+        N.require_gpu(q, meta_k, meta_v)
+        if int8_kv or force_valu or q.dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError("meta tokens inside the decode launch need bf16/fp16 caches on the matrix-core "
+                                      "kernel (merge a separate meta_token_attention with lse_merge instead)")
+        if meta_k.dim() != 3 or meta_k.shape[1:] != (Hkv, D) or meta_v.shape != meta_k.shape or \
+                meta_k.dtype != q.dtype or meta_v.dtype != q.dtype or meta_k.stride() != meta_v.stride():
+            raise ValueError(f"meta_k and meta_v must be [meta_tokens, {Hkv}, {D}] of q's dtype with equal strides")
+        _inner_contiguous(meta_k, "meta_k")
+        if meta_k.shape[0] > 0:
+            fused.update(meta_k=N.ptr(meta_k), meta_v=N.ptr(meta_v), meta_len=meta_k.shape[0],
+                         meta_stride_row=meta_k.stride(0), meta_stride_head=meta_k.stride(1))
+            balanced = False
     if max_seq_len is None:
         max_seq_len = bound
     if window_left >= 0:

@@ -138,3 +138,102 @@ def test_meta_token_argument_errors(sb, dev):
         impl.forward(None, q, kv, kv, None, k2[:16], k2[:16], runner.kv_caches[0], meta, output=out)
     with pytest.raises(ValueError):
         sb.ops.lse_merge(out, torch.zeros(8, HQ, device=dev), out[:4], torch.zeros(8, HQ, device=dev))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n_split,M", [(1, 128), (4, 128), (3, 100), (4, 1), (2, 33), (5, 200), (0, 128)])
+def test_decode_launch_takes_meta_tokens_into_its_softmax(sb, dev, dtype, n_split, M):
+    """meta_k/meta_v inside sb_swa_decode: the meta rows' chunks are dealt to the splits of each row's
+    window. Against the one-softmax oracle; and against the two-attention form the reference uses
+    (window attention, meta attention, log-sum-exp merge) computed by this library's own ops. Rows:
+    short, window-saturated, one with an empty window (key_lo past its keys: the meta rows alone);
+    with and without the fused append."""
+    bs, wl = 16, 300
+    lens = [1, 17, 300, 301, 640, 1000, 33]
+    R = len(lens)
+    g = torch.Generator().manual_seed(M + n_split)
+    nblk = [(L + bs - 1) // bs for L in lens]
+    nb = sum(nblk) + 3
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(R, max(nblk), dtype=torch.int32)
+    p0 = 0
+    for r in range(R):
+        tables[r, :nblk[r]] = perm[p0:p0 + nblk[r]]
+        p0 += nblk[r]
+    kc = torch.randn(nb, bs, HKV, D, generator=g).to(dtype)
+    vc = torch.randn(nb, bs, HKV, D, generator=g).to(dtype)
+    q = torch.randn(R, HQ, D, generator=g).to(dtype)
+    k2 = torch.randn(M, HKV, D, generator=g).to(dtype)
+    v2 = torch.randn(M, HKV, D, generator=g).to(dtype)
+    key_lo = torch.zeros(R, dtype=torch.int32)
+    key_lo[6] = lens[6]                      # nothing of this row's window is visible
+    seq = torch.tensor(lens, dtype=torch.int32)
+
+    def keys_of(r, cache):
+        rows = [cache[tables[r, i // bs], i % bs] for i in range(lens[r])]
+        return torch.stack(rows).float().numpy()
+
+    ref = np.zeros((R, HQ, D))
+    for r in range(R):
+        k1, v1 = keys_of(r, kc), keys_of(r, vc)
+        lo = int(key_lo[r])
+        k1, v1 = k1[lo:], v1[lo:]
+        if len(k1) == 0:   # a query with no window keys: plain softmax over the meta rows alone
+            for h in range(HQ):
+                ref[r, h] = A.masked_softmax_attention(q[r:r + 1, h].double().numpy(), k2[:, h // (HQ // HKV)].double().numpy(),
+                                                       v2[:, h // (HQ // HKV)].double().numpy(), np.zeros((1, M), bool),
+                                                       D ** -0.5)[0]
+        else:
+            ref[r] = A.metatoken_attention(q[r:r + 1].float().numpy(), None, k1, k2.float().numpy(), v1, v2.float().numpy(),
+                                           D ** -0.5, wl + 1)[0]
+    args = dict(block_table=tables.to(dev), window_left=wl, key_lo=key_lo.to(dev), n_split=n_split, max_seq_len=max(lens))
+    out = sb.ops.swa_decode_attention(q.to(dev), kc.to(dev), vc.to(dev), seq.to(dev), meta_k=k2.to(dev), meta_v=v2.to(dev), **args)
+    got = out.float().cpu().numpy()
+    assert np.abs(got - ref).max() <= TOL
+    # the reference's form: two attentions merged by their log-sum-exp
+    o1, l1 = sb.ops.swa_decode_attention(q.to(dev), kc.to(dev), vc.to(dev), seq.to(dev), return_lse=True, **args)
+    o2, l2 = sb.ops.meta_token_attention(q.to(dev), k2.to(dev), v2.to(dev))
+    sb.ops.lse_merge(o1, l1, o2, l2)
+    assert np.abs(got - o1.float().cpu().numpy()).max() <= TOL
+    # the log-sum-exp of the one softmax equals the merged one
+    _, lse = sb.ops.swa_decode_attention(q.to(dev), kc.to(dev), vc.to(dev), seq.to(dev), meta_k=k2.to(dev), meta_v=v2.to(dev),
+                                         return_lse=True, **args)
+    assert torch.allclose(lse, l1, atol=2e-3, rtol=1e-4)
+
+
+def test_meta_tokens_with_fused_append_and_rejections(sb, dev):
+    bs, wl, M, R = 16, 64, 128, 5
+    g = torch.Generator().manual_seed(5)
+    lens = [1, 16, 65, 100, 129]
+    nblk = [(L + bs - 1) // bs for L in lens]
+    nb = sum(nblk)
+    tables = torch.zeros(R, max(nblk), dtype=torch.int32)
+    p0 = 0
+    for r in range(R):
+        tables[r, :nblk[r]] = torch.arange(p0, p0 + nblk[r])
+        p0 += nblk[r]
+    kc = torch.randn(nb, bs, HKV, D, generator=g).bfloat16()
+    vc = torch.randn(nb, bs, HKV, D, generator=g).bfloat16()
+    q = torch.randn(R, HQ, D, generator=g).bfloat16().to(dev)
+    k2 = torch.randn(M, HKV, D, generator=g).bfloat16().to(dev)
+    v2 = torch.randn(M, HKV, D, generator=g).bfloat16().to(dev)
+    slots = torch.tensor([int(tables[r, (lens[r] - 1) // bs]) * bs + (lens[r] - 1) % bs for r in range(R)])
+    newk = torch.stack([kc.view(-1, HKV, D)[s] for s in slots]).to(dev)
+    newv = torch.stack([vc.view(-1, HKV, D)[s] for s in slots]).to(dev)
+    seq = torch.tensor(lens, dtype=torch.int32, device=dev)
+    args = dict(block_table=tables.to(dev), window_left=wl, n_split=2, max_seq_len=max(lens), meta_k=k2, meta_v=v2)
+    want = sb.ops.swa_decode_attention(q, kc.to(dev), vc.to(dev), seq, **args)
+    # the same step with the newest rows missing from the cache and appended by the launch itself
+    kd, vd = kc.clone(), vc.clone()
+    kd.view(-1, HKV, D)[slots] = float("nan")
+    vd.view(-1, HKV, D)[slots] = float("nan")
+    kd, vd = kd.to(dev), vd.to(dev)
+    got = sb.ops.swa_decode_attention(q, kd, vd, seq, new_key=newk, new_value=newv, new_slot_mapping=slots.to(dev), **args)
+    assert (got.float() - want.float()).abs().max().item() <= TOL
+    assert torch.equal(kd.cpu(), kc) and torch.equal(vd.cpu(), vc)
+    with pytest.raises(NotImplementedError):
+        sb.ops.swa_decode_attention(q.float(), kc.float().to(dev), vc.float().to(dev), seq, block_table=tables.to(dev),
+                                    window_left=wl, meta_k=k2.float(), meta_v=v2.float())
+    with pytest.raises(ValueError):
+        sb.ops.swa_decode_attention(q, kc.to(dev), vc.to(dev), seq, block_table=tables.to(dev), window_left=wl,
+                                    meta_k=k2[:, :2], meta_v=v2[:, :2])
