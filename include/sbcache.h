@@ -338,6 +338,15 @@ typedef struct sb_swa_prefill_args {
   const float *v_scale;
   int32_t kv_quant;
   float k_scale_tensor, v_scale_tensor;
+  /* Meta (sink) tokens, as for sb_swa_decode (fa_kernel_metatoken.py:235-279: the varlen attention, a
+   * second non-causal attention of all queries over k2/v2, and the log-sum-exp merge): every query
+   * also attends, unmasked, to the meta_len rows of meta_k / meta_v ([meta_len, num_kv_heads, 128] of
+   * dtype, strides in elements); their 32-row chunks are walked in front of each tile's window chunks,
+   * inside the same softmax, and lse covers both. meta_len = 0 = off. Not over a byte-code cache. */
+  const void *meta_k;
+  const void *meta_v;
+  int32_t meta_len;
+  int64_t meta_stride_row, meta_stride_head;
 } sb_swa_prefill_args;
 
 int sb_swa_prefill(const sb_swa_prefill_args *args);

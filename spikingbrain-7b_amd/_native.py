@@ -99,6 +99,7 @@ class SwaPrefillArgs(C.Structure):
         ("block_table_stride", i64),
         ("stream", vp), ("lse", vp), ("k_scale", vp), ("v_scale", vp), ("kv_quant", i32),
         ("k_scale_tensor", f32), ("v_scale_tensor", f32),
+        ("meta_k", vp), ("meta_v", vp), ("meta_len", i32), ("meta_stride_row", i64), ("meta_stride_head", i64),
     ]
 
 

@@ -61,9 +61,15 @@ struct PrefillParams {
   int64_t q_sr, q_sh, o_sr, o_sh;  // elements
   int64_t kv_sb, kv_sr, kv_sh;     // bytes
   int64_t bt_stride;
+  // Meta tokens (element caches only): meta_len rows [meta_len, Hkv, 128] every query also attends to,
+  // unmasked, in the same softmax: they are walked as the chunks in front of the window's. 0 = none.
+  const char *meta_k;
+  const char *meta_v;
+  int meta_len;
+  int64_t meta_sr, meta_sh;  // bytes
 };
 
-constexpr int kRowPad = 272;          // LDS row stride: 256 B of data + 16 B
+constexpr int kRowPad = 272;         // LDS row stride: 256 B of data + 16 B
 constexpr int kStage = 32 * kRowPad;  // one K or V chunk
 constexpr float kNegInf = kNegInfF;
 constexpr float kRaise = 8.f;
@@ -146,6 +152,9 @@ void swa_prefill_kernel(const PrefillParams p) {
   const int wg_lo = min(max(wl >= 0 ? shift + q0 - wl : 0, klo), wg_hi - 1);
   const int first_tile = wg_lo >> 4, last_tile = (wg_hi - 1) >> 4;
   const int ch_begin = wg_lo >> 5, ch_end = ((wg_hi - 1) >> 5) + 1;
+  // The walk: the meta rows' chunks first (walk index x < nm), then window chunk ch_begin + x - nm.
+  const int nm = KVQ == SB_KV_NONE ? (p.meta_len + 31) >> 5 : 0;
+  const int n_walk = nm + ch_end - ch_begin;
 
   // this wavefront's two column blocks: 16-token sub-tile ts[b] of head hd[b]
   int ts[2], hd[2];
@@ -207,8 +216,21 @@ void swa_prefill_kernel(const PrefillParams p) {
   const int rows_per_wave = 32 / S::kFetchWaves;                         // 8 or 16
   const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the 16-key tile, +4 per load
   using Set = StageSet<KVQ, S::kLoads>;
-  Set stage[2];  // chunk x travels in set (x - ch_begin) & 1
-  auto fetch = [&](int ch, Set &st) {
+  Set stage[2];  // walk index x travels in set x & 1
+  auto fetch = [&](int x, Set &st) {
+    if constexpr (KVQ == SB_KV_NONE) {
+      if (x < nm) {  // meta chunk: dense rows shared by every sequence, clamped to the last one
+        const int64_t moff = (int64_t)kvh * p.meta_sh + c * 16;
+#pragma unroll
+        for (int u = 0; u < S::kLoads; ++u) {
+          const int row = min((x << 5) + wave * rows_per_wave + (lane >> 4) + 4 * u, p.meta_len - 1);
+          st.k[u] = *reinterpret_cast<const uint4 *>(p.meta_k + moff + (int64_t)row * p.meta_sr);
+          st.v[u] = *reinterpret_cast<const uint4 *>(p.meta_v + moff + (int64_t)row * p.meta_sr);
+        }
+        return;
+      }
+    }
+    const int ch = ch_begin + x - nm;
     const int t = min(max(2 * ch + (wave * rows_per_wave) / 16, first_tile), last_tile);
     const int64_t base = tile_base(t);
 #pragma unroll
@@ -256,7 +278,9 @@ void swa_prefill_kernel(const PrefillParams p) {
   float mx[2];     // their row maxima, in log2 units
 
   // scores of chunk `ch` for both column blocks; true when some row needs a higher reference point
-  auto scores = [&](int ch, int buf) -> bool {
+  auto scores = [&](int x, int buf) -> bool {
+    const bool is_meta = x < nm;
+    const int ch = is_meta ? x : ch_begin + x - nm;
     const char *sk = smem + buf * 2 * kStage;
     uint4 k0[4], k1[4];
 #pragma unroll
@@ -266,7 +290,9 @@ void swa_prefill_kernel(const PrefillParams p) {
     }
     const int c0 = ch << 5;
     // wholly visible to all tokens of the wavefront: above every lower bound, at or below the first token
-    const bool full = (wl < 0 || c0 >= shift + jw_last - wl) && c0 >= klo && (c0 + 31 <= shift + jw0);
+    // (a meta chunk: every row that exists is visible to every token)
+    const bool full = is_meta ? c0 + 32 <= p.meta_len
+                              : (wl < 0 || c0 >= shift + jw_last - wl) && c0 >= klo && (c0 + 31 <= shift + jw0);
     bool raise = false;
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
@@ -285,7 +311,7 @@ void swa_prefill_kernel(const PrefillParams p) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int i = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-          if (i > my_pos[b] || i < my_lo[b]) sc[b][j] = kNegInf;
+          if (is_meta ? i >= p.meta_len : (i > my_pos[b] || i < my_lo[b])) sc[b][j] = kNegInf;
         }
       }
       // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
@@ -360,17 +386,17 @@ void swa_prefill_kernel(const PrefillParams p) {
     __syncthreads();
   };
   if (fetcher) {
-    fetch(ch_begin, stage[0]);
-    fetch(ch_begin + 1, stage[1]);
+    fetch(0, stage[0]);
+    fetch(1, stage[1]);
     stash(0, stage[0]);
   }
   __syncthreads();
-  int ch = ch_begin;
-  for (; ch + 1 < ch_end; ch += 2) {
-    body(ch, std::integral_constant<int, 0>{});
-    body(ch + 1, std::integral_constant<int, 1>{});
+  int x = 0;
+  for (; x + 1 < n_walk; x += 2) {
+    body(x, std::integral_constant<int, 0>{});
+    body(x + 1, std::integral_constant<int, 1>{});
   }
-  if (ch < ch_end) body(ch, std::integral_constant<int, 0>{});
+  if (x < n_walk) body(x, std::integral_constant<int, 0>{});
 
   // ---- epilogue: lane (g, c) owns token c of each block, dims 32g + 8i + mt ---------------------
 #pragma unroll
@@ -469,6 +495,20 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   p.k_scale_tensor = a->k_scale_tensor; p.v_scale_tensor = a->v_scale_tensor; p.Hkv = a->num_kv_heads;
   p.bt_stride = a->block_table_stride;
   p.num_tiles = (int)a->num_tiles;
+  p.meta_k = p.meta_v = nullptr;
+  p.meta_len = 0;
+  p.meta_sr = p.meta_sh = 0;
+  if (a->meta_len < 0) return fail(SB_ERR_INVALID, "sb_swa_prefill: negative meta_len");
+  if (a->meta_len > 0) {
+    if (!a->meta_k || !a->meta_v) return fail(SB_ERR_INVALID, "sb_swa_prefill: meta_len without meta_k / meta_v");
+    if (codes) return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: meta tokens are not taken over a byte-code cache");
+    if (((reinterpret_cast<uintptr_t>(a->meta_k) | reinterpret_cast<uintptr_t>(a->meta_v)) & 15u) ||
+        (a->meta_stride_row * 2) % 16 || (a->meta_stride_head * 2) % 16)
+      return fail(SB_ERR_INVALID, "sb_swa_prefill: meta rows must be 16-byte aligned");
+    p.meta_k = (const char *)a->meta_k; p.meta_v = (const char *)a->meta_v;
+    p.meta_len = a->meta_len;
+    p.meta_sr = a->meta_stride_row * 2; p.meta_sh = a->meta_stride_head * 2;
+  }
 
   const dim3 grid((unsigned)((a->num_tiles + 7) / 8 * 8), (unsigned)a->num_kv_heads);
   for (int h0 = 0; h0 < p.G; h0 += 4) {  // a GQA group is covered 4 heads at a time

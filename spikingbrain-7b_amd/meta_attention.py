@@ -528,9 +528,15 @@ class MetaAttentionImpl:
         prefill_output = output[num_meta_prefill_tokens - num_prefill_query_tokens:num_meta_prefill_tokens]
         decode_output = output[num_meta_prefill_tokens:]
 
+        # Over bf16/fp16 keys the kernels take the meta rows into their own softmax (meta_k/meta_v); over
+        # a byte-code cache they are a second attention merged by log-sum-exp, the reference's own form.
+        meta_inside = with_meta and not byte_kv and query.dtype in (torch.bfloat16, torch.float16)
+        meta_kv = dict(meta_k=key2, meta_v=value2) if meta_inside else {}
+        want_lse = with_meta and not meta_inside
+
         def merge_meta(q_part, out_part, lse_part):
             """out_part (attention over the window, log-sum-exp lse_part) takes in the meta tokens."""
-            if with_meta and q_part.shape[0] > 0:
+            if want_lse and q_part.shape[0] > 0:
                 meta_out, meta_lse = ops.meta_token_attention(q_part, key2, value2, self.scale)
                 ops.lse_merge(out_part, lse_part, meta_out, meta_lse)
 
@@ -548,7 +554,7 @@ class MetaAttentionImpl:
                 elif fp8_kv:  # scaled_fp8_quant of the prompt's keys and values (:853-869)
                     pk, pv = ops.fp8_round(pk.contiguous(), k_scale_f), ops.fp8_round(pv.contiguous(), v_scale_f)
                 lse = self._varlen_inflight(query, pk, pv, prefill_meta, prefill_output, window_left,
-                                            return_lse=with_meta)
+                                            return_lse=want_lse, meta_kv=meta_kv)
             else:
                 # prefix hit / chunked prefill: keys and values come from the paged cache (:885-919)
                 assert prefill_meta.seq_lens is not None
@@ -556,7 +562,7 @@ class MetaAttentionImpl:
                 lse = self._varlen_paged(query, key_cache, value_cache, prefill_meta.query_start_loc,
                                          prefill_meta.seq_lens_tensor, prefill_meta.block_tables,
                                          max(prefill_meta.seq_lens), prefill_output, window_left,
-                                         meta=prefill_meta, return_lse=with_meta, scales=scales)
+                                         meta=prefill_meta, return_lse=want_lse, scales=scales, meta_kv=meta_kv)
             merge_meta(query, prefill_output, lse)
         if decode_meta := attn_metadata.decode_metadata:
             assert decode_meta.max_decode_query_len is not None
@@ -566,7 +572,7 @@ class MetaAttentionImpl:
                 lse = self._varlen_paged(decode_query, key_cache, value_cache, decode_meta.query_start_loc,
                                          decode_meta.seq_lens_tensor, decode_meta.block_tables,
                                          decode_meta.max_decode_seq_len, decode_output, window_left,
-                                         meta=decode_meta, return_lse=with_meta, scales=scales)
+                                         meta=decode_meta, return_lse=want_lse, scales=scales, meta_kv=meta_kv)
             else:
                 # one query token per sequence (:954-981); K/V were appended above, or are appended
                 # by this very launch when the step is a pure decode step
@@ -581,20 +587,13 @@ class MetaAttentionImpl:
                         host_lens is not None and len(host_lens) >= n and
                         ops.plan_decode_split(n, self.num_kv_heads, decode_meta.max_decode_seq_len or max(host_lens[:n]),
                                               window_left, host_lens[:n]))
-                # meta tokens ride in the same launch (their chunks join each split's softmax) when the
-                # cache holds bf16/fp16 rows; over a byte-code cache they stay a second attention + merge
-                meta_inside = with_meta and not byte_kv and decode_query.dtype in (torch.bfloat16, torch.float16)
-                if meta_inside:
-                    fused.update(meta_k=key2, meta_v=value2)
                 res = ops.swa_decode_attention(
                     decode_query, key_cache, value_cache, decode_meta.seq_lens_tensor[:n],
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
-                    out=decode_output, return_lse=with_meta and not meta_inside,
+                    out=decode_output, return_lse=want_lse,
                     max_seq_len=decode_meta.max_decode_seq_len or None,
-                    balanced=False if byte_kv else decode_meta._decode_balanced, **scales, **fused)
-                if meta_inside:
-                    return output
-                lse = res[1] if with_meta else None
+                    balanced=False if byte_kv else decode_meta._decode_balanced, **scales, **fused, **meta_kv)
+                lse = res[1] if want_lse else None
             merge_meta(decode_query, decode_output, lse)
         return output
 
@@ -620,8 +619,10 @@ class MetaAttentionImpl:
             return None
         return plan
 
-    def _varlen_inflight(self, q, k, v, meta, out, window_left, return_lse=False):
-        """Returns the fp32 [T, Hq] log-sum-exp when asked for, else None."""
+    def _varlen_inflight(self, q, k, v, meta, out, window_left, return_lse=False, meta_kv=None):
+        """Returns the fp32 [T, Hq] log-sum-exp when asked for, else None. meta_kv: meta_k/meta_v for the
+        kernels to take into their softmax."""
+        meta_kv = meta_kv or {}
         T = q.shape[0]
         if T == 0:
             return None
@@ -632,7 +633,7 @@ class MetaAttentionImpl:
         if plan is not None and plan.total_k <= k.shape[0]:
             res = ops.swa_prefill_attention(q, k, v, plan=plan, window_left=window_left, scale=self.scale, out=out,
                                             kv_start=meta.seq_start_loc.to(torch.int64)[:-1].contiguous(),
-                                            return_lse=return_lse)
+                                            return_lse=return_lse, **meta_kv)
             return res[1] if return_lse else None
         row_seq, j, _ = self._rows(meta.query_start_loc, T)
         seq_lens_row = (j + 1).to(torch.int32)
@@ -640,13 +641,14 @@ class MetaAttentionImpl:
             q, k, v, seq_lens_row, kv_start=meta.seq_start_loc.to(torch.int64)[:-1].contiguous(),
             row_seq=row_seq.to(torch.int32), kv_strides=(0, k.stride(0), k.stride(1)),
             num_kv_heads=self.num_kv_heads, window_left=window_left, scale=self.scale, out=out,
-            max_seq_len=meta.max_prefill_seq_len or None, return_lse=return_lse)
+            max_seq_len=meta.max_prefill_seq_len or None, return_lse=return_lse, **meta_kv)
         return res[1] if return_lse else None
 
     def _varlen_paged(self, q, key_cache, value_cache, query_start_loc, seq_lens_tensor, block_tables,
-                      max_seq_len, out, window_left, meta=None, return_lse=False, scales=None):
+                      max_seq_len, out, window_left, meta=None, return_lse=False, scales=None, meta_kv=None):
         """scales: k_scale/v_scale of an INT8 cache or fp8_scales of an fp8 cache, passed on to whichever
-        kernel takes the step."""
+        kernel takes the step; meta_kv: meta_k/meta_v for that kernel to take into its softmax."""
+        meta_kv = meta_kv or {}
         T = q.shape[0]
         if T == 0:
             return None
@@ -655,7 +657,7 @@ class MetaAttentionImpl:
         if plan is not None and block_tables.shape[1] * key_cache.shape[1] >= plan.max_k:
             res = ops.swa_prefill_attention(q, key_cache, value_cache, plan=plan, block_table=block_tables,
                                             window_left=window_left, scale=self.scale, out=out, return_lse=return_lse,
-                                            **scales)
+                                            **scales, **meta_kv)
             return res[1] if return_lse else None
         row_seq, j, lens = self._rows(query_start_loc, T)
         # query j of a run of n queries in a sequence of L keys sits at key index L - n + j
@@ -663,5 +665,5 @@ class MetaAttentionImpl:
         res = ops.swa_decode_attention(
             q, key_cache, value_cache, seq_lens_row, block_table=block_tables, row_seq=row_seq.to(torch.int32),
             window_left=window_left, scale=self.scale, out=out, max_seq_len=max_seq_len or None,
-            return_lse=return_lse, **scales)
+            return_lse=return_lse, **scales, **meta_kv)
         return res[1] if return_lse else None

@@ -440,9 +440,13 @@ def swa_prefill_attention(
     k_scale: Optional[torch.Tensor] = None,
     v_scale: Optional[torch.Tensor] = None,
     fp8_scales: Optional[Tuple[float, float]] = None,
+    meta_k: Optional[torch.Tensor] = None,
+    meta_v: Optional[torch.Tensor] = None,
 ):
     """Causal sliding-window attention for q [total_q, Hq, D] packed sequence after sequence.
     With return_lse also the fp32 [total_q, Hq] natural-log log-sum-exp of each query's scores.
+    meta_k/meta_v [M, Hkv, D]: meta (sink) tokens every query also attends to, unmasked, in the same
+    softmax (not over byte-code caches).
 
     query_lens / seq_lens_k: per-sequence host ints (keys default to the queries: plain prompt), or a
     prebuilt `plan`. Query j of a sequence sits at key position seq_len_k - query_len + j.
@@ -533,6 +537,21 @@ def swa_prefill_attention(
     lse = torch.full((Tq, Hq), float("-inf"), dtype=torch.float32, device=dev) if return_lse else None
     if plan.num_tiles == 0:
         return (out, lse) if return_lse else out
+    meta = {}
+    if meta_k is not None or meta_v is not None:
+        if meta_k is None or meta_v is None:
+            raise ValueError("meta_k and meta_v go together")
+        N.require_gpu(q, meta_k, meta_v)
+        if kv_quant != N.SB_KV_NONE:
+            raise NotImplementedError("meta tokens are not taken over a byte-code cache (merge a separate "
+                                      "meta_token_attention with lse_merge instead)")
+        if meta_k.dim() != 3 or meta_k.shape[1:] != (Hkv, D) or meta_v.shape != meta_k.shape or \
+                meta_k.dtype != q.dtype or meta_v.dtype != q.dtype or meta_k.stride() != meta_v.stride():
+            raise ValueError(f"meta_k and meta_v must be [meta_tokens, {Hkv}, {D}] of q's dtype with equal strides")
+        _inner_contiguous(meta_k, "meta_k")
+        if meta_k.shape[0] > 0:
+            meta = dict(meta_k=N.ptr(meta_k), meta_v=N.ptr(meta_v), meta_len=meta_k.shape[0],
+                        meta_stride_row=meta_k.stride(0), meta_stride_head=meta_k.stride(1))
     a = N.SwaPrefillArgs(
         q=N.ptr(q), k=N.ptr(k), v=N.ptr(v), out=N.ptr(out),
         block_table=N.ptr(block_table), kv_start=N.ptr(kv_start) if block_table is None else None,
@@ -546,7 +565,7 @@ def swa_prefill_attention(
         block_table_stride=bt_stride, stream=N.stream_ptr(dev), lse=N.ptr(lse),
         k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale), kv_quant=kv_quant,
         k_scale_tensor=float(fp8_scales[0]) if fp8_scales is not None else 0.0,
-        v_scale_tensor=float(fp8_scales[1]) if fp8_scales is not None else 0.0)
+        v_scale_tensor=float(fp8_scales[1]) if fp8_scales is not None else 0.0, **meta)
     N.check(N.lib().sb_swa_prefill(C.byref(a)), "swa_prefill")
     return (out, lse) if return_lse else out
 

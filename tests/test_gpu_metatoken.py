@@ -237,3 +237,40 @@ def test_meta_tokens_with_fused_append_and_rejections(sb, dev):
     with pytest.raises(ValueError):
         sb.ops.swa_decode_attention(q, kc.to(dev), vc.to(dev), seq, block_table=tables.to(dev), window_left=wl,
                                     meta_k=k2[:, :2], meta_v=v2[:, :2])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,wl", [(128, 40), (33, 300), (1, -1), (64, 40)])
+def test_many_query_kernel_takes_meta_tokens_into_its_softmax(sb, dev, dtype, M, wl):
+    """meta_k/meta_v inside sb_swa_prefill: the meta chunks are walked in front of each tile's window
+    chunks. Ragged prompts, some with earlier context (their queries are the last tokens of a longer key
+    run); against the one-softmax oracle, and the log-sum-exp against this library's two-attention form."""
+    qlens = [5, 64, 100, 257, 1]
+    ctx = [0, 30, 0, 200, 77]
+    klens = [a + b for a, b in zip(qlens, ctx)]
+    g = torch.Generator().manual_seed(M + max(wl, 0))
+    Tq, Tk = sum(qlens), sum(klens)
+    q = torch.randn(Tq, HQ, D, generator=g).to(dtype)
+    k = torch.randn(Tk, HKV, D, generator=g).to(dtype)
+    v = torch.randn(Tk, HKV, D, generator=g).to(dtype)
+    k2 = torch.randn(M, HKV, D, generator=g).to(dtype)
+    v2 = torch.randn(M, HKV, D, generator=g).to(dtype)
+    kstart = torch.tensor([sum(klens[:i]) for i in range(len(klens))], dtype=torch.int64)
+    args = dict(query_lens=qlens, seq_lens_k=klens, kv_start=kstart.to(dev), window_left=wl)
+    out, lse = sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), meta_k=k2.to(dev), meta_v=v2.to(dev),
+                                            return_lse=True, **args)
+    got = out.float().cpu().numpy()
+    qo = 0
+    for i, (lq, lk) in enumerate(zip(qlens, klens)):
+        ks = int(kstart[i])
+        ref = A.metatoken_attention(q[qo:qo + lq].float().numpy(), None, k[ks:ks + lk].float().numpy(), k2.float().numpy(),
+                                    v[ks:ks + lk].float().numpy(), v2.float().numpy(), D ** -0.5, wl + 1 if wl >= 0 else 0)
+        assert np.abs(got[qo:qo + lq] - ref).max() <= TOL, i
+        qo += lq
+    o1, l1 = sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), return_lse=True, **args)
+    o2, l2 = sb.ops.meta_token_attention(q.to(dev), k2.to(dev), v2.to(dev))
+    sb.ops.lse_merge(o1, l1, o2, l2)
+    assert np.abs(got - o1.float().cpu().numpy()).max() <= TOL
+    assert torch.allclose(lse, l1, atol=2e-3, rtol=1e-4)
+    with pytest.raises(ValueError):
+        sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), meta_k=k2.to(dev), **args)
