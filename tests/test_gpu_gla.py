@@ -284,7 +284,7 @@ def test_block_form_strong_gates_and_gate_dtypes(sb, dev, gdtype):
     assert out_close(o.float().cpu().numpy(), ref_o)
 
 
-@pytest.mark.parametrize("gdtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("gdtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T", [4, 9, 24])
 def test_step_by_step_prompt_kernel_every_element_type(sb, dev, dtype, gdtype, T):
