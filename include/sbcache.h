@@ -111,9 +111,12 @@ int sb_kv_append(const sb_kv_append_args *args);
 #define SB_KV_FP8 2
 #define SB_DECODE_FORCE_VALU 1 /* bf16/fp16: use the vector-ALU split kernel instead of the matrix-core one */
 /* bf16/fp16, n_split > 1, up to 1024 rows: cut the chunks of ALL rows, laid end to end, into equal runs
- * (about one per CU) instead of cutting every row into n_split runs, so that rows of different
- * lengths leave no workgroup idle (up to 2x faster on ragged batches, about 5 % slower on even ones:
- * see sb_swa_decode_prefer_balanced). Same results up to fp32 summation order; same workspace size. */
+ * (one per CU) instead of cutting every row into n_split runs, so that neither rows of different lengths
+ * nor a row count that fits the CUs badly (96 rows x 3 splits = 256 + 32 workgroups) leave CUs idle:
+ * up to 2x faster on ragged batches, 20-30 % on even batches of such sizes, about 5 % slower where
+ * rows x splits fills the CUs exactly (see sb_swa_decode_prefer_balanced). Same results up to fp32
+ * summation order; same workspace size. Pass n_split = 2 when the fixed split would not split at all
+ * (the balanced split always goes through partial results and the merge). */
 #define SB_DECODE_BALANCED 2
 
 typedef struct sb_swa_decode_args {
@@ -182,11 +185,14 @@ typedef struct sb_swa_decode_args {
   int64_t meta_stride_row, meta_stride_head;
 } sb_swa_decode_args;
 
-/* Split count the auto rule (n_split = 0) would use for these shapes. */
+/* Split count the auto rule (n_split = 0) would use for these shapes: the one with the lowest estimated
+ * duration, counting the rounds in which rows x splits workgroups pass over the CUs (one at a time per CU). */
 int32_t sb_swa_decode_auto_split(int64_t num_rows, int32_t num_kv_heads, int32_t max_seq_len,
                                  int32_t window_left);
-/* 1 if SB_DECODE_BALANCED is expected to be faster for rows with these lengths, else 0.
- * host_seq_lens: the step's seq_lens as a HOST array (the scheduler has them); no device access. */
+/* 1 if SB_DECODE_BALANCED is expected to be faster than the fixed split into n_split (>= 1) parts for rows
+ * with these lengths, else 0. host_seq_lens: the step's seq_lens as a HOST array (the scheduler has them;
+ * a caller without them can pass max_seq_len for every row: the balanced split adapts to the real lengths
+ * on the device); no device access. */
 int32_t sb_swa_decode_prefer_balanced(const int32_t *host_seq_lens, int64_t num_rows, int32_t window_left,
                                       int32_t n_split);
 

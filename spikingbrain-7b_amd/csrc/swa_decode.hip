@@ -14,6 +14,11 @@
 //   (registers -> LDS), then either normalised and stored (n_split == 1) or written as an
 //   fp32 partial (m, l, acc) that swa_decode_merge_kernel combines.
 //   Scores are kept in log2 units: p = exp2(s*scale*log2e - m).
+#include <algorithm>
+#include <functional>
+#include <queue>
+#include <vector>
+
 #include "common.h"
 #include "swa_decode_params.h"
 
@@ -480,35 +485,62 @@ static int device_cu_count() {
   return cus;
 }
 
+// Cost model of a split launch, in units of one 32-key chunk streamed by one workgroup while every CU is
+// busy (about 2.5 us), fitted to launches of 16 .. 384 window-saturated rows of the 7B shape:
+//   fixed split    : rounds of workgroups over the CUs (one workgroup fits a CU at a time), each round
+//                    costing its workgroups' chunks + kFixedChunks (start-up chain, partial result, launch
+//                    and merge share); a last round that fills only part of the CUs runs up to 40 % faster;
+//   balanced split : one run per CU + kBalancedChunks + rows / kBalancedRowsPerChunk (every wavefront adds
+//                    up all rows' lengths, and the merge reads one more partial per row).
+constexpr double kFixedChunks = 7.0;
+constexpr double kBalancedChunks = 8.0;
+constexpr double kBalancedRowsPerChunk = 25.0;
+
+static double round_cost(double chunks_per_wg, int64_t active, int64_t cus) {
+  const double fill = active >= cus ? 1.0 : (double)active / (double)cus;
+  return (chunks_per_wg + kFixedChunks) * (0.6 + 0.4 * fill);
+}
+
+// Estimated duration of a fixed split of `wgs` (row, kv-head group) pairs of `chunks` chunks each into n
+// parts on `cus` CUs.
+static double split_cost(int64_t wgs, int64_t n, int64_t chunks, int64_t cus) {
+  const int64_t total = wgs * n, full = total / cus, rest = total % cus;
+  const double per_wg = (double)((chunks + n - 1) / n);
+  return (double)full * round_cost(per_wg, cus, cus) + (rest ? round_cost(per_wg, rest, cus) : 0.0);
+}
+
 extern "C" int32_t sb_swa_decode_auto_split(int64_t num_rows, int32_t num_kv_heads,
                                             int32_t max_seq_len, int32_t window_left) {
   if (num_rows <= 0 || num_kv_heads <= 0 || max_seq_len <= 0) return 1;
   int64_t keys = max_seq_len;
   if (window_left >= 0 && keys > (int64_t)window_left + 1) keys = (int64_t)window_left + 1;
   const int64_t chunks = (keys + 31) / 32 + 1;  // +1: an unaligned window touches one more chunk
-  // A split is one workgroup per (row, group of up to 4 kv heads). All workgroups of a launch are
-  // resident at once and each streams at the same rate, so the launch is fastest when their
-  // number is a whole multiple of the CU count: take the split count that brings it nearest to
-  // one workgroup per CU, but leave every workgroup at least 8 chunks (256 keys) of work so that
-  // filling its load pipeline and writing its partial result stay small next to the streaming.
+  // A split is one workgroup per (row, group of up to 4 kv heads). Take the split count with the lowest
+  // estimated duration (rows x splits just above a multiple of the CU count pay a whole extra round),
+  // leaving every workgroup at least 8 chunks (256 keys) so that its fixed cost stays small next to the
+  // streaming; ties go to more splits (more CUs streaming).
   const int64_t wgs = num_rows * ((num_kv_heads + 3) / 4);
   const int64_t cus = device_cu_count();
-  int64_t n = (cus + wgs / 2) / wgs;
-  const int64_t cap = chunks / 8;
-  if (n > cap) n = cap;
-  if (n > 64) n = 64;
-  if (n < 1) n = 1;
-  return (int32_t)n;
+  int64_t cap = chunks / 8;
+  if (cap > 64) cap = 64;
+  if (cap < 1) cap = 1;
+  int64_t best = 1;
+  double best_cost = split_cost(wgs, 1, chunks, cus);
+  for (int64_t n = 2; n <= cap; ++n) {
+    const double c = split_cost(wgs, n, chunks, cus);
+    if (c <= best_cost) { best = n; best_cost = c; }
+  }
+  return (int32_t)best;
 }
 
 // Rows up to which the balanced split is used (every wavefront sums over all rows' lengths).
 constexpr int64_t kBalancedMaxRows = 1024;
 
-// Workgroups per kv-head group of the balanced split: one per CU when the fixed split would have
-// launched about that many anyway, else as many as the fixed split.
+// Workgroups per kv-head group of the balanced split: one per CU (a CU holds one at a time), fewer only
+// when the fixed split would have launched less than half as many (very little work).
 static int64_t balanced_workgroups(int64_t num_rows, int64_t n_split) {
   const int64_t fixed = num_rows * n_split, cus = device_cu_count();
-  return (fixed * 2 >= cus && fixed <= cus * 2) ? cus : fixed;
+  return fixed * 2 >= cus ? cus : fixed;
 }
 
 // Partials of a launch: rows * n_split for the fixed split; the balanced split numbers them
@@ -522,21 +554,33 @@ static int64_t partial_slots(int64_t num_rows, int64_t n_split) {
 
 extern "C" int32_t sb_swa_decode_prefer_balanced(const int32_t *host_seq_lens, int64_t num_rows,
                                                  int32_t window_left, int32_t n_split) {
-  if (!host_seq_lens || num_rows <= 0 || num_rows > kBalancedMaxRows || n_split <= 1) return 0;
-  int64_t total = 0, longest = 0;
+  if (!host_seq_lens || num_rows <= 0 || num_rows > kBalancedMaxRows || n_split < 1) return 0;
+  const int64_t cus = device_cu_count();
+  std::vector<int64_t> chunks((size_t)num_rows);
+  int64_t total = 0;
   for (int64_t r = 0; r < num_rows; ++r) {
     const int64_t hi = host_seq_lens[r];
     const int64_t lo = (window_left >= 0 && hi - 1 - window_left > 0) ? hi - 1 - window_left : 0;
-    const int64_t n = hi > lo ? ((hi - 1) >> 5) - (lo >> 5) + 1 : 0;
-    total += n;
-    if (n > longest) longest = n;
+    chunks[r] = hi > lo ? ((hi - 1) >> 5) - (lo >> 5) + 1 : 0;
+    total += chunks[r];
   }
-  const int64_t n_wg = balanced_workgroups(num_rows, n_split);
-  const int64_t fixed_run = (longest + n_split - 1) / n_split;  // chunks of the busiest workgroup
-  const int64_t balanced_run = (total + n_wg - 1) / n_wg;
-  // Working out the runs and restarting at a row boundary cost a balanced workgroup about as much
-  // as streaming 4 chunks (measured: even batches are 5 % faster with the fixed split).
-  return balanced_run + 4 < fixed_run ? 1 : 0;
+  // Fixed split: its workgroups (split-major, rows fastest: the dispatch order) handed to the CUs as
+  // these fall free, one workgroup per CU at a time; each costs its chunks plus the fixed part.
+  std::priority_queue<double, std::vector<double>, std::greater<double>> free_at;
+  for (int64_t c = 0; c < cus; ++c) free_at.push(0.0);
+  double fixed_end = 0.0;
+  for (int64_t s = 0; s < n_split; ++s)
+    for (int64_t r = 0; r < num_rows; ++r) {
+      const int64_t cps = (chunks[r] + n_split - 1) / n_split;
+      const int64_t mine = std::max<int64_t>(0, std::min(cps, chunks[r] - s * cps));
+      const double end = free_at.top() + (double)mine + kFixedChunks;
+      free_at.pop();
+      free_at.push(end);
+      if (end > fixed_end) fixed_end = end;
+    }
+  const int64_t n_wg = balanced_workgroups(num_rows, n_split < 2 ? 2 : n_split);
+  const double balanced_end = (double)((total + n_wg - 1) / n_wg) + kBalancedChunks + (double)num_rows / kBalancedRowsPerChunk;
+  return balanced_end < fixed_end ? 1 : 0;
 }
 
 extern "C" size_t sb_swa_decode_workspace_bytes(int64_t num_rows, int32_t num_q_heads,

@@ -237,8 +237,22 @@ def swa_decode_attention(
     auto_balance = balanced is None
     if n_split == 0:
         n_split = L.sb_swa_decode_auto_split(R, Hkv, int(max_seq_len), int(window_left))
+    can_balance = (q.dtype in (torch.bfloat16, torch.float16) and not int8_kv and not force_valu and R <= 1024
+                   and "meta_k" not in fused)
     if auto_balance:
-        balanced = prefer_balanced_split(host_seq_lens, window_left, n_split) if host_seq_lens is not None else False
+        # from the rows' lengths when the caller has them on the host, else as if every row were as long as
+        # max_seq_len (the balanced split adapts to the real lengths on the device either way)
+        if not can_balance:
+            balanced = False
+        elif host_seq_lens is not None:
+            balanced = prefer_balanced_split(host_seq_lens, window_left, n_split)
+        else:
+            key = (R, int(max_seq_len), int(window_left), int(n_split))
+            balanced = _SHAPE_POLICY.get(key)
+            if balanced is None:
+                balanced = _SHAPE_POLICY[key] = prefer_balanced_split([int(max_seq_len)] * R, window_left, n_split)
+    if balanced and can_balance and n_split < 2:
+        n_split = 2  # the balanced split always goes through partial results and the merge
     ws_bytes = L.sb_swa_decode_workspace_bytes(R, Hq, D, n_split)
     ws = _workspace(dev, ws_bytes)
     a = N.SwaDecodeArgs(
@@ -369,11 +383,14 @@ def quantize_sym(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.T
     return out
 
 
+_SHAPE_POLICY: dict = {}  # (rows, max_seq_len, window_left, n_split) -> balanced, for calls without host lengths
+
+
 def prefer_balanced_split(host_seq_lens, window_left: int, n_split: int) -> bool:
     """Whether the balanced split is expected to beat the fixed one for rows of these lengths
     (host ints; no device access)."""
     n = len(host_seq_lens)
-    if n == 0 or n_split <= 1:
+    if n == 0 or n_split < 1:
         return False
     arr = (C.c_int32 * n)(*[int(x) for x in host_seq_lens])
     return bool(N.lib().sb_swa_decode_prefer_balanced(arr, n, int(window_left), int(n_split)))

@@ -89,8 +89,16 @@ def test_balanced_split_policy_and_workspace(sb):
     assert prefer([4097 + 16 * i for i in range(64)], 4096, 4) == 0          # all rows fill the window
     assert prefer([32768] + [256] * 31, -1, 8) == 1                          # one long row among short ones
     assert prefer([100 + 120 * i for i in range(64)], -1, 4) == 1            # lengths spread over 100..7660
-    assert prefer([5000] * 8, 4096, 1) == 0                                  # nothing to balance without a split
+    assert prefer([5000] * 8, 4096, 1) == 1                                  # 8 unsplit rows leave 248 CUs idle
     assert prefer([], 4096, 4) == 0
+    # even batches: the fixed split where rows x splits fills whole rounds of the 256 CUs, the balanced one
+    # where the last round would be mostly empty or there would be several rounds
+    auto = lambda rows: L.sb_swa_decode_auto_split(rows, 4, 8000, 4096)
+    for rows, want in ((16, 0), (64, 0), (128, 0), (256, 0), (512, 0), (96, 1), (192, 1), (200, 1), (300, 1)):
+        assert prefer([8000] * rows, 4096, auto(rows)) == want, rows
+    assert prefer([8000] * 2048, 4096, 1) == 0                               # beyond the balanced kernel's row limit
+    # the split count avoids a nearly empty extra round: 96 rows x 3 = 288 workgroups would run 256 + 32
+    assert auto(96) == 5 and auto(80) == 3 and auto(48) == 5 and auto(32) == 8 and auto(128) == 2
     # balanced numbering: (workgroups, here one per CU = 256) + rows partial slots per head
     assert L.sb_swa_decode_workspace_bytes(48, 28, 128, 5) >= (256 + 48) * 28 * 130 * 4
     assert L.sb_swa_decode_workspace_bytes(64, 28, 128, 8) >= 64 * 8 * 28 * 130 * 4
