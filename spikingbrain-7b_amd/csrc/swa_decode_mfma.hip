@@ -146,10 +146,15 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
   };
   // Edge chunk (first / last chunk of the window; also correct for any other chunk): per-lane
   // pointers, tiles and rows clamped into the visible range, the newest row taken from the step
-  // inputs when the append is fused.
-  auto load_edge = [&](int cc, Chunk &ck) {
+  // inputs when the append is fused. base0/base1 = edge_bases(cc): the block-table lookups are made apart
+  // from the loads, all of a segment's in one go, so that they cost one round trip together.
+  auto edge_bases = [&](int cc, int64_t &base0, int64_t &base1) {
+    base0 = tile_base(clamp_tile(2 * cc));
+    base1 = tile_base(clamp_tile(2 * cc + 1));
+  };
+  auto load_edge = [&](int cc, int64_t base0, int64_t base1, Chunk &ck) {
     const int t0c = clamp_tile(2 * cc), t1c = clamp_tile(2 * cc + 1);
-    const char *k0p = p.k + tile_base(t0c), *k1p = p.k + tile_base(t1c);
+    const char *k0p = p.k + base0, *k1p = p.k + base1;
     const char *v0p = p.v + (k0p - p.k), *v1p = p.v + (k1p - p.k);
     const int newest = fused ? hi - 1 : -1;
     const int r0 = clamp_row(t0c, c), r1 = clamp_row(t1c, c);
@@ -267,7 +272,14 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
     const bool e_head = is_edge(cb);
     const bool e_tail = (ce - 1 > cb) && is_edge(ce - 1);
     const int ib = cb + (e_head ? 1 : 0), ie = ce - (e_tail ? 1 : 0);  // interior chunks [ib, ie)
+    // An edge chunk is fetched only where the segment has one (a window cut into n parts has two among
+    // its 2n ends), the head first because it is computed first, the tail two chunks before the stream
+    // ends: fetched up front it only delayed every workgroup's first chunks, all workgroups asking at once.
+    // The table lookups of both are made here, together with the first interior one.
     Chunk head, tail;
+    int64_t hb0, hb1, tb0, tb1;
+    edge_bases(cb, hb0, hb1);
+    edge_bases(ce - 1, tb0, tb1);
     if (ib < ie) {
       const int lastc = ie - 1;
       int64_t b0, b1;
@@ -284,17 +296,17 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
       Chunk ring[kDepth + 1];
       int ch = ib;
       locate(ch);
+      if (e_head) load_edge(cb, hb0, hb1, head);
 #pragma unroll
       for (int u = 0; u < kDepth; ++u) issue(ch + u, ring[u]);
-      // edge loads go behind the prologue: by the time they have landed so has the prologue
-      load_edge(cb, head);
-      load_edge(ce - 1, tail);
       if (e_head) compute_chunk(cb, head, kMasked, lo, hi);
+      const int tail_at = e_tail ? max(ib, ie - 2) : -1;
       bool more = true;
       while (more) {
 #pragma unroll
         for (int u = 0; u <= kDepth; ++u) {
           if (more) {
+            if (ch == tail_at) load_edge(ce - 1, tb0, tb1, tail);
             issue(ch + kDepth, ring[(u + kDepth) % (kDepth + 1)]);
             compute_chunk(ch, ring[u], kUnmasked, lo, hi);
             ++ch;
@@ -303,8 +315,8 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
         }
       }
     } else {
-      load_edge(cb, head);
-      load_edge(ce - 1, tail);
+      if (e_head) load_edge(cb, hb0, hb1, head);
+      if (e_tail) load_edge(ce - 1, tb0, tb1, tail);
       if (e_head) compute_chunk(cb, head, kMasked, lo, hi);
     }
     if (e_tail) compute_chunk(ce - 1, tail, kMasked, lo, hi);
