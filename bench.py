@@ -30,11 +30,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the matrix-core split kernel at the default workload, from rocprofv3 --pmc
-# FETCH_SIZE (253 377 KiB, scaled x2.000 by the same counter's reading of a 1 GiB stream copy) plus
+# FETCH_SIZE (251 433 KiB, scaled x2.000 by the same counter's reading of a 1 GiB stream copy) plus
 # WRITE_SIZE (3 768 KiB, scale x1.000): profiles/swa_decode_split_mfma_config2.md. Counters cannot be
 # read from inside this script, so the figure is the recorded one and is only attached when the run
 # is the default workload the profile covers.
-MEASURED_SPLIT_TRAFFIC_BYTES = (253377 * 2 + 3768) * 1024
+MEASURED_SPLIT_TRAFFIC_BYTES = (251433 * 2 + 3768) * 1024
 HQ, HKV, D, BS, WL = 28, 4, 128, 16, 4096
 E = 2  # bf16
 
