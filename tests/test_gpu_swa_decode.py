@@ -320,3 +320,23 @@ def test_split_policy_from_host_lengths(sb, dev):
         auto = run_paged(sb, dev, q, kv, tables, lens, -1, D ** -0.5, max_seq_len=max(lens), host_seq_lens=lens)
         forced = run_paged(sb, dev, q, kv, tables, lens, -1, D ** -0.5, max_seq_len=max(lens), balanced=expect)
         assert torch.equal(auto, forced)
+
+
+@pytest.mark.parametrize("n_split", [1, 3, 7])
+@pytest.mark.parametrize("wl", [-1, 100, 1000])
+def test_prefetch_depths_and_segment_ends_agree(sb, dev, wl, n_split):
+    """The streaming loop exists in three prefetch depths (flag bits 4-6); a segment's head chunk is fetched
+    first and its tail chunk two chunks before the stream ends, whatever the depth and however few interior
+    chunks the segment has (lengths here give segments of 0, 1, 2, 3 and many interior chunks). Every depth
+    must give the depth-1 result bit for bit (same arithmetic in the same order), and that one the oracle's."""
+    Hq, Hkv, D, bs = 28, 4, 128, 16
+    lens = [1, 31, 32, 33, 64, 65, 97, 129, 161, 200, 449, 1500, 2047]
+    kv, tables = paged_problem(lens, bs, Hkv, D, torch.bfloat16, 23)
+    g = torch.Generator().manual_seed(wl + n_split)
+    q = torch.randn(len(lens), Hq, D, generator=g).bfloat16()
+    outs = [run_paged(sb, dev, q, kv, tables, lens, wl, D ** -0.5, n_split=n_split, balanced=False,
+                      pipeline_depth=depth) for depth in (1, 2, 3)]
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    ref = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(), tables.numpy(),
+                                   lens, D ** -0.5, wl)
+    assert np.abs(outs[0].float().cpu().numpy() - ref).max() <= TOL[torch.bfloat16]
