@@ -66,7 +66,7 @@ __device__ __forceinline__ int row_chunks(const DecodeParams &p, const int32_t *
 // step's K/V row into the cache). Meta tokens: the call also takes chunks meta_first,
 // meta_first + meta_step, ... of the p.meta_len shared meta rows into the same softmax (meta_step 0:
 // none); the first of them is fetched before the window is walked and computed after it.
-template <typename E, int kDepth>
+template <typename E, int kDepth, bool kAsmLookups>
 __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32_t *block_table, const int G,
                                               const int kvh, const int lane, const int64_t r, const int lo,
                                               const int hi, const int cb, const int ce, const bool owns_newest,
@@ -108,6 +108,49 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
     }
     return (dense_row0 + i0) * p.kv_sr + head_off;
   };
+  // the same for six tiles at once, under ONE paged/dense branch: the six table lookups are then
+  // independent loads of one block and cost one round trip (one tile_base call after another, each with
+  // its own branch, waits for every lookup before making the next)
+  auto tile_bases6 = [&](const int (&t)[6], int64_t (&base)[6]) {
+    if (paged) {
+      int bi[6];
+      int64_t blk[6];
+#pragma unroll
+      for (int n = 0; n < 6; ++n) bi[n] = (t[n] << 4) / p.block_size;
+      // Written out as one block of scalar loads and one wait where kAsmLookups: left to itself the
+      // compiler, short of scalar registers here, issues each load only after the previous one has
+      // returned. Not in the balanced kernel: handing the table pointer to an asm statement counts as
+      // letting it escape, the no-alias guarantee against that kernel's partial stores is gone, and the
+      // lookups of its streaming loop turn into vector loads (measured 12 % slower).
+      if constexpr (!kAsmLookups) {
+#pragma unroll
+        for (int n = 0; n < 6; ++n) blk[n] = block_table[seq * p.bt_stride + bi[n]];
+      } else {
+      const int32_t *row = block_table + seq * p.bt_stride;
+      const int32_t *a0 = row + bi[0], *a1 = row + bi[1], *a2 = row + bi[2], *a3 = row + bi[3], *a4 = row + bi[4],
+                    *a5 = row + bi[5];
+      int32_t e0, e1, e2, e3, e4, e5;
+      asm(  // not volatile: a volatile asm counts as a possible store and would do the same
+          "s_load_dword %0, %6, 0x0\n\t"
+          "s_load_dword %1, %7, 0x0\n\t"
+          "s_load_dword %2, %8, 0x0\n\t"
+          "s_load_dword %3, %9, 0x0\n\t"
+          "s_load_dword %4, %10, 0x0\n\t"
+          "s_load_dword %5, %11, 0x0\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&s"(e0), "=&s"(e1), "=&s"(e2), "=&s"(e3), "=&s"(e4), "=&s"(e5)
+          : "s"(a0), "s"(a1), "s"(a2), "s"(a3), "s"(a4), "s"(a5));  // (reads only: no memory clobber, which
+                                                                      // would turn later lookups into vector loads)
+      blk[0] = e0; blk[1] = e1; blk[2] = e2; blk[3] = e3; blk[4] = e4; blk[5] = e5;
+      }
+#pragma unroll
+      for (int n = 0; n < 6; ++n)
+        base[n] = blk[n] * p.kv_sb + (int64_t)((t[n] << 4) - bi[n] * p.block_size) * p.kv_sr + head_off;
+    } else {
+#pragma unroll
+      for (int n = 0; n < 6; ++n) base[n] = (dense_row0 + (t[n] << 4)) * p.kv_sr + head_off;
+    }
+  };
   auto clamp_tile = [&](int t) { return min(max(t, first_tile), last_tile); };
   // row of tile tc whose key index is the visible key nearest to (tc*16 + row)
   auto clamp_row = [&](int tc, int row) { return min(max((tc << 4) + row, lo), hi - 1) - (tc << 4); };
@@ -146,12 +189,8 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
   };
   // Edge chunk (first / last chunk of the window; also correct for any other chunk): per-lane
   // pointers, tiles and rows clamped into the visible range, the newest row taken from the step
-  // inputs when the append is fused. base0/base1 = edge_bases(cc): the block-table lookups are made apart
-  // from the loads, all of a segment's in one go, so that they cost one round trip together.
-  auto edge_bases = [&](int cc, int64_t &base0, int64_t &base1) {
-    base0 = tile_base(clamp_tile(2 * cc));
-    base1 = tile_base(clamp_tile(2 * cc + 1));
-  };
+  // inputs when the append is fused. base0/base1 = the bases of tiles clamp_tile(2cc), clamp_tile(2cc+1):
+  // the block-table lookups are made apart from the loads, all of a segment's in one go (tile_bases6).
   auto load_edge = [&](int cc, int64_t base0, int64_t base1, Chunk &ck) {
     const int t0c = clamp_tile(2 * cc), t1c = clamp_tile(2 * cc + 1);
     const char *k0p = p.k + base0, *k1p = p.k + base1;
@@ -277,9 +316,12 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
     // ends: fetched up front it only delayed every workgroup's first chunks, all workgroups asking at once.
     // The table lookups of both are made here, together with the first interior one.
     Chunk head, tail;
-    int64_t hb0, hb1, tb0, tb1;
-    edge_bases(cb, hb0, hb1);
-    edge_bases(ce - 1, tb0, tb1);
+    const int tiles6[6] = {clamp_tile(2 * cb),       clamp_tile(2 * cb + 1),       // head chunk
+                           clamp_tile(2 * (ce - 1)), clamp_tile(2 * (ce - 1) + 1), // tail chunk
+                           clamp_tile(2 * ib),       clamp_tile(2 * ib + 1)};      // first interior chunk
+    int64_t base6[6];
+    tile_bases6(tiles6, base6);
+    const int64_t hb0 = base6[0], hb1 = base6[1], tb0 = base6[2], tb1 = base6[3];
     if (ib < ie) {
       const int lastc = ie - 1;
       int64_t b0, b1;
@@ -295,7 +337,8 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
       };
       Chunk ring[kDepth + 1];
       int ch = ib;
-      locate(ch);
+      b0 = base6[4];
+      b1 = base6[5];
       if (e_head) load_edge(cb, hb0, hb1, head);
 #pragma unroll
       for (int u = 0; u < kDepth; ++u) issue(ch + u, ring[u]);
@@ -395,7 +438,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
   const int cps = (n_chunks + p.n_split - 1) / p.n_split;
   const int cb = first_chunk + split * cps;
   const int ce = min(cb + cps, first_chunk + n_chunks);
-  split_segment<E, kDepth>(p, p.block_table, G, kvh, tid & 63, r, lo, hi, cb, ce, ce == first_chunk + n_chunks,
+  split_segment<E, kDepth, true>(p, p.block_table, G, kvh, tid & 63, r, lo, hi, cb, ce, ce == first_chunk + n_chunks,
                            p.n_split == 1, r * p.Hq * p.n_split + split, p.n_split,
                            split, p.meta_len > 0 ? p.n_split : 0);  // meta chunks dealt round robin to the splits
 }
@@ -456,7 +499,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_balanced_mfma_kerne
       int rlo, rhi, rfc;
       const int rn = row_chunks(p, seq_lens, r, rlo, rhi, rfc);  // uniform: scalar loads
       const int cb = rfc + max(c0 - r_start, 0), ce = rfc + min(c1 - r_start, rn);
-      split_segment<E, kDepth>(p, block_table, G, kvh, lane, r, rlo, rhi, cb, ce, ce == rfc + rn, false,
+      split_segment<E, kDepth, false>(p, block_table, G, kvh, lane, r, rlo, rhi, cb, ce, ce == rfc + rn, false,
                                (int64_t)(w + r) * p.Hq, 1, 0, 0);
     }
     before += __builtin_amdgcn_readlane(incl, 63);
