@@ -431,10 +431,11 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
   const int64_t r = blockIdx.x;
   const int split = blockIdx.z;
   const int tid = threadIdx.x;
-  const int kvh = blockIdx.y * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(tid >> 6);
-  if (kvh >= Hkv) return;  // whole wavefront; there is no barrier in this kernel
+  // (the row's length is asked for before anything else: it heads the chain length -> table -> K/V)
   int lo, hi, first_chunk;
   const int n_chunks = row_chunks(p, p.seq_lens, r, lo, hi, first_chunk);
+  const int kvh = blockIdx.y * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (kvh >= Hkv) return;  // whole wavefront; there is no barrier in this kernel
   const int cps = (n_chunks + p.n_split - 1) / p.n_split;
   const int cb = first_chunk + split * cps;
   const int ce = min(cb + cps, first_chunk + n_chunks);
