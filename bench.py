@@ -169,6 +169,57 @@ def bench_prefill(sb, dev, S=16, L=8192, iters=5):
     return res
 
 
+def bench_decode_sweep(sb, dev, batches=(16, 32, 48, 64, 80, 96, 100, 128, 160, 192, 200, 256, 300, 384), iters=30):
+    """Decode attention alone over batch sizes, every sequence window-saturated (8000 tokens, window_left
+    4096): the split the library picks by itself (`auto`) next to the fixed and the balanced split forced,
+    to show what the split policy buys at row counts that fit the 256 CUs badly."""
+    rows = []
+    lib = sb._native.lib()
+    for B in batches:
+        lens_t = torch.full((B,), 8000)
+        lo_blk = torch.clamp((lens_t - 1 - WL) // BS, min=0)
+        nblk = (lens_t - 1) // BS - lo_blk + 1
+        nb = int(nblk.sum()) + 8
+        g = torch.Generator().manual_seed(0)
+        perm = torch.randperm(nb, generator=g)
+        tables = torch.zeros(B, int(nblk.max()), dtype=torch.int32)
+        p = 0
+        for b in range(B):
+            tables[b, :nblk[b]] = perm[p:p + int(nblk[b])]
+            p += int(nblk[b])
+        seqlens = (lens_t - lo_blk * BS).to(torch.int32)
+        host_lens = seqlens.tolist()
+        seqlens, tables = seqlens.to(dev), tables.to(dev)
+        kvs = [torch.randn(2, nb, BS, HKV, D, device=dev, dtype=torch.bfloat16) for _ in range(2 if B > 64 else 4)]
+        q = torch.randn(B, HQ, D, device=dev, dtype=torch.bfloat16)
+        msl = max(host_lens)
+        n_split = lib.sb_swa_decode_auto_split(B, HKV, msl, WL)
+        row = {"rows": B, "n_split": n_split, "policy": "balanced" if sb.ops.prefer_balanced_split(host_lens, WL, n_split) else "fixed"}
+        for mode in ("auto", "fixed", "balanced"):
+            kw = {} if mode == "auto" else dict(balanced=(mode == "balanced"))
+
+            def call(i):
+                kv = kvs[i % len(kvs)]
+                sb.ops.swa_decode_attention(q, kv[0], kv[1], seqlens, block_table=tables, window_left=WL,
+                                            max_seq_len=msl, host_seq_lens=host_lens, **kw)
+            for i in range(4):
+                call(i)
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for i in range(iters):
+                call(i)
+            b.record()
+            torch.cuda.synchronize()
+            us = a.elapsed_time(b) / iters * 1e3
+            row[mode + "_us"] = round(us, 1)
+            row[mode + "_TBps"] = round(B * (WL + 1) * HKV * D * 2 * E / us / 1e6, 2)
+        rows.append(row)
+        del kvs
+        torch.cuda.empty_cache()
+    return rows
+
+
 def bench_gla_prompt(sb, dev, S=16, L=8192, H=28, iters=3):
     """The GLA layers' share of BASELINE config 4 (16 prompts x 8192 tokens): one packed launch
     over token-major [tokens, H, D] projections, states read from and left in the slot cache.
@@ -293,7 +344,7 @@ def main():
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
                                                     "28-layer hybrid decode step (config 5)")
     ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "hybrid_fp8", "hybrid_lean", "hybrid_shared",
-                                       "hybrid_leanest", "gla_prompt"), default=None,
+                                       "hybrid_leanest", "gla_prompt", "decode_sweep"), default=None,
                     help="run just that section and print its JSON (short runs for profiling one kernel)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -312,6 +363,9 @@ def main():
         return
     if args.only == "gla_prompt":
         print(json.dumps({"gla_prompt": bench_gla_prompt(sb, dev)}))
+        return
+    if args.only == "decode_sweep":
+        print(json.dumps({"decode_sweep": bench_decode_sweep(sb, dev)}))
         return
     if args.only == "hybrid":
         print(json.dumps({"hybrid_decode": bench_hybrid(sb, dev, steps=min(args.steps, 128))}))
