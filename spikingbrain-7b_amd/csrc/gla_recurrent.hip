@@ -80,9 +80,9 @@ __device__ __forceinline__ void store_state4(char *base, int idx4, float4 s) {
 
 // Five wavefronts per SIMD (96 registers: the 64 of the state, and a dozen words of the vectors' addresses
 // spilled once per call) measured 1 % faster on the 28-layer step than four without spills; six (80
-// registers) is 5 % slower.
+// registers) is 5 % slower. With a bf16 state (half the bytes per register held) four stays the faster.
 template <bool kStateF32>
-__global__ __launch_bounds__(256, 5) void gla_recurrent_kernel(const GlaParams p) {
+__global__ __launch_bounds__(256, kStateF32 ? 5 : 4) void gla_recurrent_kernel(const GlaParams p) {
   const int b = blockIdx.x / p.H;
   const int h = blockIdx.x - b * p.H;
   const int64_t slot = p.slot_idx ? (int64_t)p.slot_idx[b] : (int64_t)b;
