@@ -250,6 +250,8 @@ def swa_decode_attention(
             key = (R, int(max_seq_len), int(window_left), int(n_split))
             balanced = _SHAPE_POLICY.get(key)
             if balanced is None:
+                if len(_SHAPE_POLICY) >= 4096:   # lengths that grow step by step would fill it without end
+                    _SHAPE_POLICY.clear()
                 balanced = _SHAPE_POLICY[key] = prefer_balanced_split([int(max_seq_len)] * R, window_left, n_split)
     if balanced and can_balance and n_split < 2:
         n_split = 2  # the balanced split always goes through partial results and the merge
