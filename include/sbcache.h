@@ -202,6 +202,26 @@ size_t sb_swa_decode_workspace_bytes(int64_t num_rows, int32_t num_q_heads, int3
 int sb_swa_decode(const sb_swa_decode_args *args);
 
 /* ------------------------------------------------------------------------------------
+ * sb_swa_decode without any workspace from the caller and without any allocation.
+ * No counterpart in the reference. It is for callers that cannot allocate device memory around
+ * the call: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same arguments, kernels and results as sb_swa_decode (bit for bit), except that `workspace` /
+ * `workspace_bytes` are ignored: the split-K partial results live in a device array of
+ * SB_SWA_DECODE_STATIC_SCRATCH_BYTES that is part of the library image (every GPU the library runs
+ * on holds its own copy from module load until the process ends). A call whose partials need more
+ * (sb_swa_decode_workspace_bytes for its rows, heads and split count) is rejected with
+ * SB_ERR_WORKSPACE before anything is launched. The call makes no hipMalloc / hipFree and calls no
+ * allocating routine; the first call on a device looks the array's address up once
+ * (hipGetSymbolAddress; make that call outside stream capture, with the device of the tensors
+ * current on the calling thread).
+ * All calls on one GPU share that GPU's array: calls on different streams of one GPU that overlap
+ * in time race on the partials (calls on one stream are ordered and safe). Every partial a merge
+ * reads has been written by the same call's split kernel, so nothing needs clearing between calls.
+ * ------------------------------------------------------------------------------------ */
+#define SB_SWA_DECODE_STATIC_SCRATCH_BYTES (8u << 20)
+int sb_swa_decode_static(const sb_swa_decode_args *args);
+
+/* ------------------------------------------------------------------------------------
  * GLA recurrent step(s) with in-place, slot-indexed state.
  * Replaces my_fused_recurrent_gla (vllm_hymeta/model_for_7B/my_fused_recurrent.py:9-153,
  * called from vllm_hymeta/model_for_7B/gla_attention.py:232) for T = 1, and

@@ -20,6 +20,7 @@ SB_DECODE_FORCE_VALU = 1
 SB_DECODE_BALANCED = 2
 SB_KV_NONE, SB_KV_INT8, SB_KV_FP8 = 0, 1, 2
 SB_GLA_VECTOR_ONLY = 1
+SB_SWA_DECODE_STATIC_SCRATCH_BYTES = 8 << 20
 ABI_VERSION = 1
 
 _DTYPES = {torch.bfloat16: SB_BF16, torch.float16: SB_F16, torch.float32: SB_F32}
@@ -164,6 +165,7 @@ EXPORTS = {
     "sb_swa_decode_workspace_bytes": (sz, [i64, i32, i32, i32]),
     "sb_swa_decode_prefer_balanced": (i32, [C.POINTER(i32), i64, i32, i32]),
     "sb_swa_decode": (C.c_int, [C.POINTER(SwaDecodeArgs)]),
+    "sb_swa_decode_static": (C.c_int, [C.POINTER(SwaDecodeArgs)]),
     "sb_gla_recurrent": (C.c_int, [C.POINTER(GlaRecurrentArgs)]),
     "sb_copy_blocks": (C.c_int, [vp, vp, i64, i64, i64, vp]),
     "sb_window_shift": (C.c_int, [C.POINTER(WindowShiftArgs)]),

@@ -16,6 +16,7 @@
 //   Scores are kept in log2 units: p = exp2(s*scale*log2e - m).
 #include <algorithm>
 #include <functional>
+#include <mutex>
 #include <queue>
 #include <vector>
 
@@ -770,6 +771,62 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   else if (a->dtype == SB_F16) hipLaunchKernelGGL(swa_decode_merge_kernel<F16>, mgrid, dim3(128), 0, st, p);
   else hipLaunchKernelGGL(swa_decode_merge_kernel<F32>, mgrid, dim3(128), 0, st, p);
   return check_launch("swa_decode_merge_kernel");
+}
+
+// ---- sb_swa_decode_static: the same call, partial results in memory the library itself holds ------
+// The split-K partials go into a file-scope device array instead of a caller workspace, so the call
+// touches no allocator at all. Every GPU the library runs on holds its own copy of the array (at its
+// own address) until the process ends; the array's name is only a host-side handle for
+// hipGetSymbolAddress, the address that call returns is what kernels and copies are given.
+static __device__ __align__(256) unsigned char scratch[SB_SWA_DECODE_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices];  // per device: address of that device's copy of `scratch`, once looked up
+}  // namespace
+
+extern "C" int sb_swa_decode_static(const sb_swa_decode_args *a) {
+  using namespace sb_host;
+  if (!a) return fail(SB_ERR_INVALID, "sb_swa_decode_static: null args");
+  if (a->num_rows < 0) return fail(SB_ERR_INVALID, "sb_swa_decode_static: negative num_rows");
+  if (a->num_rows == 0) return SB_OK;
+  int n_split = a->n_split;
+  if (n_split < 0) return fail(SB_ERR_INVALID, "sb_swa_decode_static: negative n_split");
+  if (n_split == 0)
+    n_split = sb_swa_decode_auto_split(a->num_rows, a->num_kv_heads, a->max_seq_len, a->window_left);
+  const size_t need = sb_swa_decode_workspace_bytes(a->num_rows, a->num_q_heads, 128, n_split);
+  if (need > (size_t)SB_SWA_DECODE_STATIC_SCRATCH_BYTES)
+    return fail(SB_ERR_WORKSPACE,
+                "sb_swa_decode_static: %lld rows x %d heads in %d splits need %zu bytes of partial results, the "
+                "library's own scratch holds %zu (use sb_swa_decode with a workspace, or fewer splits)",
+                (long long)a->num_rows, a->num_q_heads, n_split, need, (size_t)SB_SWA_DECODE_STATIC_SCRATCH_BYTES);
+  sb_swa_decode_args b = *a;
+  b.n_split = n_split;
+  b.workspace = nullptr;
+  b.workspace_bytes = 0;
+  if (need > 0) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail((int)e, "sb_swa_decode_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices)
+      return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode_static: device index %d (at most %d devices)", dev, kMaxDevices);
+    void *ptr = nullptr;
+    {
+      std::lock_guard<std::mutex> lock(g_scratch_mu);
+      ptr = g_scratch_ptr[dev];
+      if (!ptr) {  // first call on this device (must not be under stream capture)
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+          return fail(e != hipSuccess ? (int)e : SB_ERR_INVALID, "sb_swa_decode_static: hipGetSymbolAddress: %s",
+                      hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+      }
+    }
+    b.workspace = ptr;
+    b.workspace_bytes = (size_t)SB_SWA_DECODE_STATIC_SCRATCH_BYTES;
+  }
+  return sb_swa_decode(&b);
 }
 
 extern "C" int sb_lse_merge(const sb_lse_merge_args *a) {
