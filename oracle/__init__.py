@@ -26,6 +26,10 @@ this path, so nothing here is pinned by a reference fixture):
                               clamps, code saturation, |x - code*scale| <= scale/2, symmetry and
                               power-of-two invariance; bf16 rounding against torch's conversion
                               (tests/test_oracle_quant.py)
+  cpu_path.*                  (the torch-CPU restatement timed as bench.py's cpu_baseline) an independent
+                              list-of-rows model for the window update, an explicit mask-and-softmax
+                              loop for the attention, the float64 unrolled closed form for the GLA
+                              step (tests/test_oracle_cpu_path.py)
   paged.*                     brute force over every position of small sequences: the set of
                               resident (block, offset) pairs equals the window; slots are
                               bt[pos//bs]*bs + pos%bs; dense<->paged equivalence

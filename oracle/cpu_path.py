@@ -1,7 +1,11 @@
 """The reference's PyTorch CPU path for one decode step, restated with plain torch CPU ops.
 
 TEST INFRASTRUCTURE (see oracle/__init__.py): this is what `bench.py` times as `cpu_baseline`
-(kind "port") and what config-1 parity tests step next to the GPU path. It follows
+(kind "port"); the parity tests use the numpy oracles (hf_cache, attention, gla) instead. Pinned by
+tests/test_oracle_cpu_path.py: the window update against an independent list-of-rows model (the
+300/511/700/900 traces at W=512, random schedules, the overshoot quirk), the attention against a
+mask-and-softmax loop written from the prose (left padding, fully masked queries), the GLA step
+against the float64 unrolled closed form and its special cases. It follows
   - hf_7B_model/cache.py:94-107        dense sliding-window update (roll + slice-assign / cat)
   - hf_7B_model/window_attention_sdpa.py:82-91,140-148,186-214   repeat_kv + SDPA with the
                                        sliding-causal additive mask + nan_to_num

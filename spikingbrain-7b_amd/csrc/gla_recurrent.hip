@@ -5,7 +5,10 @@
 // cover the state; each lane keeps its 16 row-quads (64 values) in registers for the whole
 // call. The state therefore crosses HBM exactly twice (one read, one write) whatever T is,
 // and all 16 row loads of a lane are independent, which is what hides HBM latency.
-// Gate, outer product and the q.S column reduction are fused into the same pass.
+// Gate, outer product and the q.S column reduction are fused into the same pass, and in the
+// call's last step each row-quad is stored as soon as it is updated.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -37,11 +40,27 @@ __device__ __forceinline__ void launch_heads(const GlaParams &p, int hh, int &hk
   h = hk * p.G + p.j0 + (hh - hk * p.jn);
 }
 
+// One element of a bf16 / f16 / f32 vector as float, without a branch on the type: the aligned 32-bit word
+// holding the element is loaded unconditionally and the three readings of it are selected between. (With
+// a branch per type the compiler cannot issue the loads of q, k, v and g together: each sits behind its
+// own branch and waits out a whole memory round trip before the next is issued.)
+__device__ __forceinline__ uint32_t load_scalar_raw(const void *p, int64_t i, int dtype, uint32_t &shift) {
+  const char *a = reinterpret_cast<const char *>(p) + i * (dtype == SB_F32 ? 4 : 2);
+  const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(a) & 2u);
+  shift = mis * 8u;
+  return *reinterpret_cast<const uint32_t *>(a - mis);
+}
+__device__ __forceinline__ float scalar_value(uint32_t w, uint32_t shift, int dtype) {
+  const uint32_t h = (w >> shift) & 0xffffu;
+  const float f32 = __uint_as_float(w);
+  const float bf = __uint_as_float(h << 16);
+  const float f16 = (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+  return dtype == SB_F32 ? f32 : (dtype == SB_BF16 ? bf : f16);
+}
 __device__ __forceinline__ float load_scalar(const void *p, int64_t i, int dtype) {
-  if (dtype == SB_F32) return reinterpret_cast<const float *>(p)[i];
-  if (dtype == SB_BF16)
-    return __uint_as_float((uint32_t) reinterpret_cast<const uint16_t *>(p)[i] << 16);
-  return (float)reinterpret_cast<const _Float16 *>(p)[i];
+  uint32_t shift;
+  const uint32_t w = load_scalar_raw(p, i, dtype, shift);
+  return scalar_value(w, shift, dtype);
 }
 __device__ __forceinline__ void store_scalar(void *p, int64_t i, int dtype, float x) {
   if (dtype == SB_F32)
@@ -78,11 +97,14 @@ __device__ __forceinline__ void store_state4(char *base, int idx4, float4 s) {
   }
 }
 
-// Five wavefronts per SIMD (96 registers: the 64 of the state, and a dozen words of the vectors' addresses
-// spilled once per call) measured 1 % faster on the 28-layer step than four without spills; six (80
-// registers) is 5 % slower. With a bf16 state (half the bytes per register held) four stays the faster.
-template <bool kStateF32>
-__global__ __launch_bounds__(256, kStateF32 ? 5 : 4) void gla_recurrent_kernel(const GlaParams p) {
+// The step that ends the call stores every row-quad of the state as soon as it is updated, so a workgroup's
+// stores start while its later loads are still arriving and overlap the reduction of the outputs: on the 7B
+// decode shape that alone took the update from 0.66 to 0.76 of the HBM peak (a plain streaming copy of the
+// same bytes reaches 0.77-0.80 on the same GPU). Loading everything, computing, then storing everything kept
+// the two directions of a workgroup apart. Occupancy: 84-96 registers, five wavefronts per SIMD; four, three or
+// two (pinned through the LDS size) measured the same or slower, six (80 registers, spilling) slower.
+template <bool kStateF32, bool kOneStep>
+__global__ __launch_bounds__(256, kOneStep ? 4 : 3) void gla_recurrent_kernel(const GlaParams p) {
   const int b = blockIdx.x / p.H;
   const int h = blockIdx.x - b * p.H;
   const int64_t slot = p.slot_idx ? (int64_t)p.slot_idx[b] : (int64_t)b;
@@ -99,18 +121,42 @@ __global__ __launch_bounds__(256, kStateF32 ? 5 : 4) void gla_recurrent_kernel(c
   char *sbase = reinterpret_cast<char *>(p.state) +
                 (slot * p.s_slot + (int64_t)h * p.s_head) * (kStateF32 ? 4 : 2);
 
+  // q, k, v, g of a step are asked for before anything else (the first step's ahead of the state, whose 16
+  // loads per lane would otherwise queue in front of them; a later step's while the step before it is
+  // computed). Every thread takes part, without a branch: the lower half of the workgroup fetches q and k,
+  // the upper half v and g. (Loads under `if (tid < 128)` get sunk into that branch next to their only
+  // use, behind the state loads, and everything then waits for the whole state before the first store.)
+  const bool lower = tid < 128;
+  const int e = tid & 127;
+  const void *src0 = lower ? p.q : p.v, *src1 = lower ? p.k : p.g;
+  const int dt0 = p.dtype, dt1 = lower ? p.dtype : p.g_dtype;
+  const int64_t off0 = (lower ? b * p.q_sb + h * p.q_sh : b * p.v_sb + h * p.v_sh) + e;
+  const int64_t off1 = (lower ? b * p.k_sb + h * p.k_sh : b * p.g_sb + h * p.g_sh) + e;
+  const int64_t st0 = lower ? p.q_st : p.v_st, st1 = lower ? p.k_st : p.g_st;
+  float *const dst0 = (lower ? s_q : s_v) + e, *const dst1 = (lower ? s_k : s_eg) + e;
+  uint32_t w0, w1, sh0, sh1;
+  auto fetch = [&](const int t) {
+    w0 = load_scalar_raw(src0, off0 + t * st0, dt0, sh0);
+    w1 = load_scalar_raw(src1, off1 + t * st1, dt1, sh1);
+  };
+  fetch(0);
+
   float4 S[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) S[i] = load_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4);
+  for (int i = 0; i < 16; ++i) {
+    S[i] = load_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4);
+    __builtin_amdgcn_sched_barrier(0);  // issued in this order: the last step consumes them in this order
+  }
 
-  for (int t = 0; t < p.T; ++t) {
-    if (tid < 128) {
-      s_q[tid] = load_scalar(p.q, b * p.q_sb + h * p.q_sh + t * p.q_st + tid, p.dtype) * p.scale;
-      s_k[tid] = load_scalar(p.k, b * p.k_sb + h * p.k_sh + t * p.k_st + tid, p.dtype);
-      s_v[tid] = load_scalar(p.v, b * p.v_sb + h * p.v_sh + t * p.v_st + tid, p.dtype);
-      s_eg[tid] = expf(load_scalar(p.g, b * p.g_sb + h * p.g_sh + t * p.g_st + tid, p.g_dtype));
+  auto step = [&](const int t, auto last_tag) {
+    constexpr bool kLast = decltype(last_tag)::value;
+    {
+      const float x0 = scalar_value(w0, sh0, dt0), x1 = scalar_value(w1, sh1, dt1);
+      *dst0 = lower ? x0 * p.scale : x0;   // q * scale | v
+      *dst1 = lower ? x1 : expf(x1);       // k | exp(g)
     }
     __syncthreads();
+    if constexpr (!kLast) fetch(t + 1);
     const float4 vv = reinterpret_cast<const float4 *>(s_v)[col4];
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
@@ -125,6 +171,12 @@ __global__ __launch_bounds__(256, kStateF32 ? 5 : 4) void gla_recurrent_kernel(c
       o.y = fmaf(qq, S[i].y, o.y);
       o.z = fmaf(qq, S[i].z, o.z);
       o.w = fmaf(qq, S[i].w, o.w);
+      if constexpr (kLast) {
+        store_state4<kStateF32>(sbase, row * 32 + col4, S[i]);
+        // keep the quads in the order their loads were issued (loads return in order: the first quad can
+        // be finished and stored while the last ones are still on their way)
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     reinterpret_cast<float4 *>(s_o[rg])[col4] = o;
     __syncthreads();
@@ -134,10 +186,16 @@ __global__ __launch_bounds__(256, kStateF32 ? 5 : 4) void gla_recurrent_kernel(c
       for (int r = 0; r < 8; ++r) acc += s_o[r][tid];
       store_scalar(p.out, b * p.o_sb + h * p.o_sh + t * p.o_st + tid, p.dtype, acc);
     }
+  };
+  // kOneStep: a decode step (one token) is an instantiation of its own. Its only step is reached straight
+  // from the loads above, so its waits count exactly how many of them are still outstanding; behind a loop
+  // over earlier steps the same code has to wait for everything in flight where the two paths meet.
+  if constexpr (kOneStep) {
+    step(0, std::true_type{});
+  } else {
+    for (int t = 0; t + 1 < p.T; ++t) step(t, std::false_type{});
+    step(p.T - 1, std::true_type{});
   }
-
-#pragma unroll
-  for (int i = 0; i < 16; ++i) store_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4, S[i]);
 }
 
 // ---- shared states: one state per kv head, G query heads read it -----------------------------------
@@ -146,8 +204,8 @@ __global__ __launch_bounds__(256, kStateF32 ? 5 : 4) void gla_recurrent_kernel(c
 // crosses HBM once per group instead of once per query head.
 constexpr int kMaxGroup = 8;
 
-template <bool kStateF32>
-__global__ __launch_bounds__(256) void gla_recurrent_grouped_kernel(const GlaParams p) {
+template <bool kStateF32, bool kOneStep>
+__global__ __launch_bounds__(256, kOneStep ? 4 : 3) void gla_recurrent_grouped_kernel(const GlaParams p) {
   const int Hk = p.H / p.G;
   const int b = blockIdx.x / Hk;
   const int hk = blockIdx.x - b * Hk;
@@ -159,28 +217,59 @@ __global__ __launch_bounds__(256) void gla_recurrent_grouped_kernel(const GlaPar
   const int rg = tid >> 5;
   const int G = p.G;
 
-  __shared__ float s_q[kMaxGroup][128], s_k[128], s_eg[128];
-  __shared__ __attribute__((aligned(16))) float s_v[128];
+  // the step's vectors in LDS: rows 0 .. G-1 = the group's q heads (scaled), then k, v, exp(g)
+  __shared__ __attribute__((aligned(16))) float s_vec[kMaxGroup + 3][128];
   __shared__ __attribute__((aligned(16))) float s_o[kMaxGroup][8][128];
+  float (*const s_q)[128] = s_vec;
+  float *const s_k = s_vec[kMaxGroup], *const s_v = s_vec[kMaxGroup + 1], *const s_eg = s_vec[kMaxGroup + 2];
 
   char *sbase = reinterpret_cast<char *>(p.state) +
                 (slot * p.s_slot + (int64_t)hk * p.s_head) * (kStateF32 ? 4 : 2);
 
+  // Vectors first and one step ahead, as in the kernel above, every thread taking part without a branch:
+  // the (G + 3) * 128 elements of q (G heads), k, v, g are dealt out 256 at a time; a thread whose turn
+  // falls past the end fetches an element of g again and stores the same value a second time.
+  constexpr int kIter = ((kMaxGroup + 3) * 128 + 255) / 256;
+  const void *src[kIter];
+  float *dst[kIter];
+  int64_t off[kIter], stp[kIter];
+  int kind[kIter];  // 0 = q (times scale), 1 = k or v (as is), 2 = gate (exp)
+#pragma unroll
+  for (int it = 0; it < kIter; ++it) {
+    const int idx = tid + 256 * it, e = idx & 127;
+    const int vi = min(idx >> 7, G + 2);
+    const bool is_q = vi < G, is_k = vi == G, is_v = vi == G + 1;
+    src[it] = is_q ? p.q : (is_k ? p.k : (is_v ? p.v : p.g));
+    off[it] = (is_q ? b * p.q_sb + (hk * G + vi) * p.q_sh
+                    : (is_k ? b * p.k_sb + hk * p.k_sh : (is_v ? b * p.v_sb + hk * p.v_sh : b * p.g_sb + hk * p.g_sh))) + e;
+    stp[it] = is_q ? p.q_st : (is_k ? p.k_st : (is_v ? p.v_st : p.g_st));
+    dst[it] = (is_q ? s_vec[vi] : s_vec[kMaxGroup + vi - G]) + e;
+    kind[it] = is_q ? 0 : ((is_k || is_v) ? 1 : 2);
+  }
+  uint32_t w[kIter], sh[kIter];
+  auto fetch = [&](const int t) {
+#pragma unroll
+    for (int it = 0; it < kIter; ++it)
+      w[it] = load_scalar_raw(src[it], off[it] + t * stp[it], kind[it] == 2 ? p.g_dtype : p.dtype, sh[it]);
+  };
+  fetch(0);
+
   float4 S[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) S[i] = load_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4);
+  for (int i = 0; i < 16; ++i) {
+    S[i] = load_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4);
+    __builtin_amdgcn_sched_barrier(0);  // issued in this order: the last step consumes them in this order
+  }
 
-  for (int t = 0; t < p.T; ++t) {
-    for (int idx = tid; idx < G * 128; idx += 256) {
-      const int j = idx >> 7, e = idx & 127;
-      s_q[j][e] = load_scalar(p.q, b * p.q_sb + (hk * G + j) * p.q_sh + t * p.q_st + e, p.dtype) * p.scale;
-    }
-    if (tid < 128) {
-      s_k[tid] = load_scalar(p.k, b * p.k_sb + hk * p.k_sh + t * p.k_st + tid, p.dtype);
-      s_v[tid] = load_scalar(p.v, b * p.v_sb + hk * p.v_sh + t * p.v_st + tid, p.dtype);
-      s_eg[tid] = expf(load_scalar(p.g, b * p.g_sb + hk * p.g_sh + t * p.g_st + tid, p.g_dtype));
+  auto step = [&](const int t, auto last_tag) {
+    constexpr bool kLast = decltype(last_tag)::value;
+#pragma unroll
+    for (int it = 0; it < kIter; ++it) {
+      const float x = scalar_value(w[it], sh[it], kind[it] == 2 ? p.g_dtype : p.dtype);
+      *dst[it] = kind[it] == 0 ? x * p.scale : (kind[it] == 1 ? x : expf(x));
     }
     __syncthreads();
+    if constexpr (!kLast) fetch(t + 1);
     const float4 vv = reinterpret_cast<const float4 *>(s_v)[col4];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -190,6 +279,10 @@ __global__ __launch_bounds__(256) void gla_recurrent_grouped_kernel(const GlaPar
       S[i].y = fmaf(kk, vv.y, eg * S[i].y);
       S[i].z = fmaf(kk, vv.z, eg * S[i].z);
       S[i].w = fmaf(kk, vv.w, eg * S[i].w);
+      if constexpr (kLast) {  // as in the kernel above
+        store_state4<kStateF32>(sbase, row * 32 + col4, S[i]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     for (int j = 0; j < G; ++j) {
       float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -211,10 +304,16 @@ __global__ __launch_bounds__(256) void gla_recurrent_grouped_kernel(const GlaPar
       for (int r = 0; r < 8; ++r) acc += s_o[j][r][e];
       store_scalar(p.out, b * p.o_sb + (hk * G + j) * p.o_sh + t * p.o_st + e, p.dtype, acc);
     }
+  };
+  // kOneStep: a decode step (one token) is an instantiation of its own. Its only step is reached straight
+  // from the loads above, so its waits count exactly how many of them are still outstanding; behind a loop
+  // over earlier steps the same code has to wait for everything in flight where the two paths meet.
+  if constexpr (kOneStep) {
+    step(0, std::true_type{});
+  } else {
+    for (int t = 0; t + 1 < p.T; ++t) step(t, std::false_type{});
+    step(p.T - 1, std::true_type{});
   }
-
-#pragma unroll
-  for (int i = 0; i < 16; ++i) store_state4<kStateF32>(sbase, (i * 8 + rg) * 32 + col4, S[i]);
 }
 
 // ---- many steps per call (prompts) ---------------------------------------------------------
@@ -498,18 +597,20 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
     }
     return check_launch("gla_sequence_kernel");
   }
+  const hipStream_t st = (hipStream_t)a->stream;
+  const bool f32s = a->state_dtype == SB_F32, one = a->seq_len == 1;
   if (G > 1) {  // decode with shared states: one workgroup per (row, state head)
     const dim3 ggrid((unsigned)(a->batch * Hk));
-    if (a->state_dtype == SB_F32)
-      hipLaunchKernelGGL(gla_recurrent_grouped_kernel<true>, ggrid, dim3(256), 0, (hipStream_t)a->stream, p);
-    else
-      hipLaunchKernelGGL(gla_recurrent_grouped_kernel<false>, ggrid, dim3(256), 0, (hipStream_t)a->stream, p);
+    if (f32s && one) hipLaunchKernelGGL((gla_recurrent_grouped_kernel<true, true>), ggrid, dim3(256), 0, st, p);
+    else if (f32s) hipLaunchKernelGGL((gla_recurrent_grouped_kernel<true, false>), ggrid, dim3(256), 0, st, p);
+    else if (one) hipLaunchKernelGGL((gla_recurrent_grouped_kernel<false, true>), ggrid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gla_recurrent_grouped_kernel<false, false>), ggrid, dim3(256), 0, st, p);
     return check_launch("gla_recurrent_grouped_kernel");
   }
   const dim3 grid((unsigned)groups), block(256);
-  if (a->state_dtype == SB_F32)
-    hipLaunchKernelGGL(gla_recurrent_kernel<true>, grid, block, 0, (hipStream_t)a->stream, p);
-  else
-    hipLaunchKernelGGL(gla_recurrent_kernel<false>, grid, block, 0, (hipStream_t)a->stream, p);
+  if (f32s && one) hipLaunchKernelGGL((gla_recurrent_kernel<true, true>), grid, block, 0, st, p);
+  else if (f32s) hipLaunchKernelGGL((gla_recurrent_kernel<true, false>), grid, block, 0, st, p);
+  else if (one) hipLaunchKernelGGL((gla_recurrent_kernel<false, true>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((gla_recurrent_kernel<false, false>), grid, block, 0, st, p);
   return check_launch("gla_recurrent_kernel");
 }
