@@ -67,6 +67,33 @@ def sdpa_window_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, sliding_w
     return masked_softmax_attention(q, kr, vr, masked)
 
 
+def flash_window_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, sliding_window: int,
+                           attention_mask: Optional[np.ndarray] = None) -> np.ndarray:
+    """The inference branch of hf_7B_model/window_attention.py:186-217, step by step: the padding mask
+    is cut to the key length (attention_mask[:, -K:], :190), pad positions are dropped from K/V and
+    from the last Q query positions (_upad_input, :188-193), every sequence runs causal varlen
+    attention with window_size = (sliding_window, 0), i.e. the query sees itself and sliding_window
+    keys to its left, bottom-right aligned (:204-215), and pad_input puts the rows back with zeros
+    at pad positions (:216). q [B, Hq, Q, D]; k, v [B, Hkv, K, D]; returns [B, Hq, Q, D] float64.
+    Q is either K (prompt) or 1 (decode), the two cases _upad_input supports with a kv mask."""
+    B, Hq, Q, D = q.shape
+    K = k.shape[2]
+    keep = np.ones((B, K), bool) if attention_mask is None else (np.asarray(attention_mask)[:, -K:] != 0)
+    out = np.zeros((B, Hq, Q, D))
+    for b in range(B):
+        kidx = np.nonzero(keep[b])[0]
+        qkeep = keep[b, K - Q:]                    # the queries are the last Q positions
+        qidx = np.nonzero(qkeep)[0]
+        if len(qidx) == 0:
+            continue
+        qs = np.asarray(q[b], np.float64)[:, qidx].transpose(1, 0, 2)          # [Lq, Hq, D]
+        ks = np.asarray(k[b], np.float64)[:, kidx].transpose(1, 0, 2)          # [Lk, Hkv, D]
+        vs = np.asarray(v[b], np.float64)[:, kidx].transpose(1, 0, 2)
+        o = varlen_window_attention(qs, ks, vs, [0, len(qidx)], [0, len(kidx)], D ** -0.5, sliding_window)
+        out[b][:, qidx] = o.transpose(1, 0, 2)
+    return out
+
+
 def gather_paged(cache: np.ndarray, block_table_row: Sequence[int], n: int) -> np.ndarray:
     """Rows 0..n-1 of a sequence from a paged cache half [num_blocks, bs, Hkv, D] -> [n, Hkv, D]
     (key i lives in block block_table[i // bs] at offset i % bs; kv_cache layout of

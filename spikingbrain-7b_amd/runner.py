@@ -94,7 +94,9 @@ class SwaCacheRunner:
 
     def build_step(self, prompts: Sequence[Tuple[int, int]], decodes: Sequence[int],
                    chunked_prefill: bool = False) -> MetaAttentionMetadata:
-        """`prompts` = (seq_id, number of new prompt tokens), `decodes` = seq ids taking one token.
+        """`prompts` = (seq_id, number of new prompt tokens); `decodes` = seq ids taking one token each, or
+        (seq_id, n) pairs for decoding sequences that take n query tokens in this step (speculative /
+        multi-token decode, the `max_decode_query_len > 1` branch of meta_attention.py:924-953).
         Advances the block manager (eviction, allocation) and returns the step's metadata with
         tokens laid out [prompt tokens | decode tokens]."""
         mgr, bs = self.manager, self.block_size
@@ -118,19 +120,23 @@ class SwaCacheRunner:
                 block_tables={sid: ResidentTable(mgr, r)}))
             seq_lens.append(view_len)
             query_lens.append(n_new)
-        if decodes:
-            mgr.decode_step(list(decodes))
-        for sid in decodes:
+        decodes = [d if isinstance(d, tuple) else (d, 1) for d in decodes]
+        if decodes and all(n == 1 for _, n in decodes):
+            mgr.decode_step([sid for sid, _ in decodes])
+        else:
+            for sid, n in decodes:      # same policy, one sequence after the other in batch-row order
+                mgr.append_tokens(sid, n, False)
+        for sid, n in decodes:
             r = mgr.row_of(sid)
             total = int(mgr.n_tokens[r])
             view_len = total - int(mgr.lo[r]) * bs
             ib.inter_data_list.append(SeqGroupData(
-                is_prompt=False, seq_ids=[sid], input_tokens=[[0]], orig_seq_lens=[total], seq_lens=[view_len],
-                query_lens=[1], context_lens=[total - 1],
+                is_prompt=False, seq_ids=[sid], input_tokens=[[0] * n], orig_seq_lens=[total], seq_lens=[view_len],
+                query_lens=[n], context_lens=[total - n],
                 curr_sliding_window_blocks=[int(mgr.hi[r] - mgr.lo[r]) + 1],
                 block_tables={sid: ResidentTable(mgr, r)}))
             seq_lens.append(view_len)
-            query_lens.append(1)
+            query_lens.append(n)
         builder = MetaAttentionMetadataBuilder(ib)
         builder.prepare()
         return builder.build(seq_lens, query_lens, -1, len(seq_lens))

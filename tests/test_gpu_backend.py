@@ -37,8 +37,9 @@ class OracleEngine:
         t = 0
         for sid, n in prompts:
             slots += self.model.append_tokens(sid, n, True, store_all=chunked); spans.append((sid, t, t + n)); t += n
-        for sid in decodes:
-            slots += self.model.append_tokens(sid, 1, False); spans.append((sid, t, t + 1)); t += 1
+        for d in decodes:
+            sid, n = d if isinstance(d, tuple) else (d, 1)       # (sid, n): n query tokens for a decoding sequence
+            slots += self.model.append_tokens(sid, n, False); spans.append((sid, t, t + n)); t += n
         outs = []
         for l in range(self.layers):
             P.kv_append(k[l], v[l], self.kc[l], self.vc[l], slots)
@@ -51,32 +52,35 @@ class OracleEngine:
         return slots, outs
 
 
-def run_step(sb, dev, runner, impls, orc, prompts, decodes, g, chunked=False):
-    T = sum(n for _, n in prompts) + len(decodes)
+def run_step(sb, dev, runner, impls, orc, prompts, decodes, g, chunked=False, dtype=torch.bfloat16):
+    dec_tokens = sum(d[1] if isinstance(d, tuple) else 1 for d in decodes)
+    T = sum(n for _, n in prompts) + dec_tokens
     layers = len(impls)
-    q = [torch.randn(T, HQ, D, generator=g).bfloat16() for _ in range(layers)]
-    k = [torch.randn(T, HKV, D, generator=g).bfloat16() for _ in range(layers)]
-    v = [torch.randn(T, HKV, D, generator=g).bfloat16() for _ in range(layers)]
+    q = [torch.randn(T, HQ, D, generator=g).to(dtype) for _ in range(layers)]
+    k = [torch.randn(T, HKV, D, generator=g).to(dtype) for _ in range(layers)]
+    v = [torch.randn(T, HKV, D, generator=g).to(dtype) for _ in range(layers)]
     meta = runner.build_step(prompts, decodes, chunked_prefill=chunked)
     slots, refs = orc.step(prompts, decodes, [x.float().numpy() for x in q], [x.float().numpy() for x in k],
                            [x.float().numpy() for x in v], chunked)
     assert meta.slot_mapping.cpu().tolist() == slots                                   # bit-exact indexing
-    assert meta.num_prefill_tokens == sum(n for _, n in prompts) and meta.num_decode_tokens == len(decodes)
+    assert meta.num_prefill_tokens == sum(n for _, n in prompts) and meta.num_decode_tokens == dec_tokens
     if decodes:
         dm = meta.decode_metadata
-        for i, sid in enumerate(decodes):
+        for i, d in enumerate(decodes):
+            sid = d[0] if isinstance(d, tuple) else d
             table, seqlen, _ = orc.model.view(sid)
             assert dm.block_tables[i, :len(table)].cpu().tolist() == table
             assert (dm.block_tables[i, len(table):] == 0).all()
             assert int(dm.seq_lens_tensor[i]) == seqlen
     for l, impl in enumerate(impls):
-        out = torch.full((T, HQ, D), float("nan"), dtype=torch.bfloat16, device=dev)
+        out = torch.full((T, HQ, D), float("nan"), dtype=dtype, device=dev)
         ret = impl.forward(None, q[l].to(dev), k[l].to(dev), v[l].to(dev), None, None, None, runner.kv_caches[l], meta, output=out)
         assert ret.data_ptr() == out.data_ptr()                                         # written in place
         err = np.abs(out.float().cpu().numpy() - refs[l]).max()
-        assert err <= TOL, f"layer {l}: max-abs {err}"
+        assert err <= (TOL if dtype == torch.bfloat16 else 1e-5), f"layer {l}: max-abs {err}"
         assert np.array_equal(runner.kv_caches[l][0].float().cpu().numpy(), orc.kc[l])
         assert np.array_equal(runner.kv_caches[l][1].float().cpu().numpy(), orc.vc[l])
+    return meta
 
 
 @pytest.mark.parametrize("bs,wl", [(16, 64), (32, 80)])
@@ -101,6 +105,35 @@ def test_engine_prefill_decode_eviction(sb, dev, bs, wl):
     runner.free_seq(1); orc.model.free_seq(1)
     for _ in range(bs + 1):
         run_step(sb, dev, runner, impls, orc, [], [3, 0, 2], g)
+    assert runner.manager.free_stack() == orc.model.free
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_engine_multi_query_decode(sb, dev, dtype):
+    """Decoding sequences that take several query tokens in one step (max_decode_query_len > 1, the branch at
+    vllm_hymeta/attention/meta_attention.py:924-953: varlen attention of the decode tokens over the paged
+    cache): mixed run lengths in one batch, alone and behind a chunked prompt, across block boundaries and
+    window eviction, interleaved with ordinary one-token steps. Slots, tables, lengths and cache bytes
+    bit-exact; outputs against the oracle's varlen attention over each sequence's full history. bf16 takes
+    the many-query kernel, fp32 one single-query row per token."""
+    bs, wl, layers, nb = 16, 48, 2, 64
+    g = torch.Generator().manual_seed(11)
+    runner = sb.runner.SwaCacheRunner(layers, nb, bs, wl, HKV, D, dtype, dev, max_seqs=4, max_chunk_tokens=128)
+    impls = [sb.MetaAttentionImpl(HQ, D, D ** -0.5, HKV, None, wl + 1, "auto") for _ in range(layers)]
+    orc = OracleEngine(layers, nb, bs, wl)
+    for sid in (0, 1, 2):
+        runner.add_seq(sid); orc.add(sid)
+    step = lambda prompts, decodes, chunked=False: run_step(sb, dev, runner, impls, orc, prompts, decodes, g,
+                                                            chunked=chunked, dtype=dtype)
+    step([(0, 10), (1, wl + 9), (2, 31)], [])
+    meta = step([], [(0, 3), (1, 5), (2, 1)])                       # runs of 3, 5 and 1 query tokens
+    assert meta.max_decode_query_len == 5 and meta.decode_metadata.query_start_loc.tolist() == [0, 3, 8, 9]
+    step([], [0, 1, 2])                                             # an ordinary decode step in between
+    for _ in range(6):                                              # 6 x 4 tokens: block boundaries, eviction, recycling
+        step([], [(1, 4), (0, 4), (2, 2)])
+    runner.add_seq(3); orc.add(3)
+    step([(3, 40)], [(2, 3), (0, 2)], chunked=True)                 # behind a chunked prompt in the same batch
+    step([], [(3, 17), (1, 2)])                                     # a run longer than a block
     assert runner.manager.free_stack() == orc.model.free
 
 

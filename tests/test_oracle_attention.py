@@ -167,3 +167,24 @@ def test_metatoken_attention_is_window_attention_merged_with_meta_attention():
     for i in range(Lq):
         n = min(W, Lk - Lq + i + 1)
         np.testing.assert_allclose(o[i], (2.0 * M + 5.0 * n) / (M + n), rtol=1e-12)
+
+
+def test_flash_window_attention_is_W_plus_one_keys_and_unpads():
+    """flash window_size=(W, 0) = the query and W keys to its left. Constant scores make the output the
+    mean of the visible V rows, which names them; pads (a prefix) are invisible and pad queries give 0.
+    Against the SDPA-flavour oracle it is the same mask one key wider."""
+    B, H, K, D, W = 2, 1, 8, 4, 2
+    q = np.zeros((B, H, K, D)); k = np.zeros((B, H, K, D))
+    v = np.broadcast_to(np.arange(K, dtype=np.float64)[None, None, :, None], (B, H, K, D)).copy()
+    am = np.ones((B, K + 1), np.int64); am[1, :4] = 0          # row 1: positions 0..2 of the keys are pads
+    out = A.flash_window_attention(q, k, v, W, am)
+    # row 0, query i sees keys max(0, i-2)..i
+    np.testing.assert_allclose(out[0, 0, :, 0], [0, 0.5, 1, 2, 3, 4, 5, 6])
+    # row 1: keys 3..7 are real; queries 0..2 are pads -> zeros; query 3 sees {3}, 4 {3,4}, 5 {3,4,5}, 6 {4,5,6}
+    np.testing.assert_allclose(out[1, 0, :, 0], [0, 0, 0, 3, 3.5, 4, 5, 6])
+    # decode shape: one query at the end of K keys sees the last W+1 real keys
+    np.testing.assert_allclose(A.flash_window_attention(q[:, :, -1:], k, v, W, am)[:, 0, 0, 0], [6, 6])
+    r = rng(5)
+    q = r.standard_normal((B, 4, K, D)); k = r.standard_normal((B, 2, K, D)); v = r.standard_normal((B, 2, K, D))
+    np.testing.assert_allclose(A.flash_window_attention(q, k, v, W, am), A.sdpa_window_attention(q, k, v, W + 1, am),
+                               rtol=1e-12, atol=1e-12)
