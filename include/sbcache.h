@@ -502,6 +502,10 @@ int sb_lse_merge(const sb_lse_merge_args *args);
  *   token included), block_tables [B, table_width] int32 (oldest resident block first,
  *   0 beyond the last), status [1] int32 (sticky; bit 0 = out of blocks, bit 1 = a
  *   sequence outgrew its ring; the caller reads it when it next synchronises).
+ * A sequence that needs a block when the free stack is empty does not take its token: its slot is -1
+ * (the step's append skips it), its seq_len counts the cached keys only, its token count stays, and no
+ * block of another sequence is touched; its attention output of that step is meaningless. Callers that
+ * run steps back to back (a replayed graph) must poll `status`.
  * ------------------------------------------------------------------------------------ */
 typedef struct sb_window_advance_args {
   int64_t *n_tokens;
@@ -528,6 +532,14 @@ int sb_window_advance(const sb_window_advance_args *args);
  * (FETCH_SIZE / WRITE_SIZE) are calibrated against.
  * ------------------------------------------------------------------------------------ */
 int sb_stream_copy(void *dst, const void *src, int64_t bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------
+ * Identity of the stream capture `stream` is part of: *id = the runtime's capture sequence number,
+ * or 0 when the stream is not capturing. No counterpart in the reference (there the graph runner of
+ * vLLM owns every buffer a captured step touches); the host layer uses it to give each captured graph
+ * a split-K workspace of its own that no later call can replace or free. Returns 0 or the hipError_t.
+ * ------------------------------------------------------------------------------------ */
+int sb_stream_capture_id(void *stream, uint64_t *id);
 
 #ifdef __cplusplus
 }

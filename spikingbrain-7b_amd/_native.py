@@ -177,6 +177,7 @@ EXPORTS = {
     "sb_kv_append_fp8": (C.c_int, [C.POINTER(KvAppendFp8Args)]),
     "sb_fp8_round": (C.c_int, [vp, vp, i64, i64, i64, i64, i32, f32, vp]),
     "sb_stream_copy": (C.c_int, [vp, vp, i64, vp]),
+    "sb_stream_capture_id": (C.c_int, [vp, C.POINTER(C.c_uint64)]),
 }
 
 _lib: Optional[C.CDLL] = None

@@ -36,3 +36,14 @@ int check_launch(const char *what) {
 
 extern "C" int sb_abi_version(void) { return SB_ABI_VERSION; }
 extern "C" const char *sb_last_error(void) { return g_err; }
+
+extern "C" int sb_stream_capture_id(void *stream, uint64_t *id) {
+  if (!id) return sb_host::fail(SB_ERR_INVALID, "sb_stream_capture_id: null id");
+  *id = 0;
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long seq = 0;
+  const hipError_t e = hipStreamGetCaptureInfo((hipStream_t)stream, &status, &seq);
+  if (e != hipSuccess) return sb_host::fail((int)e, "sb_stream_capture_id: %s", hipGetErrorString(e));
+  if (status == hipStreamCaptureStatusActive) *id = seq ? (uint64_t)seq : ~(uint64_t)0;
+  return SB_OK;
+}

@@ -121,10 +121,13 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
         }
         const int jb = s_alloc[i];
         if (jb >= 0) {
-          int id = 0;
           if (top == 0) {
+            // No free block: the row does not take its token (see below); its ring entry is left as it is,
+            // so no block another sequence owns is handed out or written to.
             s_status |= 1;
+            s_newid[i] = -1;
           } else {
+            int id;
             --top;
             if (n > 0) {
               id = s_cache[--n];
@@ -132,9 +135,9 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
               id = p.free_stack[top];
               base = top;
             }
+            p.ring[(int64_t)(r0 + i) * R + jb % R] = id;
+            s_newid[i] = id;
           }
-          p.ring[(int64_t)(r0 + i) * R + jb % R] = id;
-          s_newid[i] = id;
         }
       }
       s_top = top;
@@ -148,11 +151,23 @@ __global__ __launch_bounds__(1024) void window_advance_kernel(const AdvanceParam
       const int jb = (int)(p0 / bs);
       // (the freshly allocated id comes from LDS: the global ring entry was written by another lane)
       const int id = s_alloc[tid] >= 0 ? s_newid[tid] : p.ring[(int64_t)r * R + jb % R];
-      p.slot_mapping[r] = (int64_t)id * bs + (p0 - (int64_t)jb * bs);
-      p.seq_lens[r] = (int)(p0 + 1 - (int64_t)lo * bs);
-      p.n_tokens[r] = p0 + 1;
-      p.lo[r] = lo;
-      p.hi[r] = hi;
+      if (id < 0) {
+        // Out of blocks (status bit 0 is set): the row's token is not taken. Its slot is the pad slot, so
+        // the step's append skips it; its length counts the cached keys only; its token count does not move
+        // (the next advance tries again); what left the window stays evicted. The row's attention output
+        // of this step is meaningless and the caller finds out from the status word.
+        hi = jb - 1;
+        p.slot_mapping[r] = -1;
+        p.seq_lens[r] = (int)max((int64_t)0, p0 - (int64_t)lo * bs);
+        p.lo[r] = lo;
+        p.hi[r] = hi;
+      } else {
+        p.slot_mapping[r] = (int64_t)id * bs + (p0 - (int64_t)jb * bs);
+        p.seq_lens[r] = (int)(p0 + 1 - (int64_t)lo * bs);
+        p.n_tokens[r] = p0 + 1;
+        p.lo[r] = lo;
+        p.hi[r] = hi;
+      }
     }
     __syncthreads();
   }

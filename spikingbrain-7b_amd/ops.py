@@ -12,18 +12,38 @@ from . import _native as N
 
 PAD_SLOT_ID = -1
 
-_workspaces: Dict[torch.device, torch.Tensor] = {}
+# Split-K scratch of the decode kernel. Outside stream capture: one buffer per (device, stream), grown on
+# demand (calls on one stream are ordered, so they can share it; calls on different streams must not).
+# Under stream capture: one buffer per capture, kept for the life of the process. A captured graph replays
+# into the addresses recorded at capture time, so such a buffer must never be replaced, shrunk or handed
+# back to the allocator by a later, larger request (the allocator could give the block to another tensor
+# while every replay still writes and merges partials there).
+_workspaces: Dict[Tuple[torch.device, int], torch.Tensor] = {}
+_graph_workspaces: Dict[Tuple[torch.device, int], list] = {}
+
+
+def _capture_id(dev: torch.device) -> int:
+    """Sequence number of the stream capture torch's current stream is part of, 0 if none."""
+    cid = C.c_uint64(0)
+    N.check(N.lib().sb_stream_capture_id(N.stream_ptr(dev), C.byref(cid)), "stream_capture_id")
+    return cid.value
 
 
 def _workspace(dev: torch.device, nbytes: int) -> Optional[torch.Tensor]:
-    """Per-device scratch for split-K partials, grown on demand and reused by every call on
-    the device (calls on one device are stream-ordered, so they never overlap)."""
     if nbytes == 0:
         return None
-    ws = _workspaces.get(dev)
+    cap = _capture_id(dev)
+    if cap:
+        owned = _graph_workspaces.setdefault((dev, cap), [])
+        if not owned or owned[-1].numel() < nbytes:
+            # (a smaller buffer handed out earlier in this capture stays in the list: earlier nodes use it)
+            owned.append(torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev))
+        return owned[-1]
+    key = (dev, N.stream_ptr(dev))
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
-        _workspaces[dev] = ws
+        _workspaces[key] = ws
     return ws
 
 

@@ -84,3 +84,34 @@ def test_device_advance_reports_exhaustion(sb, dev):
     state.advance()                                          # token 16 needs a second block
     with pytest.raises(RuntimeError, match="out of KV cache blocks"):
         state.check()
+
+
+def test_exhaustion_touches_no_foreign_block(sb, dev):
+    """Free stack empty while one sequence must grow into a new block: that row gets the pad slot (its append
+    is skipped), keeps its token count and length, and the other sequences' blocks, slots and cache rows are
+    what they would be anyway. The host manager raises at the same point; the device reports through status."""
+    bs, wl, Hkv, D = 16, 64, 4, 128
+    mgr = sb.WindowBlockManager(3, bs, wl, max_seqs=2)       # three blocks in total
+    mgr.add_seq(0); mgr.add_seq(1)
+    mgr.append_tokens(0, 16, True)                           # block 0 full: the next token needs a new block
+    mgr.append_tokens(1, 20, True)                           # two blocks, room in the second
+    assert mgr.num_free_blocks == 0
+    before = dict(tok=mgr.n_tokens[:2].copy(), ring=mgr.ring[:2].copy())
+    state = sb.block_manager.DeviceWindowState(mgr, [0, 1], dev)
+    kv = torch.zeros(2, 3, bs, Hkv, D, dtype=torch.bfloat16, device=dev)
+    for step in range(2):                                    # the failing row fails again on the next step
+        state.advance()
+        torch.cuda.synchronize()
+        assert state.slot_mapping.tolist()[0] == sb.PAD_SLOT_ID
+        assert state.n_tokens.tolist() == [16, 21 + step] and state.seq_lens.tolist() == [16, 21 + step]
+        assert np.array_equal(state.ring.cpu().numpy(), before["ring"])           # no id handed out, none overwritten
+        pos = 20 + step
+        assert state.slot_mapping.tolist()[1] == int(before["ring"][1][pos // bs]) * bs + pos % bs
+        assert state.block_tables[0].tolist()[:1] == [int(before["ring"][0][0])]
+        k = torch.full((2, Hkv, D), float(step + 1), dtype=torch.bfloat16, device=dev)
+        sb.ops.kv_append(k, k, kv[0], kv[1], state.slot_mapping)
+        torch.cuda.synchronize()
+        written = (kv[0] != 0).flatten(2).any(2).nonzero().tolist()               # (block, row) pairs holding data
+        assert written == [[int(before["ring"][1][1]), 4 + s] for s in range(step + 1)]
+    with pytest.raises(RuntimeError, match="out of KV cache blocks"):
+        state.check()
