@@ -102,6 +102,12 @@ int sb_kv_append(const sb_kv_append_args *args);
  * The kernel splits each row's window into n_split parts and merges them; partials live
  * in `workspace` (sb_swa_decode_workspace_bytes). n_split = 0 picks a split count from
  * the shapes alone (never from device data), so the call is graph-capturable.
+ * The first 64 KiB of the workspace are reserved for SB_DECODE_MERGE_IN_KERNEL (arrival counters):
+ * with that flag they must be ZERO when a workspace is used for the first time (hipMemset it once
+ * after allocating it); every call leaves them zero again, whatever its shape, so a workspace can be
+ * reused by any later call on the stream. (Their last word is a sticky fault flag: non-zero means
+ * partial results were merged across XCDs, which the launch geometry rules out; tests assert it
+ * stays zero.) Without the flag the region is not touched.
  * head_size must be 128. bf16/fp16 run on the matrix cores with any GQA group size
  * num_q_heads/num_kv_heads <= 16; fp32 (and SB_DECODE_FORCE_VALU) runs on the vector ALUs with
  * group sizes {1,2,4,7,8}.
@@ -118,6 +124,13 @@ int sb_kv_append(const sb_kv_append_args *args);
  * summation order; same workspace size. Pass n_split = 2 when the fixed split would not split at all
  * (the balanced split always goes through partial results and the merge). */
 #define SB_DECODE_BALANCED 2
+/* bf16/fp16 fixed split, phases 0, no meta tokens: merge the partial results inside the split kernel instead
+ * of in a kernel of its own. The splits of a row run on one XCD (the launch sees to that), so the last of
+ * its wavefronts to finish can pick the others' partials up from the shared L2 without any cache write-back;
+ * same arithmetic and order as the merge kernel, same bits. Measured NOT faster on MI355X at 16..128 rows
+ * (the hand-over chain at the end of the kernel costs what the second launch costs), hence opt-in. Needs the
+ * workspace's first 64 KiB zeroed before its first use (see below). */
+#define SB_DECODE_MERGE_IN_KERNEL 4
 
 typedef struct sb_swa_decode_args {
   const void *q;   /* [num_rows, num_q_heads, head_size] */

@@ -588,7 +588,7 @@ extern "C" size_t sb_swa_decode_workspace_bytes(int64_t num_rows, int32_t num_q_
                                                 int32_t head_size, int32_t n_split) {
   if (n_split <= 1 || num_rows <= 0 || num_q_heads <= 0 || head_size <= 0) return 0;
   const int64_t parts = partial_slots(num_rows, n_split) * num_q_heads;
-  return (size_t)(round_up(parts * head_size * 4, 256) + round_up(parts * 2 * 4, 256));
+  return (size_t)(kMergeCounterBytes + round_up(parts * head_size * 4, 256) + round_up(parts * 2 * 4, 256));
 }
 
 extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
@@ -663,8 +663,11 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   p.block_table = a->block_table; p.kv_start = a->kv_start; p.row_seq = a->row_seq;
   p.seq_lens = a->seq_lens; p.key_lo = a->key_lo;
   const int64_t parts = partial_slots(a->num_rows, n_split) * a->num_q_heads;
-  p.ws_acc = (float *)a->workspace;
-  p.ws_ml = need ? (float *)((char *)a->workspace + round_up(parts * 128 * 4, 256)) : nullptr;
+  // workspace = [arrival counters of the in-kernel merge | partial numerators | partial (max, denominator)]
+  p.merge_counter = nullptr;
+  p.Hkv = a->num_kv_heads;
+  p.ws_acc = need ? (float *)((char *)a->workspace + kMergeCounterBytes) : nullptr;
+  p.ws_ml = need ? (float *)((char *)a->workspace + kMergeCounterBytes + round_up(parts * 128 * 4, 256)) : nullptr;
   p.Hq = a->num_q_heads; p.block_size = a->block_size > 0 ? a->block_size : 16;
   p.window_left = a->window_left; p.n_split = n_split;
   p.rows = (int)a->num_rows; p.n_wg = 0;
@@ -750,6 +753,12 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   }
   if (mfma && !int8_kv && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
     p.n_wg = (int)balanced_workgroups(a->num_rows, n_split);
+  // On request the fixed split of the matrix-core kernel merges in the same launch (the last wavefront of a
+  // row to finish does it), where the arrival counters fit; otherwise the merge kernel follows as usual.
+  if ((a->flags & SB_DECODE_MERGE_IN_KERNEL) && mfma && !int8_kv && n_split > 1 && n_split <= 64 && p.n_wg == 0 &&
+      a->phases == 0 && ((a->flags >> 4) & 7) <= 1 && a->meta_len == 0 &&
+      (a->num_rows + 7) / 8 * 8 * (int64_t)a->num_kv_heads <= kMergeCounters)
+    p.merge_counter = (int *)a->workspace;
   if (a->phases != 2) {
     if (int8_kv) launch_swa_decode_split_i8(a->dtype, a->kv_quant, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p);
     else if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
@@ -759,7 +768,7 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
     else rc = launch_for_group<F32>(G, grid, st, p);
     rc = check_launch("swa_decode_split_kernel");
   }
-  if (rc != SB_OK || n_split == 1 || a->phases == 1) return rc;
+  if (rc != SB_OK || n_split == 1 || a->phases == 1 || p.merge_counter) return rc;
 
   const dim3 mgrid((unsigned)(a->num_rows * a->num_q_heads));
   if (p.n_wg > 0) {

@@ -66,7 +66,7 @@ __device__ __forceinline__ int row_chunks(const DecodeParams &p, const int32_t *
 // step's K/V row into the cache). Meta tokens: the call also takes chunks meta_first,
 // meta_first + meta_step, ... of the p.meta_len shared meta rows into the same softmax (meta_step 0:
 // none); the first of them is fetched before the window is walked and computed after it.
-template <typename E, int kDepth, bool kAsmLookups>
+template <typename E, int kDepth, int kLookups, bool kMergeHere = false>
 __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32_t *block_table, const int G,
                                               const int kvh, const int lane, const int64_t r, const int lo,
                                               const int hi, const int cb, const int ce, const bool owns_newest,
@@ -117,14 +117,24 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
       int64_t blk[6];
 #pragma unroll
       for (int n = 0; n < 6; ++n) bi[n] = (t[n] << 4) / p.block_size;
-      // Written out as one block of scalar loads and one wait where kAsmLookups: left to itself the
+      // kLookups = 1: written out as one block of scalar loads and one wait; left to itself (kLookups = 0) the
       // compiler, short of scalar registers here, issues each load only after the previous one has
-      // returned. Not in the balanced kernel: handing the table pointer to an asm statement counts as
-      // letting it escape, the no-alias guarantee against that kernel's partial stores is gone, and the
-      // lookups of its streaming loop turn into vector loads (measured 12 % slower).
-      if constexpr (!kAsmLookups) {
+      // returned: six round trips before the first K/V load. Not in the balanced kernel: handing the table
+      // pointer to an asm statement counts as letting it escape, the no-alias guarantee against that
+      // kernel's partial stores is gone, and the lookups of its streaming loop turn into vector loads
+      // (measured 12 % slower). There (kLookups = 2) lanes 0..5 fetch one entry each with ONE vector load
+      // (nothing else is in flight at the start of a segment, so it waits for nothing but itself) and
+      // the six values are read back across lanes.
+      if constexpr (kLookups == 0) {
 #pragma unroll
         for (int n = 0; n < 6; ++n) blk[n] = block_table[seq * p.bt_stride + bi[n]];
+      } else if constexpr (kLookups == 2) {
+        int mine = bi[0];
+#pragma unroll
+        for (int n = 1; n < 6; ++n) mine = lane == n ? bi[n] : mine;
+        const int32_t e = block_table[seq * p.bt_stride + mine];
+#pragma unroll
+        for (int n = 0; n < 6; ++n) blk[n] = __builtin_amdgcn_readlane(e, n);
       } else {
       const int32_t *row = block_table + seq * p.bt_stride;
       const int32_t *a0 = row + bi[0], *a1 = row + bi[1], *a2 = row + bi[2], *a3 = row + bi[3], *a4 = row + bi[4],
@@ -420,15 +430,106 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
       }
     }
   }
+
+  // ---- merge by the last wavefront of the row to arrive ------------------------------------------------
+  // The n_split wavefronts that work on (row r, kv head kvh) run in workgroups whose numbers differ by
+  // multiples of 8 (the launch pads the row count to a multiple of 8), and workgroup i of a launch runs on
+  // XCD i % 8: they all sit behind ONE L2. Inside an XCD the L2 is the point of coherence, so handing the
+  // partials from one wavefront to another takes no cache write-back: a wavefront waits until its own
+  // partial stores have been acknowledged by the L2, then bumps the pair's counter (an atomic executed in
+  // that L2); whoever sees n_split - 1 knows that every partial of the pair is in the L2, reads them with
+  // loads that skip its CU's L1 (sc1), merges exactly as swa_decode_merge_kernel does (same order, same
+  // arithmetic: the same bits) and zeroes the counter for the next launch. Nobody waits for anybody.
+  // (Across XCDs the same hand-over needs the dirty L2 lines written back to memory and the reader's L2
+  // invalidated: with agent-scope fences that made the whole step 1.5x slower.)
+  // Measured on the 7B decode shape (64 rows x 4 splits): the chain partial stores acknowledged -> counter ->
+  // partial loads -> output stores at the end of the last wavefront costs 5.7 us of kernel time, against
+  // 4.8 us for the merge kernel plus its launch gap: no gain (88 -> 94 us per step), and none at 16, 32 or 128
+  // rows either. The variant is therefore opt-in (SB_DECODE_MERGE_IN_KERNEL); it is an instantiation of its
+  // own so that its 160 extra live registers do not weigh on the default kernel.
+  if constexpr (kMergeHere) if (!direct && p.merge_counter != nullptr) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt vmcnt(0): this wavefront's partial is in the L2
+    int *counter = p.merge_counter + r * p.Hkv + kvh;
+    const int xcc = (int)__builtin_amdgcn_s_getreg(20 | (3 << 11));  // HW_REG_XCC_ID, bits 3:0
+    int arrived = 0;
+    if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1 + (xcc << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrived = __builtin_amdgcn_readfirstlane(arrived);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // (orders the compiler; the loads below skip the L1 themselves)
+    if ((arrived & 0xff) != p.n_split - 1) return;
+    if (lane == 0) {
+      *counter = 0;
+      // every contributor must have run on this XCD; if not, the sticky fault word (last counter) says so
+      if ((arrived >> 8) + xcc != p.n_split * xcc) p.merge_counter[kMergeFaultWord] = 1;
+    }
+    if (c >= G) return;
+    const int hq = kvh * G + c;
+    const int64_t part0 = (r * p.Hq + hq) * (int64_t)p.n_split;
+    const __amdgpu_buffer_rsrc_t acc_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.ws_acc, 0, 0x7fffffff, 0x00020000);
+    float tot[32];
+#pragma unroll
+    for (int d = 0; d < 32; ++d) tot[d] = 0.f;
+    float L = 0.f, M = kNegInf;
+    for (int s0 = 0; s0 < p.n_split; s0 += 4) {
+      float ms[4], ls[4];
+      u32x4_t av[4][8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t part = part0 + min(s0 + j, p.n_split - 1);
+        ms[j] = __hip_atomic_load(p.ws_ml + part * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ls[j] = __hip_atomic_load(p.ws_ml + part * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int q4 = 0; q4 < 8; ++q4)
+          av[j][q4] = __builtin_amdgcn_raw_buffer_load_b128(acc_rsrc, (int)((part * 128 + 32 * g + 4 * q4) * 4), 0, 1 << 4);
+      }
+      float Mn = M;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (s0 + j < p.n_split) Mn = fmaxf(Mn, ms[j]);
+      if (Mn != kNegInf) {
+        const float keep = (M == kNegInf) ? 0.f : fast_exp2(M - Mn);
+#pragma unroll
+        for (int d = 0; d < 32; ++d) tot[d] *= keep;
+        L *= keep;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float f = (s0 + j >= p.n_split || ms[j] == kNegInf) ? 0.f : fast_exp2(ms[j] - Mn);
+#pragma unroll
+          for (int q4 = 0; q4 < 8; ++q4) {
+            tot[4 * q4 + 0] = fmaf(__uint_as_float(av[j][q4].x), f, tot[4 * q4 + 0]);
+            tot[4 * q4 + 1] = fmaf(__uint_as_float(av[j][q4].y), f, tot[4 * q4 + 1]);
+            tot[4 * q4 + 2] = fmaf(__uint_as_float(av[j][q4].z), f, tot[4 * q4 + 2]);
+            tot[4 * q4 + 3] = fmaf(__uint_as_float(av[j][q4].w), f, tot[4 * q4 + 3]);
+          }
+          L = fmaf(ls[j], f, L);
+        }
+      }
+      M = Mn;
+    }
+    char *dst = p.out + (r * p.o_sr + (int64_t)hq * p.o_sh + 32 * g) * 2;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float o8[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o8[e] = L > 0.f ? tot[8 * i + e] / L : 0.f;
+      uint4 o;
+      o.x = E::pack(o8[0], o8[1]);
+      o.y = E::pack(o8[2], o8[3]);
+      o.z = E::pack(o8[4], o8[5]);
+      o.w = E::pack(o8[6], o8[7]);
+      *reinterpret_cast<uint4 *>(dst + 16 * i) = o;
+    }
+    if (g == 0 && p.lse) p.lse[r * p.Hq + hq] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
+  }
 }
 
 // Fixed split: grid = (query rows, kv-head groups, splits); every row's chunks are cut into
 // n_split equal runs. kMaxThreads bounds the workgroup size, which with one workgroup per CU fixes
 // the register budget (256 threads: one wavefront per SIMD, 512 registers).
-template <typename E, int kDepth, int kMaxThreads>
+template <typename E, int kDepth, int kMaxThreads, bool kMergeHere = false>
 __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(const DecodeParams p, const int G,
                                                                                 const int Hkv) {
   const int64_t r = blockIdx.x;
+  if (r >= p.rows) return;  // (the row count is padded to a multiple of 8 when the merge is done in here)
   const int split = blockIdx.z;
   const int tid = threadIdx.x;
   // (the row's length is asked for before anything else: it heads the chain length -> table -> K/V)
@@ -439,7 +540,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_split_mfma_kernel(c
   const int cps = (n_chunks + p.n_split - 1) / p.n_split;
   const int cb = first_chunk + split * cps;
   const int ce = min(cb + cps, first_chunk + n_chunks);
-  split_segment<E, kDepth, true>(p, p.block_table, G, kvh, tid & 63, r, lo, hi, cb, ce, ce == first_chunk + n_chunks,
+  split_segment<E, kDepth, 1, kMergeHere>(p, p.block_table, G, kvh, tid & 63, r, lo, hi, cb, ce, ce == first_chunk + n_chunks,
                            p.n_split == 1, r * p.Hq * p.n_split + split, p.n_split,
                            split, p.meta_len > 0 ? p.n_split : 0);  // meta chunks dealt round robin to the splits
 }
@@ -476,32 +577,43 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_balanced_mfma_kerne
   if (kvh >= Hkv) return;
   const int lane = tid & 63;
   const int w = blockIdx.x, n_wg = gridDim.x;
+  // Every wavefront works the runs out for itself from one look at seq_lens: lane i holds row base + i (its
+  // visible range and chunks); a wave-wide scan places the rows on the common chunk axis; the rows of this
+  // workgroup's run are then read back from those lanes (no second trip to memory per row).
   int total = 0;
-  for (int base = 0; base < p.rows; base += 64) {
-    int lo, hi, fc;
-    total += wave_sum(base + lane < p.rows ? row_chunks(p, seq_lens, base + lane, lo, hi, fc) : 0);
+  if (p.rows > 64) {  // more rows than lanes: the total needs a pass of its own
+    for (int base = 0; base < p.rows; base += 64) {
+      int lo, hi, fc;
+      total += wave_sum(base + lane < p.rows ? row_chunks(p, seq_lens, base + lane, lo, hi, fc) : 0);
+    }
+    total = __builtin_amdgcn_readfirstlane(total);
   }
-  total = __builtin_amdgcn_readfirstlane(total);
-  const int per = (total + n_wg - 1) / n_wg;
-  const int c0 = w * per, c1 = min(c0 + per, total);
-  if (c0 >= c1) return;
   int before = 0;  // chunks of the rows below `base`
-  for (int base = 0; base < p.rows && before < c1; base += 64) {
-    int lo, hi, fc;
+  int per = 0, c0 = 0, c1 = 0;
+  for (int base = 0; base < p.rows; base += 64) {
+    int lo = 0, hi = 0, fc = 0;
     const int n = base + lane < p.rows ? row_chunks(p, seq_lens, base + lane, lo, hi, fc) : 0;
     const int incl = wave_inclusive_scan(n, lane);
+    if (base == 0) {
+      if (p.rows <= 64) total = __builtin_amdgcn_readlane(incl, 63);
+      per = (total + n_wg - 1) / n_wg;
+      c0 = w * per;
+      c1 = min(c0 + per, total);
+      if (c0 >= c1) return;
+    }
+    if (before >= c1) break;
     const int start = before + incl - n;  // this lane's row begins at this chunk of the whole
     uint64_t todo = __builtin_amdgcn_ballot_w64(n > 0 && start < c1 && start + n > c0);
     while (todo) {
       const int i = __builtin_ctzll(todo);
       todo &= todo - 1;
       const int r_start = __builtin_amdgcn_readlane(start, i);
+      const int rlo = __builtin_amdgcn_readlane(lo, i), rhi = __builtin_amdgcn_readlane(hi, i);
+      const int rfc = __builtin_amdgcn_readlane(fc, i), rn = __builtin_amdgcn_readlane(n, i);
       const int64_t r = base + i;
-      int rlo, rhi, rfc;
-      const int rn = row_chunks(p, seq_lens, r, rlo, rhi, rfc);  // uniform: scalar loads
       const int cb = rfc + max(c0 - r_start, 0), ce = rfc + min(c1 - r_start, rn);
-      split_segment<E, kDepth, false>(p, block_table, G, kvh, lane, r, rlo, rhi, cb, ce, ce == rfc + rn, false,
-                               (int64_t)(w + r) * p.Hq, 1, 0, 0);
+      split_segment<E, kDepth, 2>(p, block_table, G, kvh, lane, r, rlo, rhi, cb, ce, ce == rfc + rn, false,
+                                  (int64_t)(w + r) * p.Hq, 1, 0, 0);
     }
     before += __builtin_amdgcn_readlane(incl, 63);
   }
@@ -532,7 +644,16 @@ void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsi
                          p.seq_lens, G, Hkv);
     return;
   }
-  const dim3 grid(rows, ygroups, n_split);
+  // merge inside this kernel: all splits of a row on one XCD (workgroup i runs on XCD i % 8, and the number of
+  // a workgroup is x + gridDim.x * (y + gridDim.y * z)), which a row count padded to a multiple of 8 gives
+  const dim3 grid(p.merge_counter ? (rows + 7u) / 8u * 8u : rows, ygroups, n_split);
+  if (p.merge_counter) {  // the variant that merges the partial results itself (depth 1 only)
+    if (dtype == SB_BF16)
+      hipLaunchKernelGGL((swa_decode_split_mfma_kernel<sb::BF16, 1, 256, true>), grid, block, 0, st, p, G, Hkv);
+    else
+      hipLaunchKernelGGL((swa_decode_split_mfma_kernel<sb::F16, 1, 256, true>), grid, block, 0, st, p, G, Hkv);
+    return;
+  }
 #define SB_LAUNCH(E, D) hipLaunchKernelGGL((swa_decode_split_mfma_kernel<E, D, 256>), grid, block, 0, st, p, G, Hkv)
   if (dtype == SB_BF16) {
     if (depth == 1) SB_LAUNCH(sb::BF16, 1);

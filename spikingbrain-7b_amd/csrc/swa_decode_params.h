@@ -4,6 +4,12 @@
 
 namespace sb {
 
+// Arrival counters of the in-kernel merge live in the first kMergeCounterBytes of the split-K workspace; the
+// last of them is a sticky fault word (set if contributors to one merge ran on different XCDs).
+constexpr int kMergeCounterBytes = 64 << 10;
+constexpr int kMergeCounters = kMergeCounterBytes / 4 - 1;
+constexpr int kMergeFaultWord = kMergeCounterBytes / 4 - 1;
+
 struct DecodeParams {
   const char *q;
   const char *k;
@@ -19,6 +25,10 @@ struct DecodeParams {
   float *ws_ml;   // [rows, Hq, n_split, 2]
   int Hq, block_size, window_left, n_split;
   int rows, n_wg;  // balanced split: query rows, workgroups per kv-head group (0 = fixed split)
+  // Merge inside the split kernel (matrix-core fixed split): arrival counters [rows, Hkv], zero before and after
+  // every launch, and the number of kv heads; null = the merge is a kernel of its own.
+  int *merge_counter;
+  int Hkv;
   float scale_log2;
   int64_t q_sr, q_sh, o_sr, o_sh;  // elements
   int64_t kv_sb, kv_sr, kv_sh;     // bytes

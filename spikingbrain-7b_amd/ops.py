@@ -37,12 +37,12 @@ def _workspace(dev: torch.device, nbytes: int) -> Optional[torch.Tensor]:
         owned = _graph_workspaces.setdefault((dev, cap), [])
         if not owned or owned[-1].numel() < nbytes:
             # (a smaller buffer handed out earlier in this capture stays in the list: earlier nodes use it)
-            owned.append(torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev))
+            owned.append(torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev))
         return owned[-1]
     key = (dev, N.stream_ptr(dev))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)   # (its merge counters start at zero)
         _workspaces[key] = ws
     return ws
 
@@ -112,6 +112,7 @@ def swa_decode_attention(
     n_split: int = 0,
     phases: int = 0,
     force_valu: bool = False,
+    merge_in_kernel: bool = False,
     balanced: Optional[bool] = None,
     host_seq_lens=None,
     k_scale: Optional[torch.Tensor] = None,
@@ -145,6 +146,8 @@ def swa_decode_attention(
     derived from the table/window shapes so that no device value is read back.
     phases: 0 = whole op; 1 = split kernel only, 2 = merge kernel only (profiling aid).
     force_valu: run bf16/fp16 on the vector-ALU split kernel instead of the matrix-core one.
+    merge_in_kernel: the matrix-core fixed split merges its partial results itself (the last wavefront of a
+    row to finish does it) instead of leaving them to the merge kernel; same bits, measured no faster.
     balanced: cut the chunks of all rows, laid end to end, into equal runs (one per CU) instead of
     cutting each row into n_split runs (bf16/fp16, <= 1024 rows): faster when the rows' lengths differ
     a lot, a little slower when they do not. Default: decided from host_seq_lens (the same numbers
@@ -285,7 +288,8 @@ def swa_decode_attention(
         num_rows=R, num_q_heads=Hq, num_kv_heads=Hkv, head_size=D, block_size=bs,
         window_left=int(window_left), max_seq_len=int(min(max_seq_len, 2**31 - 1)), n_split=int(n_split),
         dtype=N.dtype_code(q.dtype), phases=int(phases),
-        flags=(N.SB_DECODE_FORCE_VALU if force_valu else 0) | (N.SB_DECODE_BALANCED if balanced else 0) | ((int(pipeline_depth) & 7) << 4),
+        flags=(N.SB_DECODE_FORCE_VALU if force_valu else 0) | (N.SB_DECODE_BALANCED if balanced else 0)
+        | (N.SB_DECODE_MERGE_IN_KERNEL if merge_in_kernel else 0) | ((int(pipeline_depth) & 7) << 4),
         scale=float(scale),
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),

@@ -102,6 +102,7 @@ static int check_attention() {
   const size_t ws_bytes = sb_swa_decode_workspace_bytes(B, Hq, D, n_split);
   void *d_ws = nullptr;
   HIP_OK(hipMalloc(&d_ws, ws_bytes));
+  HIP_OK(hipMemset(d_ws, 0, ws_bytes));  // a workspace starts zeroed (its merge counters); calls leave it reusable
   sb_swa_decode_args a = {};
   a.q = d_q; a.k_cache = d_k; a.v_cache = d_v; a.out = d_out; a.block_table = d_table; a.seq_lens = d_lens;
   a.workspace = d_ws; a.workspace_bytes = ws_bytes;

@@ -340,3 +340,51 @@ def test_prefetch_depths_and_segment_ends_agree(sb, dev, wl, n_split):
     ref = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(), tables.numpy(),
                                    lens, D ** -0.5, wl)
     assert np.abs(outs[0].float().cpu().numpy() - ref).max() <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,n_split,wl", [(1, 2, -1), (7, 3, 300), (8, 4, 300), (21, 5, 97), (64, 4, 4096), (130, 2, -1)])
+def test_merge_inside_the_split_kernel_equals_merge_kernel(sb, dev, dtype, rows, n_split, wl):
+    """With merge_in_kernel the matrix-core fixed split merges its partial results itself (the last wavefront of a
+    row to finish does it); without, the same partials go through the merge kernel. Same arithmetic in the same
+    order: outputs and log-sum-exps must agree bit for bit, for row counts that are and are not multiples of 8
+    (the launch pads them), with empty rows, and the arrival counters must be back at zero afterwards."""
+    D, bs, Hq, Hkv = 128, 16, 28, 4
+    g = torch.Generator().manual_seed(rows * 31 + n_split)
+    lens = torch.randint(1, 900, (rows,), generator=g).tolist()
+    if rows > 2:
+        lens[1] = 0                                             # a row with nothing to attend to
+    kv, tables = paged_problem([max(n, 1) for n in lens], bs, Hkv, D, dtype, seed=rows)
+    q = torch.randn(rows, Hq, D, generator=g).to(dtype)
+    outs = []
+    for inside in (True, False):
+        outs.append(run_paged(sb, dev, q, kv, tables, lens, wl, D ** -0.5, n_split=n_split, return_lse=True,
+                              merge_in_kernel=inside, balanced=False))
+    assert torch.equal(outs[0][0].view(torch.int16), outs[1][0].view(torch.int16))
+    assert torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32))
+    ref = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(), tables.numpy(), lens,
+                                   D ** -0.5, wl)
+    assert np.abs(outs[0][0].float().cpu().numpy() - ref).max() <= TOL[dtype]
+    ws = sb.ops._workspace(dev, 1 << 16)                        # this stream's scratch: its first 64 KiB are the counters
+    torch.cuda.synchronize()
+    assert not ws[:1 << 16].any(), "arrival counters (or the XCD fault word) left non-zero"
+
+
+def test_merge_inside_the_split_kernel_many_launches_back_to_back(sb, dev):
+    """Counters re-arm themselves: many launches in a row on one workspace, alternating shapes, no host
+    synchronisation in between, each checked against its merge-kernel twin afterwards."""
+    D, bs, Hq, Hkv = 128, 16, 28, 4
+    probs = []
+    for i, (rows, n_split) in enumerate([(64, 4), (9, 7), (33, 2), (64, 8)]):
+        g = torch.Generator().manual_seed(100 + i)
+        lens = torch.randint(200, 1500, (rows,), generator=g).tolist()
+        kv, tables = paged_problem(lens, bs, Hkv, D, torch.bfloat16, seed=i)
+        q = torch.randn(rows, Hq, D, generator=g).bfloat16()
+        probs.append((q.to(dev), kv.to(dev), tables.to(dev), torch.tensor(lens, dtype=torch.int32, device=dev), n_split))
+    call = lambda pr, inside: sb.ops.swa_decode_attention(pr[0], pr[1][0], pr[1][1], pr[3], block_table=pr[2], window_left=700,
+                                                        n_split=pr[4], merge_in_kernel=inside, balanced=False)
+    want = [call(pr, False) for pr in probs]
+    got = [call(probs[i % 4], True) for i in range(40)]
+    torch.cuda.synchronize()
+    for i, o in enumerate(got):
+        assert torch.equal(o, want[i % 4]), f"launch {i}"

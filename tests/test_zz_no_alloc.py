@@ -53,7 +53,7 @@ def test_static_scratch_matches_workspace_call_twice(sb, dev, flags):
         seq_lens = torch.tensor(lens, dtype=torch.int32, device=dev)
         need = L.sb_swa_decode_workspace_bytes(len(lens), Hq, D, n_split)
         assert 0 < need <= N.SB_SWA_DECODE_STATIC_SCRATCH_BYTES
-        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        ws = torch.zeros(need, dtype=torch.uint8, device=dev)      # a workspace starts zeroed (merge counters)
         outs = []
         for fn, w in ((L.sb_swa_decode, ws), (L.sb_swa_decode_static, None)):
             out = torch.full((len(lens), Hq, D), float("nan"), dtype=torch.bfloat16, device=dev)
