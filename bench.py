@@ -29,12 +29,38 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the matrix-core split kernel at the default workload, from rocprofv3 --pmc
-# FETCH_SIZE (251 433 KiB, scaled x2.000 by the same counter's reading of a 1 GiB stream copy) plus
-# WRITE_SIZE (3 768 KiB, scale x1.000): profiles/swa_decode_split_mfma_config2.md. Counters cannot be
-# read from inside this script, so the figure is the recorded one and is only attached when the run
-# is the default workload the profile covers.
-MEASURED_SPLIT_TRAFFIC_BYTES = (251433 * 2 + 3768) * 1024
+# HBM bytes per launch of the matrix-core split kernel at the default workload come from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs (counters cannot be read from inside this script). The profile summary records
+# them together with a hash of the kernel sources it was taken with; the figure is attached to the bench line
+# only while the sources still hash to that value.
+PROFILE_FILE = os.path.join(ROOT, "profiles", "swa_decode_split_mfma_config2.md")
+KERNEL_SOURCES = ("swa_decode_mfma.hip", "swa_decode.hip", "swa_decode_params.h", "mfma_util.h", "common.h")
+
+
+def kernel_sources_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "spikingbrain-7b_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic():
+    """(bytes per launch or None, where the figure comes from)."""
+    import re
+    try:
+        text = open(PROFILE_FILE).read()
+    except OSError:
+        return None, "no profile summary"
+    m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)\s*;\s*kernel_sources_sha256_16\s*=\s*([0-9a-f]{16})", text)
+    if not m:
+        return None, "profile summary holds no traffic record"
+    if m.group(2) != kernel_sources_hash():
+        return None, "profiles/swa_decode_split_mfma_config2.md was recorded with older kernel sources"
+    return int(m.group(1)), "rocprofv3 FETCH_SIZE + WRITE_SIZE recorded in profiles/swa_decode_split_mfma_config2.md (same kernel sources)"
+
+
 HQ, HKV, D, BS, WL = 28, 4, 128, 16, 4096
 E = 2  # bf16
 
@@ -220,6 +246,28 @@ def bench_decode_sweep(sb, dev, batches=(16, 32, 48, 64, 80, 96, 100, 128, 160, 
     return rows
 
 
+def bench_gla_step(sb, dev, B3=64, H3=28, iters=100):
+    """BASELINE config 3: one GLA decode step for 64 sequences x 28 heads, fp32 state [B, H, 128, 128] updated
+    in place; rotating over state copies larger than the on-die cache. HIP events on every launch's own dispatch."""
+    g = torch.Generator().manual_seed(0)
+    states = [(torch.randn(B3, H3, D, D, generator=g) * 0.02).to(dev) for _ in range(3)]
+    q3, k3, v3 = (torch.randn(B3, H3, 1, D, generator=g).bfloat16().to(dev) for _ in range(3))
+    g3 = (torch.nn.functional.logsigmoid(torch.randn(B3, H3, 1, D, generator=g)) / 16).to(dev)
+    o3 = torch.empty(B3, H3, 1, D, dtype=torch.bfloat16, device=dev)
+    for i in range(10):
+        sb.ops.gla_recurrent(q3, k3, v3, g3, states[i % 3], None, None, o3)
+    ev3 = [sb.ops.timing_events(dev) for _ in range(iters)]   # events on each kernel's own dispatch
+    torch.cuda.synchronize()
+    for i, pair in enumerate(ev3):
+        sb.ops.gla_recurrent(q3, k3, v3, g3, states[i % 3], None, None, o3, profile_events=pair)
+    torch.cuda.synchronize()
+    ms3 = statistics.mean(a.elapsed_time(b) for a, b in ev3)
+    bytes3 = 2 * B3 * H3 * D * D * 4 + B3 * H3 * (3 * D * 2 + D * 4 + D * 2)
+    return {"workload": f"BASELINE config 3: B={B3}, H={H3}, fp32 state", "kernel": "gla_recurrent_kernel<f32 state, one step>",
+            "kernel_ms": round(ms3, 4), "bytes_per_launch": bytes3, "GBps": round(bytes3 / (ms3 * 1e-3) / 1e9, 1),
+            "frac_hbm_peak": round(bytes3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+
 def bench_gla_prompt(sb, dev, S=16, L=8192, H=28, iters=3):
     """The GLA layers' share of BASELINE config 4 (16 prompts x 8192 tokens): one packed launch
     over token-major [tokens, H, D] projections, states read from and left in the slot cache.
@@ -344,7 +392,7 @@ def main():
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
                                                     "28-layer hybrid decode step (config 5)")
     ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "hybrid_fp8", "hybrid_lean", "hybrid_shared",
-                                       "hybrid_leanest", "gla_prompt", "decode_sweep"), default=None,
+                                       "hybrid_leanest", "gla_prompt", "gla_step", "decode_sweep"), default=None,
                     help="run just that section and print its JSON (short runs for profiling one kernel)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -363,6 +411,9 @@ def main():
         return
     if args.only == "gla_prompt":
         print(json.dumps({"gla_prompt": bench_gla_prompt(sb, dev)}))
+        return
+    if args.only == "gla_step":
+        print(json.dumps({"gla_state_update": bench_gla_step(sb, dev), "gla_state_update_b256": bench_gla_step(sb, dev, B3=256, iters=40)}))
         return
     if args.only == "decode_sweep":
         print(json.dumps({"decode_sweep": bench_decode_sweep(sb, dev)}))
@@ -389,6 +440,9 @@ def main():
         print(json.dumps({"hybrid_decode_int8_kv": bench_hybrid(sb, dev, steps=min(args.steps, 128), kv_quant="int8")}))
         return
 
+    # The CPU baseline runs first: the GPU sections then come in one block at the end of the run.
+    cpu = None if args.no_cpu_baseline else cpu_baseline()
+
     prob = build_config2(dev)
     kv, n_copies = prob["kv"], len(prob["kv"])
 
@@ -397,47 +451,53 @@ def main():
     def attend(c, phases, **kw):
         sb.ops.swa_decode_attention(prob["q"], c[0], c[1], prob["seqlens"], block_table=prob["tables"],
                                     window_left=WL, out=prob["out"], max_seq_len=prob["max_seq_len"],
-                                    n_split=args.n_split, phases=phases, force_valu=args.force_valu, **kw)
+                                    n_split=args.n_split, phases=phases, force_valu=args.force_valu, balanced=False, **kw)
 
     def step(i, events=None):
         """One layer-step as MetaAttentionImpl.forward runs a pure decode batch: the split kernel
         appends each sequence's new K/V row at its slot and attends; the merge kernel follows.
-        --unfused runs the append as a launch of its own (what mixed prefill/decode steps do)."""
+        --unfused runs the append as a launch of its own (what mixed prefill/decode steps do).
+        `events`: a (start, stop) pair of HIP events attached to the split kernel's own dispatch
+        (hipExtLaunchKernel): they put no marker of their own into the stream."""
         c = kv[i % n_copies]
         kw = new_kv
         if args.unfused:
             sb.ops.kv_append(prob["k"], prob["v"], c[0], c[1], prob["slots"])
             kw = {}
-        if events is None:
-            attend(c, 0, **kw)
-        else:  # same launches, with the split kernel bracketed by events on the launch stream
-            events[0].record()
-            attend(c, 1, **kw)
-            events[1].record()
-            attend(c, 2)
+        attend(c, 0, profile_events=events, **kw)
 
+    n_split = args.n_split or sb._native.lib().sb_swa_decode_auto_split(prob["B"], HKV, prob["max_seq_len"], WL)
+    # ONE timed region: the split kernel of every 8th step carries a pair of HIP events on its own dispatch,
+    # on the stream it is launched on (torch's current stream), so the kernel time and the step time come
+    # from the same K steps. Not every step: a launch that carries events delays the launch behind it by about
+    # 6 us on this runtime (94.4 against 88.0 us per step with events on all of them), which would be charged
+    # to `value`; the kernel's own interval is not affected.
+    timed = not args.force_valu
+    EVERY = 8
+    evs = [sb.ops.timing_events(dev) for _ in range((args.steps + EVERY - 1) // EVERY)] if timed else []
     for i in range(args.warmup):
-        step(i)
+        step(i, evs[0] if timed and i % EVERY == 0 else None)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(i)
+        step(i, evs[i // EVERY] if timed and i % EVERY == 0 else None)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
     value = prob["bytes_step"] / (wall / args.steps) / 1e9
-
-    # the dominant kernel (split kernel) inside the same step sequence: HIP events on the launch
-    # stream around each of its launches (torch's current stream is the stream the library uses)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    for i in range(args.steps):
-        step(i, evs[i])
-    torch.cuda.synchronize()
+    if not timed:  # the vector-ALU comparison kernel has no timed launch: bracket its launches in a loop of their own
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for i, (a, b) in enumerate(evs):
+            a.record()
+            attend(kv[i % n_copies], 1, **({} if args.unfused else new_kv))
+            b.record()
+            attend(kv[i % n_copies], 2)
+        torch.cuda.synchronize()
     k_ms = statistics.mean(a.elapsed_time(b) for a, b in evs)
     achieved = prob["bytes_split_kernel"] / (k_ms * 1e-3) / 1e9
 
     default_workload = not (args.force_valu or args.unfused or args.n_split)
-    n_split = args.n_split or sb._native.lib().sb_swa_decode_auto_split(prob["B"], HKV, prob["max_seq_len"], WL)
+    traffic, traffic_source = recorded_traffic() if default_workload else (None, "not the default workload")
     line = {
         "metric": "SWA decode-attn+append GB/s (% of HBM peak) and decode tok/s, 7B shapes, 1 GPU",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -451,7 +511,10 @@ def main():
         "decode_tok_per_s_layer_step": round(prob["B"] / (wall / args.steps), 1),
         "roofline": {"bound": "hbm", "kernel": "swa_decode_split_kernel<BF16,7> (vector ALU)" if args.force_valu else "swa_decode_split_mfma_kernel<BF16>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_SPLIT_TRAFFIC_BYTES if default_workload else None, "kernel_ms": round(k_ms, 4), "bytes_per_launch": prob["bytes_split_kernel"]},
+                     "traffic": traffic, "traffic_source": traffic_source, "kernel_ms": round(k_ms, 4),
+                     "kernel_ms_measured": f"HIP events on the kernel's own dispatch, every {EVERY}th launch of the timed region ({len(evs)} samples)" if timed
+                     else "HIP events around the launches of a second loop (kernel + dispatch latency)",
+                     "bytes_per_launch": prob["bytes_split_kernel"]},
     }
 
     # plain streaming copy of 1 GiB in the same run: what this box's HBM gives a copy kernel
@@ -470,27 +533,7 @@ def main():
     del src, dst
 
     if args.extras:
-        B3, H3 = 64, 28
-        g = torch.Generator().manual_seed(0)
-        states = [(torch.randn(B3, H3, D, D, generator=g) * 0.02).to(dev) for _ in range(3)]
-        q3, k3, v3 = (torch.randn(B3, H3, 1, D, generator=g).bfloat16().to(dev) for _ in range(3))
-        g3 = (torch.nn.functional.logsigmoid(torch.randn(B3, H3, 1, D, generator=g)) / 16).to(dev)
-        o3 = torch.empty(B3, H3, 1, D, dtype=torch.bfloat16, device=dev)
-        for i in range(10):
-            sb.ops.gla_recurrent(q3, k3, v3, g3, states[i % 3], None, None, o3)
-        ev3 = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(100)]
-        for i, (a, b) in enumerate(ev3):
-            a.record()
-            sb.ops.gla_recurrent(q3, k3, v3, g3, states[i % 3], None, None, o3)
-            b.record()
-        torch.cuda.synchronize()
-        ms3 = statistics.mean(a.elapsed_time(b) for a, b in ev3)
-        bytes3 = 2 * B3 * H3 * D * D * 4 + B3 * H3 * (3 * D * 2 + D * 4 + D * 2)
-        line["gla_state_update"] = {"workload": "BASELINE config 3: B=64, H=28, fp32 state", "kernel_ms": round(ms3, 4),
-                                    "GBps": round(bytes3 / (ms3 * 1e-3) / 1e9, 1),
-                                    "frac_hbm_peak": round(bytes3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
-
-        del states
+        line["gla_state_update"] = bench_gla_step(sb, dev)
         line["prefill"] = bench_prefill(sb, dev)
         torch.cuda.empty_cache()
         line["gla_prompt"] = bench_gla_prompt(sb, dev)
@@ -515,8 +558,8 @@ def main():
         line["decode_tok_per_s_28_layers"] = line["hybrid_decode"]["graph_replayed"]["decode_tok_per_s"]
         torch.cuda.empty_cache()
 
-    if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline()
+    if cpu is not None:
+        line["cpu_baseline"] = cpu
     print(json.dumps(line))
 
 

@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define SB_ABI_VERSION 1
+#define SB_ABI_VERSION 2
 
 enum sb_dtype { SB_BF16 = 0, SB_F16 = 1, SB_F32 = 2 };
 
@@ -196,6 +196,13 @@ typedef struct sb_swa_decode_args {
   const void *meta_v;
   int32_t meta_len;
   int64_t meta_stride_row, meta_stride_head;
+  /* Optional timing of the split kernel alone (both NULL = off): two hipEvent_t created with timing
+   * enabled, attached to the kernel's own dispatch (hipExtLaunchKernel), i.e. recorded when that
+   * kernel starts and when it ends, without any marker of their own in the stream. hipEventElapsedTime
+   * between them is the kernel's duration as a kernel trace shows it. Fixed-split matrix-core kernel,
+   * bf16/fp16 caches; ignored elsewhere. */
+  void *profile_start_event;
+  void *profile_stop_event;
 } sb_swa_decode_args;
 
 /* Split count the auto rule (n_split = 0) would use for these shapes: the one with the lowest estimated
@@ -291,6 +298,9 @@ typedef struct sb_gla_recurrent_args {
    * step for its whole group: the state traffic of a decode step drops G-fold, results unchanged.
    * num_heads must be a multiple of G, G <= 8. */
   int32_t q_heads_per_state;
+  /* Optional timing of the decode-step kernel (one token, one state per head), as for sb_swa_decode. */
+  void *profile_start_event;
+  void *profile_stop_event;
 } sb_gla_recurrent_args;
 
 int sb_gla_recurrent(const sb_gla_recurrent_args *args);

@@ -22,7 +22,7 @@ SB_DECODE_MERGE_IN_KERNEL = 4
 SB_KV_NONE, SB_KV_INT8, SB_KV_FP8 = 0, 1, 2
 SB_GLA_VECTOR_ONLY = 1
 SB_SWA_DECODE_STATIC_SCRATCH_BYTES = 8 << 20
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _DTYPES = {torch.bfloat16: SB_BF16, torch.float16: SB_F16, torch.float32: SB_F32}
 
@@ -60,6 +60,7 @@ class SwaDecodeArgs(C.Structure):
         ("stream", vp), ("k_scale", vp), ("v_scale", vp), ("kv_quant", i32),
         ("k_scale_tensor", f32), ("v_scale_tensor", f32),
         ("meta_k", vp), ("meta_v", vp), ("meta_len", i32), ("meta_stride_row", i64), ("meta_stride_head", i64),
+        ("profile_start_event", vp), ("profile_stop_event", vp),
     ]
 
 
@@ -75,6 +76,7 @@ class GlaRecurrentArgs(C.Structure):
         ("out_stride_b", i64), ("out_stride_h", i64), ("out_stride_t", i64),
         ("state_stride_slot", i64), ("state_stride_head", i64),
         ("num_slots", i64), ("stream", vp), ("cu_seqlens", vp), ("flags", i32), ("q_heads_per_state", i32),
+        ("profile_start_event", vp), ("profile_stop_event", vp),
     ]
 
 

@@ -9,6 +9,8 @@
 // call's last step each row-quad is stored as soon as it is updated.
 #include <type_traits>
 
+#include <hip/hip_ext.h>
+
 #include "common.h"
 
 namespace {
@@ -608,6 +610,12 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
     return check_launch("gla_recurrent_grouped_kernel");
   }
   const dim3 grid((unsigned)groups), block(256);
+  if (one && a->profile_start_event && a->profile_stop_event) {  // timed launch: events on the kernel's own dispatch
+    const hipEvent_t e0 = (hipEvent_t)a->profile_start_event, e1 = (hipEvent_t)a->profile_stop_event;
+    if (f32s) hipExtLaunchKernelGGL((gla_recurrent_kernel<true, true>), grid, block, 0, st, e0, e1, 0, p);
+    else hipExtLaunchKernelGGL((gla_recurrent_kernel<false, true>), grid, block, 0, st, e0, e1, 0, p);
+    return check_launch("gla_recurrent_kernel");
+  }
   if (f32s && one) hipLaunchKernelGGL((gla_recurrent_kernel<true, true>), grid, block, 0, st, p);
   else if (f32s) hipLaunchKernelGGL((gla_recurrent_kernel<true, false>), grid, block, 0, st, p);
   else if (one) hipLaunchKernelGGL((gla_recurrent_kernel<false, true>), grid, block, 0, st, p);

@@ -25,7 +25,7 @@
 
 namespace sb_host {
 void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
-                                  hipStream_t st, const sb::DecodeParams &p);
+                                  hipStream_t st, const sb::DecodeParams &p, hipEvent_t ev_start, hipEvent_t ev_stop);
 void launch_swa_decode_split_i8(int dtype, int kv_quant, int G, int Hkv, unsigned rows, unsigned n_split, hipStream_t st,
                                 const sb::DecodeParams &p);
 }
@@ -762,7 +762,8 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   if (a->phases != 2) {
     if (int8_kv) launch_swa_decode_split_i8(a->dtype, a->kv_quant, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p);
     else if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
-                                           (a->flags >> 4) & 7, st, p);
+                                           (a->flags >> 4) & 7, st, p, (hipEvent_t)a->profile_start_event,
+                                           (hipEvent_t)a->profile_stop_event);
     else if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
     else if (a->dtype == SB_F16) rc = launch_for_group<F16>(G, grid, st, p);
     else rc = launch_for_group<F32>(G, grid, st, p);

@@ -33,6 +33,8 @@
 // cannot leak NaNs through 0 * NaN.
 #include <type_traits>
 
+#include <hip/hip_ext.h>
+
 #include "common.h"
 #include "mfma_util.h"
 #include "swa_decode_params.h"
@@ -627,7 +629,7 @@ namespace sb_host {
 // `rows`, `n_split` give grid x and z; the kv heads are spread over wavefronts and grid y.
 // With p.n_wg > 0 the balanced kernel runs instead: p.n_wg workgroups per kv-head group.
 void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
-                                  hipStream_t st, const sb::DecodeParams &p) {
+                                  hipStream_t st, const sb::DecodeParams &p, hipEvent_t ev_start, hipEvent_t ev_stop) {
   // up to 4 wavefronts (kv heads) per workgroup: one per SIMD, each with the whole register file
   const int waves = Hkv < 4 ? Hkv : 4;
   const unsigned ygroups = (unsigned)((Hkv + waves - 1) / waves);
@@ -652,6 +654,13 @@ void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsi
       hipLaunchKernelGGL((swa_decode_split_mfma_kernel<sb::BF16, 1, 256, true>), grid, block, 0, st, p, G, Hkv);
     else
       hipLaunchKernelGGL((swa_decode_split_mfma_kernel<sb::F16, 1, 256, true>), grid, block, 0, st, p, G, Hkv);
+    return;
+  }
+  if (ev_start && ev_stop && depth == 1) {  // timed launch: the events ride on the kernel's own dispatch
+    if (dtype == SB_BF16)
+      hipExtLaunchKernelGGL((swa_decode_split_mfma_kernel<sb::BF16, 1, 256>), grid, block, 0, st, ev_start, ev_stop, 0, p, G, Hkv);
+    else
+      hipExtLaunchKernelGGL((swa_decode_split_mfma_kernel<sb::F16, 1, 256>), grid, block, 0, st, ev_start, ev_stop, 0, p, G, Hkv);
     return;
   }
 #define SB_LAUNCH(E, D) hipLaunchKernelGGL((swa_decode_split_mfma_kernel<E, D, 256>), grid, block, 0, st, p, G, Hkv)

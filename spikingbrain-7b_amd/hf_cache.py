@@ -45,14 +45,25 @@ def _capacity_for(rows: int, window: Optional[int]) -> int:
     return ((2 * base + 64 + 15) // 16) * 16
 
 
-class Cache:
+try:  # the reference's class derives from transformers' Cache (cache.py:9-11); so does this one when it is there
+    from transformers.cache_utils import Cache as _HFCache
+except Exception:  # transformers missing or too old to have cache_utils
+    _HFCache = object
+
+
+class Cache(_HFCache):
     """Drop-in for the reference `Cache` (hf_7B_model/cache.py:11).
 
     states[layer] is a dict with keys recurrent_state / attn_state / conv_state, appended in
-    layer order on each layer's first `update`.
+    layer order on each layer's first `update`. Like the reference it subclasses
+    `transformers.cache_utils.Cache` without calling its constructor (cache.py:19-25), so callers
+    that test `isinstance(past_key_values, transformers.Cache)` (HF generate plumbing) accept it;
+    every method those callers use is overridden here, none of the base class's own storage exists
+    (`layers` is an empty list).
     """
 
     def __init__(self, seen_tokens: int = 0):
+        self.layers = []  # the transformers base class's own per-layer storage: unused, kept empty
         self.states: List[Dict[str, Any]] = []
         self._seen_tokens = seen_tokens  # cache.py:25
         self._buffers: Dict[int, Tuple[_WindowBuffer, _WindowBuffer]] = {}

@@ -48,7 +48,11 @@ class MetaAttentionBackend:
 
     @staticmethod
     def get_supported_head_sizes() -> List[int]:
-        return [32, 64, 96, 128, 160, 192, 224, 256]
+        """The reference lists 32 .. 256 in steps of 32 (meta_attention.py:57-59: what flash-attn builds);
+        the gfx950 kernels here are built for head_dim 128, the 7B model's, and the list says so, so that an
+        unsupported size is refused when the layer is constructed (`MetaAttentionImpl.__init__`, the
+        reference's own check at :694-699) and not at the first launch."""
+        return [128]
 
     @staticmethod
     def get_name() -> str:

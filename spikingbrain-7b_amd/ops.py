@@ -124,8 +124,13 @@ def swa_decode_attention(
     new_slot_mapping: Optional[torch.Tensor] = None,
     meta_k: Optional[torch.Tensor] = None,
     meta_v: Optional[torch.Tensor] = None,
+    profile_events=None,
 ):
     """Single-query window attention for each row of q [R, Hq, D].
+
+    profile_events: (start, stop) torch.cuda.Event pair made by `timing_events()`: attached to the split
+    kernel's own dispatch, so start.elapsed_time(stop) is that kernel's duration alone (fixed-split
+    matrix-core kernel only).
 
     meta_k/meta_v [M, Hkv, D]: meta (sink) tokens every row also attends to, unmasked, inside the same
     softmax (key2/value2 of vllm_hymeta/attention/fa_kernel_metatoken.py:110-194, there a second
@@ -298,9 +303,26 @@ def swa_decode_attention(
         k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale),
         kv_quant=N.SB_KV_FP8 if fp8_kv else (N.SB_KV_INT8 if int8_kv else N.SB_KV_NONE),
         k_scale_tensor=float(fp8_scales[0]) if fp8_kv else 0.0, v_scale_tensor=float(fp8_scales[1]) if fp8_kv else 0.0,
-        **fused)
+        **fused, **_event_args(profile_events))
     N.check(L.sb_swa_decode(C.byref(a)), "swa_decode")
     return (out, lse) if return_lse else out
+
+
+def timing_events(device) -> Tuple[torch.cuda.Event, torch.cuda.Event]:
+    """A (start, stop) pair of timing events whose runtime handles exist already (torch creates the handle at
+    the first record), to be handed to a kernel launch through `profile_events`."""
+    pair = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+    with torch.cuda.device(device):
+        for e in pair:
+            e.record()
+    return pair
+
+
+def _event_args(profile_events) -> dict:
+    if profile_events is None:
+        return {}
+    start, stop = profile_events
+    return dict(profile_start_event=start.cuda_event, profile_stop_event=stop.cuda_event)
 
 
 def alloc_int8_kv_cache(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int, device):
@@ -656,7 +678,7 @@ def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, sc
 
 def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
                   slot_idx: Optional[torch.Tensor] = None, scale: Optional[float] = None,
-                  out: Optional[torch.Tensor] = None, vector_only: bool = False) -> torch.Tensor:
+                  out: Optional[torch.Tensor] = None, vector_only: bool = False, profile_events=None) -> torch.Tensor:
     """q, k, v, g [B, H, T, D] (any batch/head/time strides, contiguous D); state
     [slots, H, D, D] fp32 or bf16, updated in place; returns o [B, H, T, D] in q's dtype.
     Rows with slot_idx == -1 are skipped (state and output untouched).
@@ -707,7 +729,7 @@ def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
         out_stride_b=out.stride(0), out_stride_h=out.stride(1), out_stride_t=out.stride(2),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
         num_slots=state.shape[0], stream=N.stream_ptr(dev), flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0,
-        q_heads_per_state=H // Hk)
+        q_heads_per_state=H // Hk, **_event_args(profile_events))
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
 

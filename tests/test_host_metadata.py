@@ -93,3 +93,18 @@ def test_gla_slot_cache_bookkeeping(sb):
     assert cleared == [2] and (m2.cache[:, 2] == 0).all() and m2.cache[:, 1].isnan().all()
     cap = m2.get_seqlen_agnostic_capture_inputs(5)
     assert cap[1].tolist() == [sb.PAD_SLOT_ID] * 5
+
+
+def test_cache_is_a_transformers_cache(sb):
+    """hf_7B_model/cache.py:11 derives from transformers.cache_utils.Cache: code that checks the type (HF
+    generate plumbing) must accept the drop-in, and the container protocol must be the class's own."""
+    from transformers.cache_utils import Cache as HFCache
+    c = sb.Cache(seen_tokens=3)
+    assert isinstance(c, HFCache)
+    assert len(c) == 0 and list(c) == [] and c.get_seq_length(0) == 0 and c.get_max_length() is None
+    assert c._seen_tokens == 3
+    with pytest.raises(KeyError):
+        c[0]
+    legacy = ({"recurrent_state": None, "attn_state": None, "conv_state": None},)
+    c2 = sb.Cache.from_legacy_cache(legacy, seen_tokens=7)
+    assert isinstance(c2, HFCache) and len(c2) == 1 and c2.get_seq_length(0) == 7 and c2.to_legacy_cache() == legacy
