@@ -366,7 +366,8 @@ __global__ __launch_bounds__(128) void swa_decode_merge_balanced_kernel(const De
       if (p.key_lo) lo = max(lo, p.key_lo[rr]);
       n = hi > lo ? ((hi - 1) >> 5) - (lo >> 5) + 1 : 0;
     }
-    int t = n, b = rr < r ? n : 0;
+    const int len = n > 0 ? n + kBalancedRowStartChunks : 0;  // as the split kernel lays the rows out
+    int t = len, b = rr < r ? len : 0;
 #pragma unroll
     for (int k = 1; k < 64; k <<= 1) {
       t += __shfl_xor(t, k);
@@ -385,7 +386,8 @@ __global__ __launch_bounds__(128) void swa_decode_merge_balanced_kernel(const De
   float tot = 0.f, L = 0.f, M = kNegInf;
   if (n_r > 0) {
     const int per = (total + p.n_wg - 1) / p.n_wg;
-    const int w_lo = before / per, w_hi = (before + n_r - 1) / per;
+    const int own = before + kBalancedRowStartChunks;          // the row's own chunks start behind its virtual ones
+    const int w_lo = own / per, w_hi = (own + n_r - 1) / per;
     // a long row among short ones can have hundreds of partials: loads go out eight at a time
     for (int w = w_lo; w <= w_hi; w += 8) {
       float ms[8];
@@ -580,7 +582,10 @@ extern "C" int32_t sb_swa_decode_prefer_balanced(const int32_t *host_seq_lens, i
       if (end > fixed_end) fixed_end = end;
     }
   const int64_t n_wg = balanced_workgroups(num_rows, n_split < 2 ? 2 : n_split);
-  const double balanced_end = (double)((total + n_wg - 1) / n_wg) + kBalancedChunks + (double)num_rows / kBalancedRowsPerChunk;
+  int64_t nonempty = 0;
+  for (int64_t r = 0; r < num_rows; ++r) nonempty += chunks[r] > 0;
+  const int64_t laid_out = total + nonempty * kBalancedRowStartChunks;
+  const double balanced_end = (double)((laid_out + n_wg - 1) / n_wg) + kBalancedChunks + (double)num_rows / kBalancedRowsPerChunk;
   return balanced_end < fixed_end ? 1 : 0;
 }
 

@@ -586,7 +586,8 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_balanced_mfma_kerne
   if (p.rows > 64) {  // more rows than lanes: the total needs a pass of its own
     for (int base = 0; base < p.rows; base += 64) {
       int lo, hi, fc;
-      total += wave_sum(base + lane < p.rows ? row_chunks(p, seq_lens, base + lane, lo, hi, fc) : 0);
+      const int nn = base + lane < p.rows ? row_chunks(p, seq_lens, base + lane, lo, hi, fc) : 0;
+      total += wave_sum(nn > 0 ? nn + kBalancedRowStartChunks : 0);
     }
     total = __builtin_amdgcn_readfirstlane(total);
   }
@@ -595,7 +596,8 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_balanced_mfma_kerne
   for (int base = 0; base < p.rows; base += 64) {
     int lo = 0, hi = 0, fc = 0;
     const int n = base + lane < p.rows ? row_chunks(p, seq_lens, base + lane, lo, hi, fc) : 0;
-    const int incl = wave_inclusive_scan(n, lane);
+    const int len = n > 0 ? n + kBalancedRowStartChunks : 0;   // the row on the common axis: virtual chunks, then its own
+    const int incl = wave_inclusive_scan(len, lane);
     if (base == 0) {
       if (p.rows <= 64) total = __builtin_amdgcn_readlane(incl, 63);
       per = (total + n_wg - 1) / n_wg;
@@ -604,7 +606,7 @@ __global__ __launch_bounds__(kMaxThreads, 1) void swa_decode_balanced_mfma_kerne
       if (c0 >= c1) return;
     }
     if (before >= c1) break;
-    const int start = before + incl - n;  // this lane's row begins at this chunk of the whole
+    const int start = before + incl - n;  // this lane's row's own chunks begin at this chunk of the whole
     uint64_t todo = __builtin_amdgcn_ballot_w64(n > 0 && start < c1 && start + n > c0);
     while (todo) {
       const int i = __builtin_ctzll(todo);

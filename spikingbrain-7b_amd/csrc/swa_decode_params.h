@@ -1,6 +1,9 @@
 // Kernel parameter block shared by the two split kernels (VALU and matrix-core) and the merge.
 #pragma once
 #include <stdint.h>
+#ifndef SB_BALANCED_T
+#define SB_BALANCED_T 3
+#endif
 
 namespace sb {
 
@@ -9,6 +12,12 @@ namespace sb {
 constexpr int kMergeCounterBytes = 64 << 10;
 constexpr int kMergeCounters = kMergeCounterBytes / 4 - 1;
 constexpr int kMergeFaultWord = kMergeCounterBytes / 4 - 1;
+
+// Balanced split: on the common chunk axis every non-empty row is preceded by this many virtual chunks. A
+// workgroup whose run crosses into a new row drains and refills its load pipeline there (a round trip to
+// memory with nothing in flight); the virtual chunks charge that to its run, so it gets fewer real chunks
+// than a workgroup that stays inside one row. Split kernel, merge kernel and the host's cost model share it.
+constexpr int kBalancedRowStartChunks = SB_BALANCED_T;
 
 struct DecodeParams {
   const char *q;
