@@ -190,8 +190,10 @@ typedef struct sb_swa_decode_args {
    * here the 32-row chunks of the meta rows are dealt round robin to the splits of each query row's
    * window and enter the same online softmax, so out and lse are those of ONE softmax over window
    * and meta keys (a row with an empty window attends to the meta rows alone). meta_len = 0 = off.
-   * bf16/fp16 matrix-core kernel with the fixed split only (rejected with SB_DECODE_BALANCED,
-   * SB_DECODE_FORCE_VALU, fp32 or a byte-code cache). */
+   * bf16/fp16 queries on the matrix-core kernels with the fixed split only (rejected with
+   * SB_DECODE_BALANCED, SB_DECODE_FORCE_VALU or fp32). Over a byte-code cache (kv_quant) the meta rows
+   * are still elements of dtype: they are not quantised, and an fp8 cache's tensor scales do not apply
+   * to them. */
   const void *meta_k;
   const void *meta_v;
   int32_t meta_len;
@@ -391,7 +393,8 @@ typedef struct sb_swa_prefill_args {
    * second non-causal attention of all queries over k2/v2, and the log-sum-exp merge): every query
    * also attends, unmasked, to the meta_len rows of meta_k / meta_v ([meta_len, num_kv_heads, 128] of
    * dtype, strides in elements); their 32-row chunks are walked in front of each tile's window chunks,
-   * inside the same softmax, and lse covers both. meta_len = 0 = off. Not over a byte-code cache. */
+   * inside the same softmax, and lse covers both. meta_len = 0 = off. Over a byte-code cache the meta
+   * rows are still elements of dtype (not quantised, no scales). */
   const void *meta_k;
   const void *meta_v;
   int32_t meta_len;

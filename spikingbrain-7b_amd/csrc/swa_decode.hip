@@ -743,18 +743,23 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   p.meta_k = p.meta_v = nullptr;
   p.meta_len = 0;
   p.meta_sr = p.meta_sh = 0;
+  p.meta_k_mult = p.meta_v_mult = 1.f;
   if (a->meta_len < 0) return fail(SB_ERR_INVALID, "sb_swa_decode: negative meta_len");
   if (a->meta_len > 0) {
     if (!a->meta_k || !a->meta_v) return fail(SB_ERR_INVALID, "sb_swa_decode: meta_len without meta_k / meta_v");
-    if (!mfma || int8_kv || (a->flags & SB_DECODE_BALANCED))
+    if (!mfma || (a->flags & SB_DECODE_BALANCED))
       return fail(SB_ERR_UNSUPPORTED,
-                  "sb_swa_decode: meta tokens need bf16/fp16 caches on the matrix-core kernel with the fixed split");
+                  "sb_swa_decode: meta tokens need bf16/fp16 queries on the matrix-core kernel with the fixed split");
     if (((reinterpret_cast<uintptr_t>(a->meta_k) | reinterpret_cast<uintptr_t>(a->meta_v)) & 15u) ||
         (a->meta_stride_row * esz) % 16 || (a->meta_stride_head * esz) % 16 || a->meta_stride_row <= 0)
       return fail(SB_ERR_INVALID, "sb_swa_decode: meta rows must be 16-byte aligned");
     p.meta_k = (const char *)a->meta_k; p.meta_v = (const char *)a->meta_v;
     p.meta_len = a->meta_len;
     p.meta_sr = a->meta_stride_row * esz; p.meta_sh = a->meta_stride_head * esz;
+    if (fp8_kv) {
+      p.meta_k_mult = 1.f / a->k_scale_tensor;
+      p.meta_v_mult = 1.f / a->v_scale_tensor;
+    }
   }
   if (mfma && !int8_kv && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
     p.n_wg = (int)balanced_workgroups(a->num_rows, n_split);

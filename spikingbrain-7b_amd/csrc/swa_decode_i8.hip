@@ -15,7 +15,9 @@
 //     range (rows of a resident block are always addressable) and mask by key index; scales of
 //     masked keys may be stale, so masked probabilities are selected to zero, never multiplied;
 //   * the append is a launch of its own (sb_kv_append_int8): the newest row has to be quantised
-//     before it can be attended to.
+//     before it can be attended to;
+//   * meta tokens (rows every query also attends to) are not part of the cache: they stay elements of the
+//     query's type and are taken, ahead of the window, in chunks of 32 dealt round robin to the splits.
 #include "common.h"
 #include "mfma_util.h"
 #include "swa_decode_params.h"
@@ -194,6 +196,60 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     acc[6] = Mma<E>::run(v_column<E, Q, 2>(vq, 1), pb, acc[6]);
     acc[7] = Mma<E>::run(v_column<E, Q, 3>(vq, 1), pb, acc[7]);
   };
+
+  // ---- meta rows: dense element tensors [meta_len, Hkv, 128], chunk cc = rows 32cc .. 32cc+31 clamped to the
+  // last row (masked by their true index). K operand in this kernel's dim order (lane (g, c): bytes
+  // [64g, 64g+64) of row c), V rows as the element kernel takes them (lane (g, c): bytes [16c, 16c+16) of its
+  // 8 keys, transposed in registers). The rows have no scales: meta_k_mult / meta_v_mult undo the tensor
+  // scales an fp8 cache folds into scale_log2 and kv_out_scale.
+  auto meta_chunk = [&](int cc) {
+    const char *mk = p.meta_k + (int64_t)kvh * p.meta_sh, *mv = p.meta_v + (int64_t)kvh * p.meta_sh;
+    const int last = p.meta_len - 1, i0 = cc << 5;
+    const char *pk0 = mk + (int64_t)min(i0 + c, last) * p.meta_sr + g * 64;
+    const char *pk1 = mk + (int64_t)min(i0 + 16 + c, last) * p.meta_sr + g * 64;
+    uint4 v[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = *reinterpret_cast<const uint4 *>(mv + (int64_t)min(i0 + 4 * g + j, last) * p.meta_sr + c * 16);
+      v[4 + j] = *reinterpret_cast<const uint4 *>(mv + (int64_t)min(i0 + 16 + 4 * g + j, last) * p.meta_sr + c * 16);
+    }
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      s0 = Mma<E>::run(*reinterpret_cast<const uint4 *>(pk0 + s * 16), qb[s], s0);
+      s1 = Mma<E>::run(*reinterpret_cast<const uint4 *>(pk1 + s * 16), qb[s], s1);
+    }
+    float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+    bool vis[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      vis[j] = i0 + ((j >> 2) << 4) + 4 * g + (j & 3) < p.meta_len;
+      sc[j] = vis[j] ? sc[j] * p.meta_k_mult : kNegInf;
+    }
+    float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m, mx * p.scale_log2);
+    const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = fast_exp2(m - m_safe);
+    m = m_new;
+    float psum = 0.f, pv[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float e = fast_exp2(fmaf(sc[j], p.scale_log2, -m_safe));
+      psum += e;
+      pv[j] = vis[j] ? e * p.meta_v_mult : 0.f;
+    }
+    l = fmaf(l, alpha, psum);
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) acc[mt] *= alpha;
+    const uint4 pb = make_uint4(Mma<E>::pack(pv[0], pv[1]), Mma<E>::pack(pv[2], pv[3]),
+                                Mma<E>::pack(pv[4], pv[5]), Mma<E>::pack(pv[6], pv[7]));
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) acc[mt] = Mma<E>::run(v_transposed(v, mt), pb, acc[mt]);
+  };
+  if (p.meta_len > 0)
+    for (int cc = split; cc < (p.meta_len + 31) >> 5; cc += p.n_split) meta_chunk(cc);
 
   // one chunk of loads in flight behind the one being computed; two register sets, the loop
   // written out for both so that neither is ever copied

@@ -51,12 +51,15 @@ struct DecodeParams {
   const float *k_scale;
   const float *v_scale;
   float kv_out_scale;  // multiplies the result (fp8 cache: the V tensor scale; else 1)
-  // Meta tokens (matrix-core fixed split only): meta_len rows [meta_len, Hkv, 128] every query row also
-  // attends to, without mask; meta_len = 0 = none
+  // Meta tokens (matrix-core fixed split only): meta_len rows [meta_len, Hkv, 128] of the query's type every
+  // query row also attends to, without mask; meta_len = 0 = none
   const char *meta_k;
   const char *meta_v;
   int meta_len;
   int64_t meta_sr, meta_sh;  // bytes
+  // Over a byte-code cache the meta rows are still elements: their scores and probabilities are multiplied by
+  // these so that the scales folded into scale_log2 and kv_out_scale (fp8 cache) cancel for them; else 1.
+  float meta_k_mult, meta_v_mult;
 };
 
 }  // namespace sb

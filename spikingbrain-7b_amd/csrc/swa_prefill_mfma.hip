@@ -61,7 +61,7 @@ struct PrefillParams {
   int64_t q_sr, q_sh, o_sr, o_sh;  // elements
   int64_t kv_sb, kv_sr, kv_sh;     // bytes
   int64_t bt_stride;
-  // Meta tokens (element caches only): meta_len rows [meta_len, Hkv, 128] every query also attends to,
+  // Meta tokens: meta_len rows [meta_len, Hkv, 128] of the query's type every query also attends to,
   // unmasked, in the same softmax: they are walked as the chunks in front of the window's. 0 = none.
   const char *meta_k;
   const char *meta_v;
@@ -153,7 +153,10 @@ void swa_prefill_kernel(const PrefillParams p) {
   const int first_tile = wg_lo >> 4, last_tile = (wg_hi - 1) >> 4;
   const int ch_begin = wg_lo >> 5, ch_end = ((wg_hi - 1) >> 5) + 1;
   // The walk: the meta rows' chunks first (walk index x < nm), then window chunk ch_begin + x - nm.
-  const int nm = KVQ == SB_KV_NONE ? (p.meta_len + 31) >> 5 : 0;
+  // (Over a byte-code cache the meta rows, which are elements, do not fit the registers a chunk of codes
+  // travels in: there they are taken in a loop of their own in front of the walk.)
+  const int meta_chunks = (p.meta_len + 31) >> 5;
+  const int nm = KVQ == SB_KV_NONE ? meta_chunks : 0;
   const int n_walk = nm + ch_end - ch_begin;
 
   // this wavefront's two column blocks: 16-token sub-tile ts[b] of head hd[b]
@@ -278,9 +281,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   float mx[2];     // their row maxima, in log2 units
 
   // scores of chunk `ch` for both column blocks; true when some row needs a higher reference point
-  auto scores = [&](int x, int buf) -> bool {
-    const bool is_meta = x < nm;
-    const int ch = is_meta ? x : ch_begin + x - nm;
+  auto scores = [&](bool is_meta, int ch, int buf) -> bool {
     const char *sk = smem + buf * 2 * kStage;
     uint4 k0[4], k1[4];
 #pragma unroll
@@ -380,7 +381,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   auto body = [&](int x, auto par) {
     constexpr int P = decltype(par)::value;
     if (fetcher) fetch(x + 2, stage[P]);
-    if (scores(x, P)) rescale();
+    if (scores(x < nm, x < nm ? x : ch_begin + x - nm, P)) rescale();
     accumulate(P);
     if (fetcher) stash(P ^ 1, stage[P ^ 1]);
     __syncthreads();
@@ -388,8 +389,30 @@ void swa_prefill_kernel(const PrefillParams p) {
   if (fetcher) {
     fetch(0, stage[0]);
     fetch(1, stage[1]);
-    stash(0, stage[0]);
   }
+  if constexpr (KVQ != SB_KV_NONE) {
+    // meta rows over a byte-code cache: global -> LDS buffer 0 -> scores, one chunk at a time, while the
+    // first two chunks of codes are on their way
+    for (int mc = 0; mc < meta_chunks; ++mc) {
+      if (fetcher) {
+        const int64_t moff = (int64_t)kvh * p.meta_sh + c * 16;
+#pragma unroll
+        for (int u = 0; u < S::kLoads; ++u) {
+          const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
+          const int64_t row = min((mc << 5) + kk, p.meta_len - 1);
+          *reinterpret_cast<uint4 *>(smem + kk * kRowPad + c * 16) =
+              *reinterpret_cast<const uint4 *>(p.meta_k + moff + row * p.meta_sr);
+          *reinterpret_cast<uint4 *>(smem + kStage + kk * kRowPad + c * 16) =
+              *reinterpret_cast<const uint4 *>(p.meta_v + moff + row * p.meta_sr);
+        }
+      }
+      __syncthreads();
+      if (scores(true, mc, 0)) rescale();
+      accumulate(0);
+      __syncthreads();
+    }
+  }
+  if (fetcher) stash(0, stage[0]);
   __syncthreads();
   int x = 0;
   for (; x + 1 < n_walk; x += 2) {
@@ -501,7 +524,6 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   if (a->meta_len < 0) return fail(SB_ERR_INVALID, "sb_swa_prefill: negative meta_len");
   if (a->meta_len > 0) {
     if (!a->meta_k || !a->meta_v) return fail(SB_ERR_INVALID, "sb_swa_prefill: meta_len without meta_k / meta_v");
-    if (codes) return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: meta tokens are not taken over a byte-code cache");
     if (((reinterpret_cast<uintptr_t>(a->meta_k) | reinterpret_cast<uintptr_t>(a->meta_v)) & 15u) ||
         (a->meta_stride_row * 2) % 16 || (a->meta_stride_head * 2) % 16)
       return fail(SB_ERR_INVALID, "sb_swa_prefill: meta rows must be 16-byte aligned");

@@ -532,9 +532,10 @@ class MetaAttentionImpl:
         prefill_output = output[num_meta_prefill_tokens - num_prefill_query_tokens:num_meta_prefill_tokens]
         decode_output = output[num_meta_prefill_tokens:]
 
-        # Over bf16/fp16 keys the kernels take the meta rows into their own softmax (meta_k/meta_v); over
-        # a byte-code cache they are a second attention merged by log-sum-exp, the reference's own form.
-        meta_inside = with_meta and not byte_kv and query.dtype in (torch.bfloat16, torch.float16)
+        # With bf16/fp16 queries the kernels take the meta rows into their own softmax (meta_k/meta_v), over
+        # element and byte-code caches alike; fp32 queries run a second attention over the meta rows that is
+        # merged by log-sum-exp, the reference's own form.
+        meta_inside = with_meta and query.dtype in (torch.bfloat16, torch.float16)
         meta_kv = dict(meta_k=key2, meta_v=value2) if meta_inside else {}
         want_lse = with_meta and not meta_inside
 

@@ -246,8 +246,8 @@ def swa_decode_attention(
         if meta_k is None or meta_v is None:
             raise ValueError("meta_k and meta_v go together")
         N.require_gpu(q, meta_k, meta_v)
-        if int8_kv or force_valu or q.dtype not in (torch.bfloat16, torch.float16):
-            raise NotImplementedError("meta tokens inside the decode launch need bf16/fp16 caches on the matrix-core "
+        if force_valu or q.dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError("meta tokens inside the decode launch need bf16/fp16 queries on the matrix-core "
                                       "kernel (merge a separate meta_token_attention with lse_merge instead)")
         if meta_k.dim() != 3 or meta_k.shape[1:] != (Hkv, D) or meta_v.shape != meta_k.shape or \
                 meta_k.dtype != q.dtype or meta_v.dtype != q.dtype or meta_k.stride() != meta_v.stride():
@@ -607,9 +607,6 @@ def swa_prefill_attention(
         if meta_k is None or meta_v is None:
             raise ValueError("meta_k and meta_v go together")
         N.require_gpu(q, meta_k, meta_v)
-        if kv_quant != N.SB_KV_NONE:
-            raise NotImplementedError("meta tokens are not taken over a byte-code cache (merge a separate "
-                                      "meta_token_attention with lse_merge instead)")
         if meta_k.dim() != 3 or meta_k.shape[1:] != (Hkv, D) or meta_v.shape != meta_k.shape or \
                 meta_k.dtype != q.dtype or meta_v.dtype != q.dtype or meta_k.stride() != meta_v.stride():
             raise ValueError(f"meta_k and meta_v must be [meta_tokens, {Hkv}, {D}] of q's dtype with equal strides")

@@ -77,13 +77,18 @@ def expected_with_meta(q, hist_k, hist_v, k2, v2, wl, q2=None):
     return A.metatoken_attention(q, q2, hist_k, k2, hist_v, v2, D ** -0.5, wl + 1)
 
 
+@pytest.mark.parametrize("kv_quant", [None, "int8"])
 @pytest.mark.parametrize("M", [128, 32])
-def test_backend_forward_with_meta_tokens(sb, dev, M):
+def test_backend_forward_with_meta_tokens(sb, dev, M, kv_quant):
     """Prompt step with query2 (meta outputs first), chunked second prompt + decodes, then decode
-    steps, all with key2/value2; cache contents are those of the plain path."""
+    steps, all with key2/value2; cache contents are those of the plain path. kv_quant="int8": the same
+    over Int8KVCache layers (the window keys are what quantize_sym makes of them, the meta rows stay bf16)."""
+    from oracle import quant as Q
     bs, wl, nb = 16, 40, 64
     g = torch.Generator().manual_seed(M)
-    runner = sb.runner.SwaCacheRunner(1, nb, bs, wl, HKV, D, torch.bfloat16, dev, max_seqs=3, max_chunk_tokens=128)
+    runner = sb.runner.SwaCacheRunner(1, nb, bs, wl, HKV, D, torch.bfloat16, dev, max_seqs=3, max_chunk_tokens=128,
+                                      kv_quant=kv_quant)
+    stored = (lambda x: Q.quantize_sym(x, "bf16").astype(np.float32)) if kv_quant else (lambda x: x)
     impl = sb.MetaAttentionImpl(HQ, D, D ** -0.5, HKV, None, wl + 1, "auto", num_meta_tokens=M)
     k2 = torch.randn(M, HKV, D, generator=g).bfloat16()
     v2 = torch.randn(M, HKV, D, generator=g).bfloat16()
@@ -106,7 +111,8 @@ def test_backend_forward_with_meta_tokens(sb, dev, M):
         t = 0
         for sid, n in list(prompts) + [(s, 1) for s in decodes]:
             hk, hv = hist.get(sid, (np.zeros((0, HKV, D), np.float32), np.zeros((0, HKV, D), np.float32)))
-            hk = np.concatenate([hk, k[t:t + n].float().numpy()]); hv = np.concatenate([hv, v[t:t + n].float().numpy()])
+            hk = np.concatenate([hk, stored(k[t:t + n].float().numpy())])
+            hv = np.concatenate([hv, stored(v[t:t + n].float().numpy())])
             hist[sid] = (hk, hv)
             ref = expected_with_meta(q[t:t + n].float().numpy(), hk, hv, k2n, v2n, wl)
             assert np.abs(got[extra + t:extra + t + n] - ref).max() <= TOL, (sid, n)
@@ -274,3 +280,120 @@ def test_many_query_kernel_takes_meta_tokens_into_its_softmax(sb, dev, dtype, M,
     assert torch.allclose(lse, l1, atol=2e-3, rtol=1e-4)
     with pytest.raises(ValueError):
         sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), meta_k=k2.to(dev), **args)
+
+
+def _byte_code_cache(sb, dev, kind, k, v, slots, nb, bs):
+    """K/V rows stored as INT8 codes + per-row scales, or as fp8 codes with tensor scales (0.25, 0.5);
+    returns (k cache, v cache, kernel kwargs, rows as the reference's quantise-dequantise leaves them)."""
+    from oracle import quant as Q
+    Hkv = k.shape[1]
+    if kind == "int8":
+        kv, sc = sb.ops.alloc_int8_kv_cache(nb, bs, Hkv, D, dev)
+        sc.fill_(float("nan"))
+        sb.ops.kv_append_int8(k.to(dev), v.to(dev), kv[0], kv[1], sc[0], sc[1], slots.to(dev))
+        return kv[0], kv[1], dict(k_scale=sc[0], v_scale=sc[1]), \
+            Q.quantize_sym(k.float().numpy(), "bf16"), Q.quantize_sym(v.float().numpy(), "bf16")
+    raw = torch.full((2, nb, bs, Hkv, D), 0x7F, dtype=torch.uint8, device=dev)      # unwritten bytes are NaN codes
+    kv = raw.view(torch.float8_e4m3fn)
+    sb.ops.kv_append_fp8(k.to(dev), v.to(dev), kv[0], kv[1], slots.to(dev), 0.25, 0.5)
+    return kv[0], kv[1], dict(fp8_scales=(0.25, 0.5)), \
+        Q.fp8_round(k.float().numpy(), 0.25, "bf16"), Q.fp8_round(v.float().numpy(), 0.5, "bf16")
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+@pytest.mark.parametrize("n_split,M", [(1, 128), (3, 100), (4, 1), (2, 33), (0, 200)])
+def test_decode_over_byte_code_cache_takes_meta_tokens(sb, dev, kind, n_split, M):
+    """meta_k/meta_v inside the decode launch over an INT8 / fp8 cache: the meta rows stay bf16 (they are not
+    part of the cache) and share the softmax with the dequantised window keys; an fp8 cache's tensor scales,
+    folded into the softmax scale and the result, must cancel for them. One-softmax oracle over
+    [meta rows | code * scale rounded to bf16]; one row's window is empty (the meta rows alone)."""
+    bs, wl = 16, 300
+    lens = [1, 17, 300, 301, 640, 1000, 33]
+    R = len(lens)
+    g = torch.Generator().manual_seed(M + n_split)
+    nblk = [(L + bs - 1) // bs for L in lens]
+    nb = sum(nblk) + 3
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(R, max(nblk), dtype=torch.int32)
+    p0 = 0
+    for r in range(R):
+        tables[r, :nblk[r]] = perm[p0:p0 + nblk[r]]
+        p0 += nblk[r]
+    T = sum(lens)
+    k = (torch.randn(T, HKV, D, generator=g) * (0.5 + torch.rand(T, HKV, 1, generator=g))).bfloat16()
+    v = (torch.randn(T, HKV, D, generator=g) * (1 + torch.rand(T, HKV, 1, generator=g))).bfloat16()
+    slots = torch.cat([torch.tensor([int(tables[r, i // bs]) * bs + i % bs for i in range(n)], dtype=torch.int64)
+                       for r, n in enumerate(lens)])
+    kc, vc, kw, kd, vd = _byte_code_cache(sb, dev, kind, k, v, slots, nb, bs)
+    q = torch.randn(R, HQ, D, generator=g).bfloat16()
+    k2 = torch.randn(M, HKV, D, generator=g).bfloat16()
+    v2 = (torch.randn(M, HKV, D, generator=g) * 2).bfloat16()
+    key_lo = torch.zeros(R, dtype=torch.int32)
+    key_lo[6] = lens[6]
+    ref = np.zeros((R, HQ, D))
+    t0 = 0
+    for r, n in enumerate(lens):
+        k1, v1 = kd[t0 + int(key_lo[r]):t0 + n], vd[t0 + int(key_lo[r]):t0 + n]
+        t0 += n
+        if len(k1) == 0:
+            for h in range(HQ):
+                ref[r, h] = A.masked_softmax_attention(q[r:r + 1, h].double().numpy(), k2[:, h // (HQ // HKV)].double().numpy(),
+                                                       v2[:, h // (HQ // HKV)].double().numpy(), np.zeros((1, M), bool),
+                                                       D ** -0.5)[0]
+        else:
+            ref[r] = A.metatoken_attention(q[r:r + 1].float().numpy(), None, k1, k2.float().numpy(), v1, v2.float().numpy(),
+                                           D ** -0.5, wl + 1)[0]
+    args = dict(block_table=tables.to(dev), window_left=wl, key_lo=key_lo.to(dev), n_split=n_split, max_seq_len=max(lens), **kw)
+    seq = torch.tensor(lens, dtype=torch.int32, device=dev)
+    out, lse = sb.ops.swa_decode_attention(q.to(dev), kc, vc, seq, meta_k=k2.to(dev), meta_v=v2.to(dev), return_lse=True, **args)
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    assert (np.abs(got - ref) <= TOL + 2.0 ** -8 * np.abs(ref)).all()
+    # the reference's form over the same cache: two attentions merged by their log-sum-exp
+    o1, l1 = sb.ops.swa_decode_attention(q.to(dev), kc, vc, seq, return_lse=True, **args)
+    o2, l2 = sb.ops.meta_token_attention(q.to(dev), k2.to(dev), v2.to(dev))
+    sb.ops.lse_merge(o1, l1, o2, l2)
+    assert (np.abs(got - o1.float().cpu().numpy()) <= TOL + 2.0 ** -8 * np.abs(ref)).all()
+    assert torch.allclose(lse, l1, atol=2e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+@pytest.mark.parametrize("M,wl", [(128, 40), (33, 300), (1, -1), (70, 70)])
+def test_many_query_kernel_over_byte_code_cache_takes_meta_tokens(sb, dev, kind, M, wl):
+    """meta_k/meta_v inside the many-query launch reading an INT8 / fp8 paged cache (chunked prefill): the
+    meta chunks go through the kernel's LDS stage as elements ahead of the dequantised window chunks."""
+    bs = 16
+    qlens, klens = [40, 5, 130, 1], [100, 5, 230, 64]
+    g = torch.Generator().manual_seed(M + max(wl, 0))
+    need = [(n + bs - 1) // bs for n in klens]
+    nb = sum(need) + 2
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(len(klens), max(need), dtype=torch.int32)
+    p = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[p:p + n]; p += n
+    Tk, Tq = sum(klens), sum(qlens)
+    k = (torch.randn(Tk, HKV, D, generator=g) * (0.5 + torch.rand(Tk, HKV, 1, generator=g))).bfloat16()
+    v = (torch.randn(Tk, HKV, D, generator=g) * (1 + torch.rand(Tk, HKV, 1, generator=g))).bfloat16()
+    q = torch.randn(Tq, HQ, D, generator=g).bfloat16()
+    k2 = torch.randn(M, HKV, D, generator=g).bfloat16()
+    v2 = (torch.randn(M, HKV, D, generator=g) * 2).bfloat16()
+    slots = torch.cat([torch.tensor([int(tables[b, i // bs]) * bs + i % bs for i in range(n)], dtype=torch.int64)
+                       for b, n in enumerate(klens)])
+    kc, vc, kw, kd, vd = _byte_code_cache(sb, dev, kind, k, v, slots, nb, bs)
+    args = dict(query_lens=qlens, seq_lens_k=klens, block_table=tables.to(dev), window_left=wl, return_lse=True, **kw)
+    out, lse = sb.ops.swa_prefill_attention(q.to(dev), kc, vc, meta_k=k2.to(dev), meta_v=v2.to(dev), **args)
+    got = out.float().cpu().numpy()
+    assert not np.isnan(got).any() and not torch.isnan(lse).any()
+    qo = ko = 0
+    for i, (lq, lk) in enumerate(zip(qlens, klens)):
+        ref = A.metatoken_attention(q[qo:qo + lq].float().numpy(), None, kd[ko:ko + lk], k2.float().numpy(),
+                                    vd[ko:ko + lk], v2.float().numpy(), D ** -0.5, wl + 1 if wl >= 0 else 0)
+        assert (np.abs(got[qo:qo + lq] - ref) <= TOL + 2.0 ** -8 * np.abs(ref)).all(), i
+        qo += lq
+        ko += lk
+    o1, l1 = sb.ops.swa_prefill_attention(q.to(dev), kc, vc, **args)
+    o2, l2 = sb.ops.meta_token_attention(q.to(dev), k2.to(dev), v2.to(dev))
+    sb.ops.lse_merge(o1, l1, o2, l2)
+    assert (np.abs(got - o1.float().cpu().numpy()) <= TOL + 2.0 ** -7 * np.abs(got)).all()
+    assert torch.allclose(lse, l1, atol=2e-3, rtol=1e-4)
