@@ -4,23 +4,32 @@
 //   o_t  = (q_t * exp(B_t)) S_0 + sum_{s<=t} [(q_t * exp(B_t)) . (k_s * exp(-B_s))] v_s
 //   S_16 = diag(exp(B_16)) S_0 + sum_s (k_s * exp(B_16 - B_s))^T v_s
 // i.e. per block one [16x16] score product, two products into o and a rank-16 update of the state,
-// all v_mfma_f32_16x16x32_bf16 with fp32 accumulation. The reference computes prompts with fla's
+// all v_mfma_f32_16x16x32_bf16 with fp32 accumulation.
+// The decay of the state is applied every SECOND block: in between the registers hold S' = diag(exp(-L)) S,
+// L = the log-decay of the block just done, and the operands of the next block carry L in their exponents,
+//   o_t = (q_t * exp(B_t + L)) S' + intra-block term,   S' <- S' + (k_s * exp(-(B_s + L)))^T v_s,
+// after which S = diag(exp(L + B_16)) S' is formed. This halves the multiplies on the 64 state registers,
+// and k * exp(-(B_s + L)) serves both as the score operand and, transposed, as the state-update operand. The reference computes prompts with fla's
 // fused_chunk_gla (vllm_hymeta/model_for_7B/gla_attention.py:207-208), the same block mathematics.
 //
 // One workgroup per (sequence, head), four wavefronts; wavefront w keeps the state columns
 // [32w, 32w+32) as 16 accumulator tiles (64 registers) for the whole prompt: the state crosses HBM
-// once each way. Per block: all threads turn q, k, g, v into the five LDS operands (gate scan per
-// key dim in fp32), one barrier, then each wavefront runs its 30 matrix instructions. LDS is
-// double-buffered, so one barrier per block is enough; the loads of the next block are in flight
-// during the matrix phase.
+// once each way. Per block: thread (dim group r = tid / 16, token t = tid % 16) loads 8 consecutive dims of
+// its token's q, k, v (16 bytes each) and gate, five or four 16-byte loads instead of 48 two- and
+// four-byte ones (the vector memory pipe takes a wave's load at a fixed rate whatever its width); the
+// 16 tokens of a dim sit in the 16 lanes of a DPP row, so the gate scan over tokens is four row-shift
+// adds per dim. The threads turn their pieces into the five LDS operands, one barrier, then each
+// wavefront runs its 30 matrix instructions. LDS is double-buffered, so one barrier per block is
+// enough, and a wavefront prepares block n + 1 in the same stretch of code as it multiplies block n.
 //
 // Precision: 16 tokens fill half of the instruction's K = 32, and the other half carries a second
 // bf16 term: the state update uses k * exp(B_16 - B_s) as hi + lo, so the state keeps fp32-level
 // accuracy (decay and accumulation are fp32; v is bf16 as given), and the scores enter o = A v as
 // hi + lo as well (their 16 signed products per row do not average out a 2^-9 rounding). The rest of
 // the output path rounds its operands (q*exp(B), k*exp(-B), S_0) to bf16 like any bf16 GEMM.
-// exp(-B_s) grows with the gates inside one block only: 16 * max|g| stays far below the fp32/bf16
-// exponent range for any log-sigmoid gate; the exponent is clamped at 80 as a guard.
+// exp(-(B_s + L)) grows with the gates of at most two blocks: 32 * max|g| stays far below the fp32/bf16
+// exponent range for any log-sigmoid gate (|g| up to 2.5 per token, sustained); the exponent is clamped at
+// 80 as a guard.
 //
 // Tile row order: accumulator tile rt of the state holds rows 32*(rt/2) + 8*(m/4) + 4*(rt%2) + m%4
 // (m = tile row), so that the 8 consecutive rows a lane needs as the B operand of q S_0 are exactly
@@ -52,7 +61,8 @@ struct GlaChunkParams {
 
 constexpr int kCB = 16;      // tokens per block
 constexpr int kRow = 136;    // elements per row of the [16][128] operands (272 B: 16-byte aligned, banks spread)
-constexpr int kTRow = 24;    // elements per row of the transposed [128][16] operands (48 B)
+constexpr int kTRow = 20;    // elements per row of the transposed [128][16] operands (40 B: the 2-byte stores of the four
+                             // dim groups of a wavefront, 8 rows apart, then fall into different LDS banks)
 constexpr float kMaxExp = 80.f;
 
 struct Stage {
@@ -64,11 +74,20 @@ struct Stage {
   float dec[128];               // exp(B_16)
 };
 
-template <int GDT>
-__device__ __forceinline__ float load_gate(const void *p, int64_t i) {
-  if constexpr (GDT == SB_F32) return reinterpret_cast<const float *>(p)[i];
-  else if constexpr (GDT == SB_BF16) return __uint_as_float((uint32_t) reinterpret_cast<const uint16_t *>(p)[i] << 16);
-  else return (float)reinterpret_cast<const _Float16 *>(p)[i];
+// Loads through buffer descriptors: the descriptor holds a block's first row (wave-uniform, scalar registers),
+// the thread's token row and column are a 32-bit vector offset that is the same for every block: no vector
+// arithmetic per load.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_from(const char *first_row) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(first_row), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ uint4 load16(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+// x of the lane `shift` places down the row of 16 lanes, 0 where the row has no such lane
+template <int kShift>
+__device__ __forceinline__ float row_shr(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x110 + kShift, 0xf, 0xf, true));
 }
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t x) { return __uint_as_float((uint32_t)x << 16); }
@@ -98,8 +117,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int g = lane >> 4, c = lane & 15;
-  const int d = tid & 127;        // key dim (gate scan) / value column (transpose) of this thread
-  const bool second = tid >= 128;  // threads 0..127: q and k operands; 128..255: k-hat and v
+  const int r = tid >> 4;          // dims 8r .. 8r+7 of token c: this thread's piece of a block's inputs
 
   __shared__ __attribute__((aligned(16))) Stage stage[2];
 
@@ -120,87 +138,105 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                  : bf16_to_f32(reinterpret_cast<const uint16_t *>(sbase)[idx]);
       }
 
-  // ---- block inputs in registers: gates and k for every thread, q (first half) or v (second half) ----
-  float rg[kCB];
-  uint16_t rk[kCB], rx[kCB];
-  // per-thread column pointers once; a token adds a wave-uniform multiple of the row stride
-  const char *gp = reinterpret_cast<const char *>(p.g) + (go + d) * (GDT == SB_F32 ? 4 : 2);
-  const uint16_t *kp = p.k + ko + d;
-  const uint16_t *xp = second ? p.v + vo + d : p.q + qo + d;
-  const int64_t xs = second ? p.v_st : p.q_st;
-  auto fetch = [&](int t0) {
-    const int last = T - 1 - t0;  // rows past the end re-read the last token; they are zeroed when used
-    if (last >= kCB - 1) {
+  // ---- block inputs in registers: 8 dims of one token's q, k, v (bf16) and gate ---------------------------
+  constexpr int kGateBytes = GDT == SB_F32 ? 4 : 2;
+  const char *gb = reinterpret_cast<const char *>(p.g) + go * kGateBytes;
+  const char *qb = reinterpret_cast<const char *>(p.q + qo), *kb = reinterpret_cast<const char *>(p.k + ko),
+             *vb_ = reinterpret_cast<const char *>(p.v + vo);
+  const int64_t g_row = p.g_st * kGateBytes, q_row = p.q_st * 2, k_row = p.k_st * 2, v_row = p.v_st * 2, o_row = p.o_st * 2;
+  struct BlockIn {
+    uint4 q, k, v;
+    uint4 g[kGateBytes / 2];  // fp32: dims 8r..8r+3, 8r+4..8r+7; 16-bit: all 8
+  };
+  auto fetch = [&](int t0, BlockIn &in) {
+    const int tok = min(c, T - 1 - t0);  // rows past the end re-read the last token; prepare() zeroes them
+    in.q = load16(rows_from(qb + t0 * q_row), tok * (int)q_row + r * 16);
+    in.k = load16(rows_from(kb + t0 * k_row), tok * (int)k_row + r * 16);
+    in.v = load16(rows_from(vb_ + t0 * v_row), tok * (int)v_row + r * 16);
+    const __amdgpu_buffer_rsrc_t gr = rows_from(gb + t0 * g_row);
 #pragma unroll
-      for (int t = 0; t < kCB; ++t) {
-        rg[t] = load_gate<GDT>(gp, (t0 + t) * p.g_st);
-        rk[t] = kp[(t0 + t) * p.k_st];
-        rx[t] = xp[(t0 + t) * xs];
-      }
+    for (int j = 0; j < kGateBytes / 2; ++j) in.g[j] = load16(gr, tok * (int)g_row + r * 8 * kGateBytes + 16 * j);
+  };
+
+  // ---- the five LDS operands of one block. Gates in log2 units (bare v_exp afterwards); a token past the
+  // end of the prompt is a token with g = 0, q = k = v = 0 ------------------------------------------------
+  auto fix_tail = [&](BlockIn &in, int t0) {
+    if (t0 + kCB > T && t0 + c >= T) {
+      in.q = in.k = in.v = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int j = 0; j < kGateBytes / 2; ++j) in.g[j] = make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+  // kSecond = false: first block of a pair (state undecayed on entry: L = 0); leaves L = its total log-decay
+  // in `carry` and, for the case that the prompt ends here, in st.dec (log2 units).
+  // kSecond = true: exponents carry L; st.dec = exp(L + B_16), the decay multiply() applies afterwards.
+  float carry[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) carry[i] = 0.f;
+  auto prepare = [&](const BlockIn &in, Stage &st, auto second_tag) {
+    constexpr bool kSecond = decltype(second_tag)::value;
+    const uint4 rq = in.q, rk = in.k, rv = in.v;
+    float B[8], tot[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float x;
+      if constexpr (GDT == SB_F32) x = __uint_as_float(word(in.g[i >> 2], i & 3));
+      else if constexpr (GDT == SB_BF16) x = (i & 1) ? bf16_hi(word(in.g[0], i >> 1)) : bf16_lo(word(in.g[0], i >> 1));
+      else x = (i & 1) ? f16_hi(word(in.g[0], i >> 1)) : f16_lo(word(in.g[0], i >> 1));
+      x *= kLog2e;
+      // inclusive scan over the 16 tokens = the 16 lanes of this row
+      x += row_shr<1>(x);
+      x += row_shr<2>(x);
+      x += row_shr<4>(x);
+      x += row_shr<8>(x);
+      if constexpr (kSecond) x += carry[i];
+      B[i] = x;
+      tot[i] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane | 15) << 2, __builtin_bit_cast(int, x)));
+    }
+    float qf[8], kf[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      qf[2 * i] = bf16_lo(word(rq, i));
+      qf[2 * i + 1] = bf16_hi(word(rq, i));
+      kf[2 * i] = bf16_lo(word(rk, i));
+      kf[2 * i + 1] = bf16_hi(word(rk, i));
+    }
+    uint32_t qs[4], ks[4];
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      qs[i / 2] = Mma<BF16>::pack(qf[i] * p.scale * fast_exp2(B[i]), qf[i + 1] * p.scale * fast_exp2(B[i + 1]));
+      const float x0 = kf[i] * fast_exp2(fminf(-B[i], kMaxExp * kLog2e)), x1 = kf[i + 1] * fast_exp2(fminf(-B[i + 1], kMaxExp * kLog2e));
+      // the rounded value is the score operand and the high part of the state-update operand
+      const uint32_t h = Mma<BF16>::pack(x0, x1);
+      const uint32_t l = Mma<BF16>::pack(x0 - __uint_as_float(h << 16), x1 - __uint_as_float(h & 0xffff0000u));
+      const uint32_t vv = word(rv, i / 2);
+      ks[i / 2] = h;
+      // the transposed operands [dim][token]: one 2-byte store per dim
+      st.kh_hi[8 * r + i][c] = (uint16_t)h;
+      st.kh_hi[8 * r + i + 1][c] = (uint16_t)(h >> 16);
+      st.kh_lo[8 * r + i][c] = (uint16_t)l;
+      st.kh_lo[8 * r + i + 1][c] = (uint16_t)(l >> 16);
+      st.vt[8 * r + i][c] = (uint16_t)vv;
+      st.vt[8 * r + i + 1][c] = (uint16_t)(vv >> 16);
+    }
+    *reinterpret_cast<uint4 *>(&st.qs[c][8 * r]) = make_uint4(qs[0], qs[1], qs[2], qs[3]);
+    *reinterpret_cast<uint4 *>(&st.ks[c][8 * r]) = make_uint4(ks[0], ks[1], ks[2], ks[3]);
+    // (every lane of the row holds the same totals and stores them to the same address: no branch here)
+    if constexpr (kSecond) {
+      *reinterpret_cast<float4 *>(&st.dec[8 * r]) = make_float4(fast_exp2(tot[0]), fast_exp2(tot[1]), fast_exp2(tot[2]), fast_exp2(tot[3]));
+      *reinterpret_cast<float4 *>(&st.dec[8 * r + 4]) = make_float4(fast_exp2(tot[4]), fast_exp2(tot[5]), fast_exp2(tot[6]), fast_exp2(tot[7]));
     } else {
+      *reinterpret_cast<float4 *>(&st.dec[8 * r]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
+      *reinterpret_cast<float4 *>(&st.dec[8 * r + 4]) = make_float4(tot[4], tot[5], tot[6], tot[7]);
 #pragma unroll
-      for (int t = 0; t < kCB; ++t) {
-        const int64_t tt = t0 + min(t, last);
-        rg[t] = load_gate<GDT>(gp, tt * p.g_st);
-        rk[t] = kp[tt * p.k_st];
-        rx[t] = xp[tt * xs];
-      }
+      for (int i = 0; i < 8; ++i) carry[i] = tot[i];
     }
   };
 
-  const int n_blocks = (T + kCB - 1) / kCB;
-  fetch(0);
-  for (int blk = 0; blk < n_blocks; ++blk) {
-    Stage &st = stage[blk & 1];
-    const int t0 = blk * kCB;
-    // ---- operands of this block ------------------------------------------------------------------
-    {
-      float B[kCB];
-      float run = 0.f;
-#pragma unroll
-      for (int t = 0; t < kCB; ++t) {
-        run += (t0 + t < T) ? rg[t] : 0.f;
-        B[t] = run;
-      }
-      if (!second) {
-#pragma unroll
-        for (int t = 0; t < kCB; ++t) {
-          const bool live = t0 + t < T;
-          const float qv = live ? bf16_to_f32(rx[t]) : 0.f, kv = live ? bf16_to_f32(rk[t]) : 0.f;
-          st.qs[t][d] = f32_to_bf16(qv * __expf(B[t]) * p.scale);
-          st.ks[t][d] = f32_to_bf16(kv * __expf(fminf(-B[t], kMaxExp)));
-        }
-        st.dec[d] = __expf(run);
-      } else {
-        uint32_t hi[kCB / 2], lo[kCB / 2], vv[kCB / 2];
-#pragma unroll
-        for (int t = 0; t < kCB; t += 2) {
-          float x[2];
-          uint16_t xh[2], xl[2], xv[2];
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            const bool live = t0 + t + u < T;
-            x[u] = live ? bf16_to_f32(rk[t + u]) * __expf(run - B[t + u]) : 0.f;
-            xh[u] = f32_to_bf16(x[u]);
-            xl[u] = f32_to_bf16(x[u] - bf16_to_f32(xh[u]));
-            xv[u] = live ? rx[t + u] : (uint16_t)0;
-          }
-          hi[t / 2] = xh[0] | ((uint32_t)xh[1] << 16);
-          lo[t / 2] = xl[0] | ((uint32_t)xl[1] << 16);
-          vv[t / 2] = xv[0] | ((uint32_t)xv[1] << 16);
-        }
-        reinterpret_cast<uint4 *>(&st.kh_hi[d][0])[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        reinterpret_cast<uint4 *>(&st.kh_hi[d][0])[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-        reinterpret_cast<uint4 *>(&st.kh_lo[d][0])[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        reinterpret_cast<uint4 *>(&st.kh_lo[d][0])[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-        reinterpret_cast<uint4 *>(&st.vt[d][0])[0] = make_uint4(vv[0], vv[1], vv[2], vv[3]);
-        reinterpret_cast<uint4 *>(&st.vt[d][0])[1] = make_uint4(vv[4], vv[5], vv[6], vv[7]);
-      }
-    }
-    if (blk + 1 < n_blocks) fetch(t0 + kCB);  // in flight during the matrix phase
-    __syncthreads();
-
-    // ---- scores (transposed): at[i] = A[t = c][s = 4g + i], zero above the diagonal ------------------
+  // ---- the 30 matrix instructions of one block on this wavefront's 32 state columns ---------------------
+  auto multiply = [&](int t0, const Stage &st, auto second_tag) {
+    constexpr bool kSecond = decltype(second_tag)::value;
+    // scores (transposed): at[i] = A[t = c][s = 4g + i], zero above the diagonal
     uint4 qa[4];
     f32x4_t at = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -215,15 +251,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // as the A operand of o = A v: row t = c, k index 8g + j <-> s = 4g + j for j < 4; the scores go in
     // as two bf16 terms (hi in k index 0..3, lo in 4..7, against v repeated), so that the 16 signed
     // products of a row are summed from scores good to 16 bits
-    float at_lo[4];
-    uint16_t at_hi[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      at_hi[i] = f32_to_bf16(at[i]);
-      at_lo[i] = at[i] - bf16_to_f32(at_hi[i]);
-    }
-    const uint4 pa = make_uint4(at_hi[0] | ((uint32_t)at_hi[1] << 16), at_hi[2] | ((uint32_t)at_hi[3] << 16),
-                                Mma<BF16>::pack(at_lo[0], at_lo[1]), Mma<BF16>::pack(at_lo[2], at_lo[3]));
+    const uint32_t h01 = Mma<BF16>::pack(at[0], at[1]), h23 = Mma<BF16>::pack(at[2], at[3]);
+    const uint4 pa = make_uint4(h01, h23,
+                                Mma<BF16>::pack(at[0] - __uint_as_float(h01 << 16), at[1] - __uint_as_float(h01 & 0xffff0000u)),
+                                Mma<BF16>::pack(at[2] - __uint_as_float(h23 << 16), at[3] - __uint_as_float(h23 & 0xffff0000u)));
 
     // v as the B operand of both products: v[s = 4g + j][col] at k index j and again at 4 + j, so
     // that the A operands can carry a high term in k index 0..3 and a low term in 4..7 (16 tokens
@@ -235,7 +266,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       vb[nt] = make_uint4(x.x, x.y, x.x, x.y);
     }
 
-    // ---- o^T = v^T A^T + S_0^T (q exp B)^T: lane (g, c) ends up with token c, columns 4g..4g+3 of each tile:
+    // o^T = v^T A^T + S_0^T (q exp B)^T: lane (g, c) ends up with token c, columns 4g..4g+3 of each tile:
     // one 8-byte store per tile (the operand registers are the same either way round: a lane holds
     // index c of the tile's outer dimension and 8g..8g+7 of the contraction in both operands)
     f32x4_t o[2];
@@ -250,26 +281,75 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         o[nt] = Mma<BF16>::run(sb16, qa[s4], o[nt]);
       }
     }
-    if (t0 + c < T) {
+    {  // rows past the end of the prompt fall outside the descriptor and are dropped: no branch in this code
+      const __amdgpu_buffer_rsrc_t orows = __builtin_amdgcn_make_buffer_rsrc(
+          reinterpret_cast<char *>(p.out + oo) + t0 * o_row, 0, min(kCB, T - t0) * (int)o_row, 0x00020000);
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-        *reinterpret_cast<uint2 *>(p.out + oo + (int64_t)(t0 + c) * p.o_st + 32 * w + 16 * nt + 4 * g) =
-            make_uint2(Mma<BF16>::pack(o[nt][0], o[nt][1]), Mma<BF16>::pack(o[nt][2], o[nt][3]));
+      for (int nt = 0; nt < 2; ++nt) {
+        typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+        u32x2_t val;
+        val.x = Mma<BF16>::pack(o[nt][0], o[nt][1]);
+        val.y = Mma<BF16>::pack(o[nt][2], o[nt][3]);
+        __builtin_amdgcn_raw_buffer_store_b64(val, orows, c * (int)o_row + (32 * w + 16 * nt + 4 * g) * 2, 0, 0);
+      }
     }
 
-    // ---- S <- diag(exp B_16) S + k-hat^T v ------------------------------------------------------------
+    // S' <- S' + k-hat^T v, and after the second block of a pair S <- diag(exp(L + B_16)) S'
 #pragma unroll
     for (int rt = 0; rt < 8; ++rt) {
-      const float4 dc = *reinterpret_cast<const float4 *>(&st.dec[32 * (rt >> 1) + 8 * g + 4 * (rt & 1)]);
       const int row = 32 * (rt >> 1) + 8 * (c >> 2) + 4 * (rt & 1) + (c & 3);
       const uint2 h2 = *reinterpret_cast<const uint2 *>(&st.kh_hi[row][4 * g]);
       const uint2 l2 = *reinterpret_cast<const uint2 *>(&st.kh_lo[row][4 * g]);
       const uint4 ka = make_uint4(h2.x, h2.y, l2.x, l2.y);
 #pragma unroll
+      for (int nt = 0; nt < 2; ++nt) S[rt][nt] = Mma<BF16>::run(ka, vb[nt], S[rt][nt]);
+      if constexpr (kSecond) {
+        const float4 dc = *reinterpret_cast<const float4 *>(&st.dec[32 * (rt >> 1) + 8 * g + 4 * (rt & 1)]);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+          S[rt][nt][0] *= dc.x; S[rt][nt][1] *= dc.y; S[rt][nt][2] *= dc.z; S[rt][nt][3] *= dc.w;
+        }
+      }
+    }
+  };
+
+  // ---- block loop. An iteration runs the matrix instructions of block blk and turns the inputs of block
+  // blk + 1 into the other LDS stage, then fetches the inputs of block blk + 2 into the registers just used; a
+  // fetch past the last block re-reads it, and the block after the last is prepared as 16 dead tokens (never
+  // multiplied). One barrier per block: what an iteration writes was last read one iteration before the
+  // barrier it follows. Blocks go in pairs (first, second); a prompt that ends on a first block leaves
+  // S' = diag(exp(-L)) S in the registers, put right after the loop.
+  const int n_blocks = (T + kCB - 1) / kCB;
+  const std::false_type kFirst{};
+  const std::true_type kSecond{};
+  BlockIn in;
+  fetch(0, in);
+  fix_tail(in, 0);
+  prepare(in, stage[0], kFirst);
+  fetch(min(1, n_blocks - 1) * kCB, in);
+  int blk = 0;
+  for (; blk + 1 < n_blocks; blk += 2) {
+    __syncthreads();
+    fix_tail(in, (blk + 1) * kCB);
+    multiply(blk * kCB, stage[0], kFirst);
+    prepare(in, stage[1], kSecond);
+    fetch(min(blk + 2, n_blocks - 1) * kCB, in);
+    __syncthreads();
+    fix_tail(in, (blk + 2) * kCB);
+    multiply((blk + 1) * kCB, stage[1], kSecond);
+    prepare(in, stage[0], kFirst);
+    fetch(min(blk + 3, n_blocks - 1) * kCB, in);
+  }
+  if (blk < n_blocks) {
+    __syncthreads();
+    multiply(blk * kCB, stage[0], kFirst);
+#pragma unroll
+    for (int rt = 0; rt < 8; ++rt) {
+      const float4 dc = *reinterpret_cast<const float4 *>(&stage[0].dec[32 * (rt >> 1) + 8 * g + 4 * (rt & 1)]);
+#pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
-        f32x4_t s = S[rt][nt];
-        s[0] *= dc.x; s[1] *= dc.y; s[2] *= dc.z; s[3] *= dc.w;
-        S[rt][nt] = Mma<BF16>::run(ka, vb[nt], s);
+        S[rt][nt][0] *= fast_exp2(dc.x); S[rt][nt][1] *= fast_exp2(dc.y);
+        S[rt][nt][2] *= fast_exp2(dc.z); S[rt][nt][3] *= fast_exp2(dc.w);
       }
     }
   }
