@@ -18,7 +18,7 @@
 // its token's q, k, v (16 bytes each) and gate, five or four 16-byte loads instead of 48 two- and
 // four-byte ones (the vector memory pipe takes a wave's load at a fixed rate whatever its width); the
 // 16 tokens of a dim sit in the 16 lanes of a DPP row, so the gate scan over tokens is four row-shift
-// adds per dim. The threads turn their pieces into the five LDS operands, one barrier, then each
+// adds per dim. The threads turn their pieces into the four LDS operands, one barrier, then each
 // wavefront runs its 30 matrix instructions. LDS is double-buffered, so one barrier per block is
 // enough, and a wavefront prepares block n + 1 in the same stretch of code as it multiplies block n.
 //
@@ -60,19 +60,32 @@ struct GlaChunkParams {
 };
 
 constexpr int kCB = 16;      // tokens per block
-constexpr int kRow = 136;    // elements per row of the [16][128] operands (272 B: 16-byte aligned, banks spread)
-constexpr int kTRow = 20;    // elements per row of the transposed [128][16] operands (40 B: the 2-byte stores of the four
-                             // dim groups of a wavefront, 8 rows apart, then fall into different LDS banks)
+#ifndef SB_GLA_ROW
+#define SB_GLA_ROW 152
+#endif
+constexpr int kRow = SB_GLA_ROW;    // elements per row of the [16 tokens][128] LDS operands (304 B = 76 dwords: the 16-byte
+                             // stores and loads of 16 rows and the transposing loads of 4 rows spread over the banks)
 constexpr float kMaxExp = 80.f;
 
+// All operands are stored token-major, one 16-byte store per thread each. The state update and the output
+// product contract over tokens and need [dim][token] operands: those are read with the transposing LDS load
+// (ds_read_b64_tr_b16), no transposed copy is ever written.
 struct Stage {
-  uint16_t qs[kCB][kRow];       // q * exp(B_t) * scale
-  uint16_t ks[kCB][kRow];       // k * exp(-B_t)
-  uint16_t kh_hi[128][kTRow];   // (k * exp(B_16 - B_t))^T, high part
-  uint16_t kh_lo[128][kTRow];   // low part
-  uint16_t vt[128][kTRow];      // v^T
-  float dec[128];               // exp(B_16)
+  uint16_t qs[kCB][kRow];  // q * exp(B_t + L) * scale
+  uint16_t ks[kCB][kRow];  // k * exp(-(B_t + L)) rounded to bf16: score operand, and high part of the state-update operand
+  uint16_t kl[kCB][kRow];  // what the rounding left: low part of the state-update operand
+  uint16_t vs[kCB][kRow];  // v as loaded
+  float dec[128];          // exp(L + B_16) (second block of a pair), L + B_16 in log2 units (first block)
 };
+
+// ds_read_b64_tr_b16: in every group of 16 lanes, lane i names 8 bytes (4 elements) of LDS, "row i"; lane l
+// receives element l % 4 of rows l / 4, l / 4 + 4, l / 4 + 8, l / 4 + 12 (checked on the GPU). With row
+// i = (token t0 + i / 4, dims f(i % 4) .. + 3), lane l gets dim f(l / 4) + l % 4 of tokens t0 .. t0 + 3.
+__device__ __forceinline__ uint2 load_transposed(const uint16_t *row) {
+  typedef short v4s __attribute__((ext_vector_type(4)));
+  const v4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)row);
+  return __builtin_bit_cast(uint2, v);
+}
 
 // Loads through buffer descriptors: the descriptor holds a block's first row (wave-uniform, scalar registers),
 // the thread's token row and column are a 32-bit vector offset that is the same for every block: no vector
@@ -158,7 +171,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int j = 0; j < kGateBytes / 2; ++j) in.g[j] = load16(gr, tok * (int)g_row + r * 8 * kGateBytes + 16 * j);
   };
 
-  // ---- the five LDS operands of one block. Gates in log2 units (bare v_exp afterwards); a token past the
+  // ---- the four LDS operands of one block. Gates in log2 units (bare v_exp afterwards); a token past the
   // end of the prompt is a token with g = 0, q = k = v = 0 ------------------------------------------------
   auto fix_tail = [&](BlockIn &in, int t0) {
     if (t0 + kCB > T && t0 + c >= T) {
@@ -201,7 +214,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       kf[2 * i] = bf16_lo(word(rk, i));
       kf[2 * i + 1] = bf16_hi(word(rk, i));
     }
-    uint32_t qs[4], ks[4];
+    uint32_t qs[4], ks[4], kl[4];
 #pragma unroll
     for (int i = 0; i < 8; i += 2) {
       qs[i / 2] = Mma<BF16>::pack(qf[i] * p.scale * fast_exp2(B[i]), qf[i + 1] * p.scale * fast_exp2(B[i + 1]));
@@ -209,18 +222,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       // the rounded value is the score operand and the high part of the state-update operand
       const uint32_t h = Mma<BF16>::pack(x0, x1);
       const uint32_t l = Mma<BF16>::pack(x0 - __uint_as_float(h << 16), x1 - __uint_as_float(h & 0xffff0000u));
-      const uint32_t vv = word(rv, i / 2);
       ks[i / 2] = h;
-      // the transposed operands [dim][token]: one 2-byte store per dim
-      st.kh_hi[8 * r + i][c] = (uint16_t)h;
-      st.kh_hi[8 * r + i + 1][c] = (uint16_t)(h >> 16);
-      st.kh_lo[8 * r + i][c] = (uint16_t)l;
-      st.kh_lo[8 * r + i + 1][c] = (uint16_t)(l >> 16);
-      st.vt[8 * r + i][c] = (uint16_t)vv;
-      st.vt[8 * r + i + 1][c] = (uint16_t)(vv >> 16);
+      kl[i / 2] = l;
     }
     *reinterpret_cast<uint4 *>(&st.qs[c][8 * r]) = make_uint4(qs[0], qs[1], qs[2], qs[3]);
     *reinterpret_cast<uint4 *>(&st.ks[c][8 * r]) = make_uint4(ks[0], ks[1], ks[2], ks[3]);
+    *reinterpret_cast<uint4 *>(&st.kl[c][8 * r]) = make_uint4(kl[0], kl[1], kl[2], kl[3]);
+    *reinterpret_cast<uint4 *>(&st.vs[c][8 * r]) = rv;
     // (every lane of the row holds the same totals and stores them to the same address: no branch here)
     if constexpr (kSecond) {
       *reinterpret_cast<float4 *>(&st.dec[8 * r]) = make_float4(fast_exp2(tot[0]), fast_exp2(tot[1]), fast_exp2(tot[2]), fast_exp2(tot[3]));
@@ -262,7 +270,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     uint4 vb[2];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
-      const uint2 x = *reinterpret_cast<const uint2 *>(&st.vt[32 * w + 16 * nt + c][4 * g]);
+      const uint2 x = load_transposed(&st.vs[4 * g + (c >> 2)][32 * w + 16 * nt + 4 * (c & 3)]);
       vb[nt] = make_uint4(x.x, x.y, x.x, x.y);
     }
 
@@ -297,9 +305,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // S' <- S' + k-hat^T v, and after the second block of a pair S <- diag(exp(L + B_16)) S'
 #pragma unroll
     for (int rt = 0; rt < 8; ++rt) {
-      const int row = 32 * (rt >> 1) + 8 * (c >> 2) + 4 * (rt & 1) + (c & 3);
-      const uint2 h2 = *reinterpret_cast<const uint2 *>(&st.kh_hi[row][4 * g]);
-      const uint2 l2 = *reinterpret_cast<const uint2 *>(&st.kh_lo[row][4 * g]);
+      // this lane's operand row is state row 32 (rt / 2) + 8 (c / 4) + 4 (rt % 2) + c % 4: f(j) = 32 (rt / 2) + 8 j + 4 (rt % 2)
+      const int tok = 4 * g + (c >> 2), dims = 32 * (rt >> 1) + 8 * (c & 3) + 4 * (rt & 1);
+      const uint2 h2 = load_transposed(&st.ks[tok][dims]);
+      const uint2 l2 = load_transposed(&st.kl[tok][dims]);
       const uint4 ka = make_uint4(h2.x, h2.y, l2.x, l2.y);
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) S[rt][nt] = Mma<BF16>::run(ka, vb[nt], S[rt][nt]);
