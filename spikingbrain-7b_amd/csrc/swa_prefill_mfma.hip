@@ -15,11 +15,12 @@
 //   The workgroup walks the union of its tokens' windows in chunks of 32 keys. Each chunk of K and V
 //   (32 rows x 256 B each) is fetched from global memory ONCE per workgroup (the first four wavefronts
 //   fetch 8 rows each with whole-row 16-byte lanes) into a double-buffered LDS stage whose rows are
-//   padded to 272 B; all wavefronts then read their MFMA operands from LDS. Global loads run two chunks
+//   padded to 272 B (K) and 288 B (V); all wavefronts then read their MFMA operands from LDS. Global loads run two chunks
 //   ahead of the arithmetic (two register sets used alternately, the loop written out for both).
 //   Per chunk and column block: S^T = K Q^T (8 MFMA 16x16x32, tokens on the N axis), softmax numerators
 //   per lane for token lane%16 in log2 units, O^T += V^T P^T (8 MFMA). P stays in the lane that produced
-//   it; V^T operands come from an in-register 8x8 transpose shared by the two blocks.
+//   it; V^T operands come out of the [key][dim] stage through the transposing LDS load, shared by the two
+//   blocks.
 //   Workgroups are numbered so that each XCD (own L2) works through one contiguous run of tiles.
 //
 // Softmax reference point
@@ -69,8 +70,22 @@ struct PrefillParams {
   int64_t meta_sr, meta_sh;  // bytes
 };
 
-constexpr int kRowPad = 272;         // LDS row stride: 256 B of data + 16 B
-constexpr int kStage = 32 * kRowPad;  // one K or V chunk
+#ifndef SB_PREFILL_HEADS
+#define SB_PREFILL_HEADS 4
+#endif
+constexpr int kRowPad = 272;   // LDS row stride of a K chunk: 256 B of data + 16 B (16-byte operand loads, 16 rows at a time)
+constexpr int kRowPadV = 288;  // of a V chunk: 256 B + 32 B (transposing loads: 4 rows x 32 B at a time)
+constexpr int kStageK = 32 * kRowPad, kStageV = 32 * kRowPadV;
+constexpr int kStage = kStageK + kStageV;  // one chunk of K and V
+
+// ds_read_b64_tr_b16: in every group of 16 lanes, lane i names 8 bytes (4 elements) of LDS, "row i"; lane l
+// receives element l % 4 of rows l / 4, l / 4 + 4, l / 4 + 8, l / 4 + 12. With row i = (key k0 + i / 4, dims
+// d0 + 4 (i % 4) .. + 3), lane l gets dim d0 + l of keys k0 .. k0 + 3: V^T straight out of a [key][dim] stage.
+__device__ __forceinline__ uint2 load_transposed(const char *row) {
+  typedef short v4s __attribute__((ext_vector_type(4)));
+  const v4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)row);
+  return __builtin_bit_cast(uint2, v);
+}
 constexpr float kNegInf = kNegInfF;
 constexpr float kRaise = 8.f;
 
@@ -121,7 +136,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * Shape<NHEADS>::kWaves
                           amdgpu_waves_per_eu(2, 2)))
 void swa_prefill_kernel(const PrefillParams p) {
   using S = Shape<NHEADS>;
-  __shared__ __attribute__((aligned(16))) char smem[2 * 2 * kStage];  // [buffer][K|V]
+  __shared__ __attribute__((aligned(16))) char smem[2 * kStage];  // [buffer][K|V]
 
   // Workgroups are handed to the 8 XCDs round-robin by index, and each XCD has its own L2. Give XCD x
   // the x-th contiguous eighth of the tiles, so that the workgroups resident on one XCD at a time are
@@ -257,7 +272,7 @@ void swa_prefill_kernel(const PrefillParams p) {
     }
   };
   auto stash = [&](int buf, const Set &st) {
-    char *sk = smem + buf * 2 * kStage, *sv = sk + kStage;
+    char *sk = smem + buf * kStage, *sv = sk + kStageK;
 #pragma unroll
     for (int u = 0; u < S::kLoads; ++u) {
       const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
@@ -273,7 +288,7 @@ void swa_prefill_kernel(const PrefillParams p) {
         vq = dequant8<E, KVQ>(st.v[u], p.v_scale_tensor);
       }
       *reinterpret_cast<uint4 *>(sk + kk * kRowPad + c * 16) = kq;
-      *reinterpret_cast<uint4 *>(sv + kk * kRowPad + c * 16) = vq;
+      *reinterpret_cast<uint4 *>(sv + kk * kRowPadV + c * 16) = vq;
     }
   };
 
@@ -282,7 +297,7 @@ void swa_prefill_kernel(const PrefillParams p) {
 
   // scores of chunk `ch` for both column blocks; true when some row needs a higher reference point
   auto scores = [&](bool is_meta, int ch, int buf) -> bool {
-    const char *sk = smem + buf * 2 * kStage;
+    const char *sk = smem + buf * kStage;
     uint4 k0[4], k1[4];
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -326,7 +341,7 @@ void swa_prefill_kernel(const PrefillParams p) {
 
   // numerators against the current reference points, then O^T += V^T P^T
   auto accumulate = [&](int buf) {
-    const char *sv = smem + buf * 2 * kStage + kStage;
+    const char *sv = smem + buf * kStage + kStageK;
     uint4 pb[2];
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
@@ -341,15 +356,13 @@ void swa_prefill_kernel(const PrefillParams p) {
       pb[b] = make_uint4(Mma<E>::pack(sc[b][0], sc[b][1]), Mma<E>::pack(sc[b][2], sc[b][3]),
                          Mma<E>::pack(sc[b][4], sc[b][5]), Mma<E>::pack(sc[b][6], sc[b][7]));
     }
-    uint4 v[8];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      v[j] = *reinterpret_cast<const uint4 *>(sv + (4 * g + j) * kRowPad + c * 16);
-      v[4 + j] = *reinterpret_cast<const uint4 *>(sv + (16 + 4 * g + j) * kRowPad + c * 16);
-    }
+    // V^T operand of dims 16 mt + c: this lane's 8 keys (4g .. 4g+3 of either 16-key tile, the order of its
+    // probabilities) by two transposing loads; built once, used by both blocks
+    const char *v0 = sv + (4 * g + (c >> 2)) * kRowPadV + (c & 3) * 8, *v1 = v0 + 16 * kRowPadV;
 #pragma unroll
     for (int mt = 0; mt < 8; ++mt) {
-      const uint4 vt = v_transposed(v, mt);  // built once, used by both blocks
+      const uint2 lo = load_transposed(v0 + mt * 32), hi = load_transposed(v1 + mt * 32);
+      const uint4 vt = make_uint4(lo.x, lo.y, hi.x, hi.y);
 #pragma unroll
       for (int b = 0; b < 2; ++b) acc[b][mt] = Mma<E>::run(vt, pb[b], acc[b][mt]);
     }
@@ -402,7 +415,7 @@ void swa_prefill_kernel(const PrefillParams p) {
           const int64_t row = min((mc << 5) + kk, p.meta_len - 1);
           *reinterpret_cast<uint4 *>(smem + kk * kRowPad + c * 16) =
               *reinterpret_cast<const uint4 *>(p.meta_k + moff + row * p.meta_sr);
-          *reinterpret_cast<uint4 *>(smem + kStage + kk * kRowPad + c * 16) =
+          *reinterpret_cast<uint4 *>(smem + kStageK + kk * kRowPadV + c * 16) =
               *reinterpret_cast<const uint4 *>(p.meta_v + moff + row * p.meta_sr);
         }
       }
@@ -421,7 +434,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   }
   if (x < n_walk) body(x, std::integral_constant<int, 0>{});
 
-  // ---- epilogue: lane (g, c) owns token c of each block, dims 32g + 8i + mt ---------------------
+  // ---- epilogue: lane (g, c) owns token c of each block, dims 16 mt + 4g + i --------------------------
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
     float lt = l[b];
@@ -430,16 +443,11 @@ void swa_prefill_kernel(const PrefillParams p) {
     if (q0 + 16 * ts[b] + c < Lq) {
       const float inv = lt > 0.f ? 1.f / lt : 0.f;
       char *dst = p.out + ((int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.o_sr + (int64_t)(head0 + hd[b]) * p.o_sh +
-                           32 * g) * 2;
+                           4 * g) * 2;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        uint4 o;
-        o.x = E::pack(acc[b][0][i] * inv, acc[b][1][i] * inv);
-        o.y = E::pack(acc[b][2][i] * inv, acc[b][3][i] * inv);
-        o.z = E::pack(acc[b][4][i] * inv, acc[b][5][i] * inv);
-        o.w = E::pack(acc[b][6][i] * inv, acc[b][7][i] * inv);
-        *reinterpret_cast<uint4 *>(dst + 16 * i) = o;
-      }
+      for (int mt = 0; mt < 8; ++mt)
+        *reinterpret_cast<uint2 *>(dst + 32 * mt) = make_uint2(E::pack(acc[b][mt][0] * inv, acc[b][mt][1] * inv),
+                                                               E::pack(acc[b][mt][2] * inv, acc[b][mt][3] * inv));
       if (p.lse && g == 0)
         p.lse[(int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.Hq + head0 + hd[b]] =
             lt > 0.f ? (m[b] + log2f(lt)) * kLn2 : kNegInf;
@@ -533,9 +541,9 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   }
 
   const dim3 grid((unsigned)((a->num_tiles + 7) / 8 * 8), (unsigned)a->num_kv_heads);
-  for (int h0 = 0; h0 < p.G; h0 += 4) {  // a GQA group is covered 4 heads at a time
+  for (int h0 = 0; h0 < p.G; h0 += SB_PREFILL_HEADS) {  // a GQA group is covered SB_PREFILL_HEADS heads at a time
     p.head_begin = h0;
-    const int nh = p.G - h0 < 4 ? p.G - h0 : 4;
+    const int nh = p.G - h0 < SB_PREFILL_HEADS ? p.G - h0 : SB_PREFILL_HEADS;
     if (a->dtype == SB_BF16) launch_prefill<BF16>(a->kv_quant, nh, grid, (hipStream_t)a->stream, p);
     else launch_prefill<F16>(a->kv_quant, nh, grid, (hipStream_t)a->stream, p);
     const int rc = check_launch("swa_prefill_kernel");
