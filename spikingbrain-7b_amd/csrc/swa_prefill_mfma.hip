@@ -70,6 +70,11 @@ struct PrefillParams {
   int64_t meta_sr, meta_sh;  // bytes
 };
 
+#ifdef SB_PREFILL_FENCES
+#define SB_FENCE __builtin_amdgcn_sched_barrier(0)
+#else
+#define SB_FENCE
+#endif
 #ifndef SB_PREFILL_HEADS
 #define SB_PREFILL_HEADS 4
 #endif
@@ -96,7 +101,7 @@ template <int NHEADS>
 struct Shape {
   static constexpr int kPairs = NHEADS / 2;
   static constexpr int kWaves = 4 * kPairs + 2 * (NHEADS % 2);
-  static constexpr int kFetchWaves = kWaves < 4 ? kWaves : 4;   // wavefronts that move K/V into LDS
+  static constexpr int kFetchWaves = kWaves == 8 ? 8 : (kWaves < 4 ? kWaves : 4);   // wavefronts that move K/V into LDS
   static constexpr int kLoads = 8 / kFetchWaves;                // 4-row loads per fetching lane, per K and per V
 };
 
@@ -136,7 +141,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * Shape<NHEADS>::kWaves
                           amdgpu_waves_per_eu(2, 2)))
 void swa_prefill_kernel(const PrefillParams p) {
   using S = Shape<NHEADS>;
-  __shared__ __attribute__((aligned(16))) char smem[2 * kStage];  // [buffer][K|V]
+  __shared__ __attribute__((aligned(16))) char smem[3 * kStage];  // ring of three chunks, each [K|V]
 
   // Workgroups are handed to the 8 XCDs round-robin by index, and each XCD has its own L2. Give XCD x
   // the x-th contiguous eighth of the tiles, so that the workgroups resident on one XCD at a time are
@@ -216,7 +221,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   const int64_t dense_row0 = (!paged && p.kv_start) ? p.kv_start[seq] : 0;
   const int64_t head_off = (int64_t)kvh * p.kv_sh;
   int64_t scale_base = 0;  // INT8: index of the tile's first row in the scale tensors (set by tile_base)
-  auto tile_base = [&](int t) -> int64_t {  // t inside [first_tile, last_tile], wave-uniform
+  auto tile_base = [&](int t) __attribute__((always_inline)) -> int64_t {  // t inside [first_tile, last_tile], wave-uniform
     const int i0 = t << 4;
     if (paged) {
       const int bi = i0 / p.block_size;
@@ -235,7 +240,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the 16-key tile, +4 per load
   using Set = StageSet<KVQ, S::kLoads>;
   Set stage[2];  // walk index x travels in set x & 1
-  auto fetch = [&](int x, Set &st) {
+  auto fetch = [&](int x, Set &st) __attribute__((always_inline)) {
     if constexpr (KVQ == SB_KV_NONE) {
       if (x < nm) {  // meta chunk: dense rows shared by every sequence, clamped to the last one
         const int64_t moff = (int64_t)kvh * p.meta_sh + c * 16;
@@ -271,8 +276,8 @@ void swa_prefill_kernel(const PrefillParams p) {
       }
     }
   };
-  auto stash = [&](int buf, const Set &st) {
-    char *sk = smem + buf * kStage, *sv = sk + kStageK;
+  auto stash = [&](int slot, const Set &st) __attribute__((always_inline)) {  // slot = byte offset of a ring slot
+    char *sk = smem + slot, *sv = sk + kStageK;
 #pragma unroll
     for (int u = 0; u < S::kLoads; ++u) {
       const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
@@ -292,84 +297,131 @@ void swa_prefill_kernel(const PrefillParams p) {
     }
   };
 
-  float sc[2][8];  // scores of the chunk in flight (raw dot products; -inf where masked)
+  float sc[2][8];  // scores of the chunk whose softmax comes next (raw dot products; -inf where masked)
   float mx[2];     // their row maxima, in log2 units
+  uint4 pb[2];     // probabilities of the chunk whose P V product comes next
 
-  // scores of chunk `ch` for both column blocks; true when some row needs a higher reference point
-  auto scores = [&](bool is_meta, int ch, int buf) -> bool {
-    const char *sk = smem + buf * kStage;
-    uint4 k0[4], k1[4];
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      k0[s] = *reinterpret_cast<const uint4 *>(sk + c * kRowPad + (4 * s + g) * 16);
-      k1[s] = *reinterpret_cast<const uint4 *>(sk + (16 + c) * kRowPad + (4 * s + g) * 16);
+  // The two halves of an iteration. Each runs 16 matrix instructions and, BETWEEN them in issue order, the
+  // vector work of another chunk that does not depend on them, so that a wavefront keeps both pipes busy by
+  // itself (the two wavefronts of a SIMD run in step, from barrier to barrier, and do not fill each other's
+  // gaps). sched_barrier pins that order.
+  //
+  // first half: S^T = K Q^T of walk index xn (kNext; K from ring slot `slot`) into `sn`, interleaved with the
+  // numerators of the chunk in `sc` against the current reference points (kCur) -> pb, l.
+  auto first_half = [&](int slot, float (&sn)[2][8], auto next_tag, auto cur_tag) __attribute__((always_inline)) {
+    constexpr bool kNext = decltype(next_tag)::value, kCur = decltype(cur_tag)::value;
+    const char *sk0 = smem + slot + c * kRowPad + g * 16, *sk1 = sk0 + 16 * kRowPad;
+    uint4 k0[4], k1[4];  // operand loads run one step ahead of their use (two pairs live)
+    if constexpr (kNext) {
+      k0[0] = *reinterpret_cast<const uint4 *>(sk0);
+      k1[0] = *reinterpret_cast<const uint4 *>(sk1);
     }
-    const int c0 = ch << 5;
-    // wholly visible to all tokens of the wavefront: above every lower bound, at or below the first token
-    // (a meta chunk: every row that exists is visible to every token)
-    const bool full = is_meta ? c0 + 32 <= p.meta_len
-                              : (wl < 0 || c0 >= shift + jw_last - wl) && c0 >= klo && (c0 + 31 <= shift + jw0);
-    bool raise = false;
+    f32x4_t s0[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, s1[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    float m_safe[2], psum[2] = {0.f, 0.f};
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < 2; ++b) m_safe[b] = (m[b] == kNegInf) ? 0.f : m[b];
+    SB_FENCE;
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        s0 = Mma<E>::run(k0[s], qb[b][s], s0);
-        s1 = Mma<E>::run(k1[s], qb[b][s], s1);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        sc[b][j] = s0[j];
-        sc[b][4 + j] = s1[j];
-      }
-      if (!full) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int i = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-          if (is_meta ? i >= p.meta_len : (i > my_pos[b] || i < my_lo[b])) sc[b][j] = kNegInf;
+    for (int i = 0; i < 16; ++i) {
+      if constexpr (kNext) {  // four chains (block, tile), each four instructions deep, taken in turn
+        const int s = i >> 2, b = (i >> 1) & 1;
+        if ((i & 3) == 0 && s + 1 < 4) {
+          k0[s + 1] = *reinterpret_cast<const uint4 *>(sk0 + (s + 1) * 64);
+          k1[s + 1] = *reinterpret_cast<const uint4 *>(sk1 + (s + 1) * 64);
         }
+        if (i & 1) s1[b] = Mma<E>::run(k1[s], qb[b][s], s1[b]);
+        else s0[b] = Mma<E>::run(k0[s], qb[b][s], s0[b]);
       }
-      // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
-      const float t = fmaxf(fmaxf(fmaxf(sc[b][0], sc[b][1]), fmaxf(sc[b][2], sc[b][3])),
-                            fmaxf(fmaxf(sc[b][4], sc[b][5]), fmaxf(sc[b][6], sc[b][7])));
-      mx[b] = t * p.scale_log2;
-      raise |= mx[b] > m[b] + kRaise;  // also true for the first finite score of a row (m = -inf)
+      if constexpr (kCur) {
+        const int b = i >> 3, j = i & 7;
+        sc[b][j] = fast_exp2(fmaf(sc[b][j], p.scale_log2, -m_safe[b]));
+        psum[b] += sc[b][j];
+      }
+      SB_FENCE;
+    }
+    if constexpr (kCur) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        l[b] += psum[b];
+        pb[b] = make_uint4(Mma<E>::pack(sc[b][0], sc[b][1]), Mma<E>::pack(sc[b][2], sc[b][3]),
+                           Mma<E>::pack(sc[b][4], sc[b][5]), Mma<E>::pack(sc[b][6], sc[b][7]));
+      }
+    }
+    if constexpr (kNext) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          sn[b][j] = s0[b][j];
+          sn[b][4 + j] = s1[b][j];
+        }
+    }
+  };
+
+  // second half: O^T += V^T P^T (kPV; V from ring slot `slot`, probabilities pb), interleaved with the row
+  // maxima of the (masked) scores `sn` of the next chunk (kPost), which become `sc`. True when some row of
+  // that chunk needs a higher reference point.
+  auto second_half = [&](int slot, const float (&sn)[2][8], auto pv_tag, auto post_tag) __attribute__((always_inline)) -> bool {
+    constexpr bool kPV = decltype(pv_tag)::value, kPost = decltype(post_tag)::value;
+    // V^T operand of dims 16 mt + c: this lane's 8 keys (4g .. 4g+3 of either 16-key tile, the order of its
+    // probabilities) by two transposing loads, one step ahead of their use; built once, used by both blocks
+    const char *v0 = smem + slot + kStageK + (4 * g + (c >> 2)) * kRowPadV + (c & 3) * 8, *v1 = v0 + 16 * kRowPadV;
+    uint2 vlo[8], vhi[8];
+    if constexpr (kPV) {
+      vlo[0] = load_transposed(v0);
+      vhi[0] = load_transposed(v1);
+    }
+    float t[2] = {kNegInf, kNegInf};
+    SB_FENCE;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if constexpr (kPV) {
+        const int mt = i >> 1, b = i & 1;
+        if (b == 0 && mt + 1 < 8) {
+          vlo[mt + 1] = load_transposed(v0 + (mt + 1) * 32);
+          vhi[mt + 1] = load_transposed(v1 + (mt + 1) * 32);
+        }
+        acc[b][mt] = Mma<E>::run(make_uint4(vlo[mt].x, vlo[mt].y, vhi[mt].x, vhi[mt].y), pb[b], acc[b][mt]);
+      }
+      if constexpr (kPost) {
+        const int b = i >> 3, j = i & 7;
+        sc[b][j] = sn[b][j];
+        t[b] = fmaxf(t[b], sn[b][j]);  // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
+      }
+      SB_FENCE;
+    }
+    bool raise = false;
+    if constexpr (kPost) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        mx[b] = t[b] * p.scale_log2;
+        raise |= mx[b] > m[b] + kRaise;  // also true for the first finite score of a row (m = -inf)
+      }
     }
     return __builtin_amdgcn_ballot_w64(raise) != 0;
   };
-
-  // numerators against the current reference points, then O^T += V^T P^T
-  auto accumulate = [&](int buf) {
-    const char *sv = smem + buf * kStage + kStageK;
-    uint4 pb[2];
+  // Masking of the scores of walk index xn, in place. Most chunks are wholly visible to all tokens of the
+  // wavefront (above every lower bound, at or below the first token; a meta chunk: every row that exists is
+  // visible to every token) and skip it; the others pay for it outside the interleaved code.
+  auto mask_scores = [&](int xn, float (&sn)[2][8]) __attribute__((always_inline)) {
+    const bool is_meta = xn < nm;
+    const int c0 = (is_meta ? xn : ch_begin + xn - nm) << 5;
+    const bool full = is_meta ? c0 + 32 <= p.meta_len
+                              : (wl < 0 || c0 >= shift + jw_last - wl) && c0 >= klo && (c0 + 31 <= shift + jw0);
+    if (full) return;
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      const float m_safe = (m[b] == kNegInf) ? 0.f : m[b];
-      float psum = 0.f;
+    for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        sc[b][j] = fast_exp2(fmaf(sc[b][j], p.scale_log2, -m_safe));
-        psum += sc[b][j];
+        const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+        if (is_meta ? key >= p.meta_len : (key > my_pos[b] || key < my_lo[b])) sn[b][j] = kNegInf;
       }
-      l[b] += psum;
-      pb[b] = make_uint4(Mma<E>::pack(sc[b][0], sc[b][1]), Mma<E>::pack(sc[b][2], sc[b][3]),
-                         Mma<E>::pack(sc[b][4], sc[b][5]), Mma<E>::pack(sc[b][6], sc[b][7]));
-    }
-    // V^T operand of dims 16 mt + c: this lane's 8 keys (4g .. 4g+3 of either 16-key tile, the order of its
-    // probabilities) by two transposing loads; built once, used by both blocks
-    const char *v0 = sv + (4 * g + (c >> 2)) * kRowPadV + (c & 3) * 8, *v1 = v0 + 16 * kRowPadV;
-#pragma unroll
-    for (int mt = 0; mt < 8; ++mt) {
-      const uint2 lo = load_transposed(v0 + mt * 32), hi = load_transposed(v1 + mt * 32);
-      const uint4 vt = make_uint4(lo.x, lo.y, hi.x, hi.y);
-#pragma unroll
-      for (int b = 0; b < 2; ++b) acc[b][mt] = Mma<E>::run(vt, pb[b], acc[b][mt]);
-    }
   };
+  const std::true_type kYes{};
+  const std::false_type kNo{};
 
   // lift the reference points to the running maxima and rescale what has been accumulated
-  auto rescale = [&]() {
+  auto rescale = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       float t = mx[b];  // row maximum over the four lanes that share a token
@@ -387,24 +439,33 @@ void swa_prefill_kernel(const PrefillParams p) {
 
   // ---- chunk loop: one barrier per chunk, every wavefront visits every chunk -------------------
   // (chunks outside a wavefront's own band come out fully masked and add zero)
-  // Global loads run TWO chunks ahead of the arithmetic, in two register sets used alternately; the
-  // loop is written out for both sets so that every register index is static. Loads are issued
-  // unconditionally (past the end they re-read the last rows), so the wait in front of each LDS store
-  // counts exactly the loads that may still be in flight.
-  auto body = [&](int x, auto par) {
-    constexpr int P = decltype(par)::value;
-    if (fetcher) fetch(x + 2, stage[P]);
-    if (scores(x < nm, x < nm ? x : ch_begin + x - nm, P)) rescale();
-    accumulate(P);
-    if (fetcher) stash(P ^ 1, stage[P ^ 1]);
+  // Iteration x: scores of chunk x+1 while the numerators of chunk x are formed, then P V of chunk x while the
+  // scores of chunk x+1 are masked and searched for their maxima; chunk x+2 goes from registers into the ring
+  // slot that chunk x-1 has left, and chunk x+3 is requested from global memory into the registers chunk x+1
+  // has left (two register sets used alternately; the loop is written out for both so that every register
+  // index is static). Loads are issued unconditionally (past the end they re-read the last rows), so the wait
+  // in front of each LDS store counts exactly the loads that may still be in flight.
+  int r0 = 0, r1 = kStage, r2 = 2 * kStage;  // ring slots of chunks x, x+1, x+2
+  float sn[2][8];
+  auto body = [&](int x, auto par) __attribute__((always_inline)) {
+    constexpr int P = decltype(par)::value;  // chunk y travels in register set y & 1
+    if (fetcher) fetch(x + 3, stage[P ^ 1]);
+    first_half(r1, sn, kYes, kYes);
+    mask_scores(x + 1, sn);
+    if (second_half(r0, sn, kYes, kYes)) rescale();
+    if (fetcher) stash(r2, stage[P]);
     __syncthreads();
+    const int t = r0;
+    r0 = r1;
+    r1 = r2;
+    r2 = t;
   };
   if (fetcher) {
     fetch(0, stage[0]);
     fetch(1, stage[1]);
   }
   if constexpr (KVQ != SB_KV_NONE) {
-    // meta rows over a byte-code cache: global -> LDS buffer 0 -> scores, one chunk at a time, while the
+    // meta rows over a byte-code cache: global -> ring slot 0 -> scores, one chunk at a time, while the
     // first two chunks of codes are on their way
     for (int mc = 0; mc < meta_chunks; ++mc) {
       if (fetcher) {
@@ -420,19 +481,53 @@ void swa_prefill_kernel(const PrefillParams p) {
         }
       }
       __syncthreads();
-      if (scores(true, mc, 0)) rescale();
-      accumulate(0);
+      // (a meta chunk of its own: walk index -1 - mc never collides with the window's; masked by meta_len)
+      first_half(0, sn, kYes, kNo);
+      {
+        const int c0 = mc << 5;
+        float t[2] = {kNegInf, kNegInf};
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+            sc[b][j] = key >= p.meta_len ? kNegInf : sn[b][j];
+            t[b] = fmaxf(t[b], sc[b][j]);
+          }
+        bool raise = false;
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          mx[b] = t[b] * p.scale_log2;
+          raise |= mx[b] > m[b] + kRaise;
+        }
+        if (__builtin_amdgcn_ballot_w64(raise) != 0) rescale();
+      }
+      first_half(0, sn, kNo, kYes);
+      second_half(0, sn, kYes, kNo);
       __syncthreads();
     }
   }
-  if (fetcher) stash(0, stage[0]);
+  if (fetcher) {
+    stash(r0, stage[0]);
+    fetch(2, stage[0]);
+    stash(r1, stage[1]);
+  }
   __syncthreads();
+  first_half(r0, sn, kYes, kNo);
+  mask_scores(0, sn);
+  if (second_half(r0, sn, kNo, kYes)) rescale();
   int x = 0;
-  for (; x + 1 < n_walk; x += 2) {
+  for (; x + 2 < n_walk; x += 2) {
     body(x, std::integral_constant<int, 0>{});
     body(x + 1, std::integral_constant<int, 1>{});
   }
-  if (x < n_walk) body(x, std::integral_constant<int, 0>{});
+  if (x + 1 < n_walk) {
+    body(x, std::integral_constant<int, 0>{});
+    ++x;
+  }
+  // the last chunk: its numerators and its P V product
+  first_half(r1, sn, kNo, kYes);
+  second_half(r0, sn, kYes, kNo);
 
   // ---- epilogue: lane (g, c) owns token c of each block, dims 16 mt + 4g + i --------------------------
 #pragma unroll
