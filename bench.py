@@ -467,13 +467,13 @@ def main():
         attend(c, 0, profile_events=events, **kw)
 
     n_split = args.n_split or sb._native.lib().sb_swa_decode_auto_split(prob["B"], HKV, prob["max_seq_len"], WL)
-    # ONE timed region: the split kernel of every 8th step carries a pair of HIP events on its own dispatch,
+    # ONE timed region: the split kernel of every 16th step carries a pair of HIP events on its own dispatch,
     # on the stream it is launched on (torch's current stream), so the kernel time and the step time come
     # from the same K steps. Not every step: a launch that carries events delays the launch behind it by about
     # 6 us on this runtime (94.4 against 88.0 us per step with events on all of them), which would be charged
     # to `value`; the kernel's own interval is not affected.
     timed = not args.force_valu
-    EVERY = 8
+    EVERY = 16
     evs = [sb.ops.timing_events(dev) for _ in range((args.steps + EVERY - 1) // EVERY)] if timed else []
     for i in range(args.warmup):
         step(i, evs[0] if timed and i % EVERY == 0 else None)
