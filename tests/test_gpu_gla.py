@@ -267,15 +267,19 @@ def test_block_form_on_matrix_cores_vs_oracle(sb, dev, state_dtype, T):
         assert out_close(o.float().cpu().numpy(), ref_o), vector_only
 
 
+@pytest.mark.parametrize("strength", [1.5, 3.2])
 @pytest.mark.parametrize("gdtype", [torch.float32, torch.bfloat16, torch.float16])
-def test_block_form_strong_gates_and_gate_dtypes(sb, dev, gdtype):
+def test_block_form_strong_gates_and_gate_dtypes(sb, dev, gdtype, strength):
     """Gates down to -1.5 per step (exp(-B) reaches e^24 inside a block) and every gate dtype; the
-    layout is token-major with a fused q|k|v projection, as the layers produce it."""
+    layout is token-major with a fused q|k|v projection, as the layers produce it. strength 3.2: gates
+    uniform in (-3.2, 0), 1.6 per step on average: the kernel applies the decay of the state every second
+    block and carries the log-decay of the block in between in the operands' exponents, which then reach
+    e^50 to e^75 (the guard clamps at e^80; beyond it results would be wrong, not just imprecise)."""
     B, H, T, D = 1, 2, 70, 128
     g = torch.Generator().manual_seed(5)
     fused = torch.randn(B, T, H, 3 * D, generator=g).bfloat16()
     q, k, v = (fused[..., i * D:(i + 1) * D].transpose(1, 2) for i in range(3))
-    gate = (-1.5 * torch.rand(B, T, H, D, generator=g)).to(gdtype).transpose(1, 2)
+    gate = (-strength * torch.rand(B, T, H, D, generator=g)).to(gdtype).transpose(1, 2)
     ref_o, ref_S = G.gla_recurrent(q.float().numpy(), k.float().numpy(), v.float().numpy(), gate.float().numpy(), None)
     fd = fused.to(dev)
     qd, kd, vd = (fd[..., i * D:(i + 1) * D].transpose(1, 2) for i in range(3))
