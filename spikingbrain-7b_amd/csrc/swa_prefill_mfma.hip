@@ -58,6 +58,7 @@ struct PrefillParams {
   int Hq;
   int num_tiles;
   int block_size, window_left;
+  int bs_shift;               // log2(block_size) when it is a power of two, else -1
   float scale_log2;
   int64_t q_sr, q_sh, o_sr, o_sh;  // elements
   int64_t kv_sb, kv_sr, kv_sh;     // bytes
@@ -224,7 +225,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   auto tile_base = [&](int t) __attribute__((always_inline)) -> int64_t {  // t inside [first_tile, last_tile], wave-uniform
     const int i0 = t << 4;
     if (paged) {
-      const int bi = i0 / p.block_size;
+      const int bi = p.bs_shift >= 0 ? i0 >> p.bs_shift : i0 / p.block_size;
       const int64_t blk = p.block_table[(int64_t)seq * p.bt_stride + bi];
       if constexpr (KVQ == SB_KV_INT8) scale_base = (blk * p.Hkv + kvh) * p.block_size + (i0 - bi * p.block_size);
       return blk * p.kv_sb + (int64_t)(i0 - bi * p.block_size) * p.kv_sr + head_off;
@@ -409,13 +410,22 @@ void swa_prefill_kernel(const PrefillParams p) {
     const bool full = is_meta ? c0 + 32 <= p.meta_len
                               : (wl < 0 || c0 >= shift + jw_last - wl) && c0 >= klo && (c0 + 31 <= shift + jw0);
     if (full) return;
+    // (selects, not branches: the comparison results are combined as bits)
+    if (is_meta) {
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+      for (int b = 0; b < 2; ++b)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-        if (is_meta ? key >= p.meta_len : (key > my_pos[b] || key < my_lo[b])) sn[b][j] = kNegInf;
-      }
+        for (int j = 0; j < 8; ++j)
+          sn[b][j] = (c0 + ((j >> 2) << 4) + 4 * g + (j & 3) >= p.meta_len) ? kNegInf : sn[b][j];
+    } else {
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+          sn[b][j] = bool((key > my_pos[b]) | (key < my_lo[b])) ? kNegInf : sn[b][j];
+        }
+    }
   };
   const std::true_type kYes{};
   const std::false_type kNo{};
@@ -614,6 +624,7 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   p.cu_q = a->cu_seqlens_q; p.seq_lens_k = a->seq_lens_k; p.tile_seq = a->tile_seq; p.tile_q0 = a->tile_q0;
   p.G = a->num_q_heads / a->num_kv_heads; p.head_begin = 0;
   p.block_size = a->block_size > 0 ? a->block_size : 16; p.window_left = a->window_left;
+  p.bs_shift = (p.block_size & (p.block_size - 1)) == 0 ? __builtin_ctz((unsigned)p.block_size) : -1;
   p.scale_log2 = a->scale * sb::kLog2e;
   p.q_sr = a->q_stride_row; p.q_sh = a->q_stride_head; p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
   p.kv_sb = a->kv_stride_block * kv_esz; p.kv_sr = a->kv_stride_row * kv_esz; p.kv_sh = a->kv_stride_head * kv_esz;
