@@ -41,23 +41,57 @@ def compute_slot_mapping_start_idx(is_prompt: bool, query_len: int, context_len:
     return start_idx
 
 
-def compute_slot_mapping(is_profile_run: bool, slot_mapping: List[int], seq_id, seq_len: int, context_len: int,
+class SlotBuffer:
+    """A step's slot mapping while it is being built: behaves like the reference's `slot_mapping: List[int]`
+    for what the builder does with it (`extend`, `len`), but keeps what compute_slot_mapping produces as
+    numpy pieces, so that a prompt step of 10^5 tokens never becomes 10^5 Python ints."""
+
+    def __init__(self):
+        self._parts: List[np.ndarray] = []
+        self._n = 0
+
+    def extend(self, values) -> None:
+        a = values if isinstance(values, np.ndarray) else np.asarray(list(values), dtype=np.int64)
+        if a.size:
+            self._parts.append(a.astype(np.int64, copy=False))
+            self._n += int(a.size)
+
+    def __len__(self) -> int:
+        return self._n
+
+    def array(self) -> np.ndarray:
+        if not self._parts:
+            return np.zeros(0, dtype=np.int64)
+        return self._parts[0] if len(self._parts) == 1 else np.concatenate(self._parts)
+
+    def tolist(self) -> List[int]:
+        return self.array().tolist()
+
+
+def compute_slot_mapping(is_profile_run: bool, slot_mapping, seq_id, seq_len: int, context_len: int,
                          start_idx: int, block_size: int, block_tables) -> None:
     """Append one slot per new token i in [context_len, seq_len) (call site meta_attention.py:492-494):
     PAD_SLOT_ID below start_idx, else block_tables[seq_id][i // block_size] * block_size + i % block_size.
     `block_tables[seq_id]` must be indexable by ABSOLUTE logical block (a list, or the
-    `LogicalTable` view of this module)."""
+    `LogicalTable` view of this module). `slot_mapping` is a list (as in the reference) or a SlotBuffer."""
+    fast = isinstance(slot_mapping, SlotBuffer)
     if is_profile_run:
-        slot_mapping.extend([PAD_SLOT_ID] * seq_len)
+        slot_mapping.extend(np.full(seq_len, PAD_SLOT_ID, np.int64) if fast else [PAD_SLOT_ID] * seq_len)
         return
-    slot_mapping.extend([PAD_SLOT_ID] * max(0, start_idx - context_len))
+    n_pad = max(0, start_idx - context_len)
+    if n_pad:
+        slot_mapping.extend(np.full(n_pad, PAD_SLOT_ID, np.int64) if fast else [PAD_SLOT_ID] * n_pad)
     table = block_tables[seq_id]
     first = max(start_idx, context_len)
     if seq_len > first:
         pos = np.arange(first, seq_len, dtype=np.int64)
-        blocks = np.asarray([table[j] for j in range(first // block_size, (seq_len - 1) // block_size + 1)],
-                            dtype=np.int64)
-        slot_mapping.extend((blocks[pos // block_size - first // block_size] * block_size + pos % block_size).tolist())
+        jb, je = first // block_size, (seq_len - 1) // block_size
+        if hasattr(table, "blocks"):
+            blocks = table.blocks(jb, je)
+        else:
+            blocks = np.asarray([table[j] for j in range(jb, je + 1)], dtype=np.int64)
+        slots = blocks[pos // block_size - jb] * block_size + pos % block_size
+        slot_mapping.extend(slots if fast else slots.tolist())
 
 
 class LogicalTable:
@@ -71,6 +105,13 @@ class LogicalTable:
         if j < m.lo[r] or j > m.hi[r]:
             raise IndexError(f"logical block {j} is not resident (resident {m.lo[r]}..{m.hi[r]})")
         return int(m.ring[r, j % m.ring_blocks])
+
+    def blocks(self, jb: int, je: int) -> np.ndarray:
+        """Physical blocks of logical blocks jb..je (all of them must be resident) as int64."""
+        m, r = self._mgr, self._row
+        if jb < m.lo[r] or je > m.hi[r]:
+            raise IndexError(f"logical blocks {jb}..{je} are not all resident (resident {m.lo[r]}..{m.hi[r]})")
+        return m.ring[r, np.arange(jb, je + 1) % m.ring_blocks].astype(np.int64)
 
 
 class WindowBlockManager:
@@ -140,8 +181,10 @@ class WindowBlockManager:
         p0 = int(self.n_tokens[r])
         lo_new = max(0, (p0 - wl) // bs)
         lo, hi = int(self.lo[r]), int(self.hi[r])
-        for j in range(lo, min(lo_new, hi + 1)):
-            self._push(int(self.ring[r, j % R]))
+        n_evict = min(lo_new, hi + 1) - lo
+        if n_evict > 0:  # pushed in order of logical block, as one slice
+            self._stack[self._top:self._top + n_evict] = self.ring[r, np.arange(lo, lo + n_evict) % R]
+            self._top += n_evict
         if hi >= lo:
             lo = max(lo, lo_new)
             if lo > hi:  # everything evicted
@@ -155,19 +198,28 @@ class WindowBlockManager:
                 lo, hi = jb, jb - 1
             if je - lo + 1 > R:
                 raise RuntimeError(f"{je - lo + 1} resident blocks exceed the ring of {R}; raise max_chunk_tokens")
-            for j in range(max(jb, hi + 1), je + 1):
-                self.ring[r, j % R] = self._pop()
+            j0 = max(jb, hi + 1)
+            n_new = je + 1 - j0
+            if n_new > 0:  # popped one after the other from the top of the stack, as one reversed slice
+                if n_new > self._top:
+                    raise RuntimeError("out of KV cache blocks")
+                self.ring[r, np.arange(j0, je + 1) % R] = self._stack[self._top - n_new:self._top][::-1]
+                self._top -= n_new
             hi = max(hi, je)
         self.lo[r], self.hi[r] = lo, hi
         self.n_tokens[r] = end
         return p0, first
 
-    def append_tokens(self, seq_id, count: int, is_prompt: bool, store_all: bool = False) -> List[int]:
+    def append_tokens(self, seq_id, count: int, is_prompt: bool, store_all: bool = False,
+                      want_slots: bool = True) -> List[int]:
         """Slots of `count` new tokens of one sequence (one prompt chunk or one decode token).
-        store_all=True keeps every prompt token (chunked prefill through the paged cache)."""
+        store_all=True keeps every prompt token (chunked prefill through the paged cache).
+        want_slots=False only advances the sequence (the caller works the slots out from the tables)."""
         r = self._rows[seq_id]
         p0, first = self._advance_row(r, count, is_prompt, store_all)
         slots: List[int] = []
+        if not want_slots:
+            return slots
         compute_slot_mapping(False, slots, r, p0 + count, p0, first, self.block_size, {r: LogicalTable(self, r)})
         return slots
 

@@ -16,7 +16,7 @@ from typing import Any, Dict, List, Optional, Tuple, Type
 import torch
 
 from . import ops
-from .block_manager import PAD_SLOT_ID, compute_slot_mapping, compute_slot_mapping_start_idx
+from .block_manager import PAD_SLOT_ID, SlotBuffer, compute_slot_mapping, compute_slot_mapping_start_idx
 
 
 class AttentionType:
@@ -266,7 +266,7 @@ class MetaAttentionMetadataBuilder:
         self.block_size = input_builder.block_size
 
     def prepare(self):
-        self.slot_mapping: List[int] = []
+        self.slot_mapping = SlotBuffer()   # the reference's List[int], kept as numpy pieces
         self.prefill_seq_lens: List[int] = []
         self.context_lens: List[int] = []
         self.block_tables: List[List[int]] = []
@@ -353,6 +353,9 @@ class MetaAttentionMetadataBuilder:
         pin = bool(getattr(self.runner, "pin_memory", False)) and torch.device(device).type == "cuda"
 
         def h2d(data, dtype):
+            if isinstance(data, SlotBuffer):
+                t = torch.from_numpy(data.array()).to(dtype)
+                return (t.pin_memory() if pin else t).to(device, non_blocking=True)
             return torch.tensor(data, dtype=dtype, pin_memory=pin).to(device, non_blocking=True)
 
         return MetaAttentionMetadata(

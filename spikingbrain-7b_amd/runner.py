@@ -10,6 +10,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from .block_manager import LogicalTable, WindowBlockManager
@@ -47,7 +48,7 @@ class ResidentTable(LogicalTable):
             if j.stop is not None or j.step is not None or j.start is None or j.start >= 0:
                 raise IndexError("only t[-n:] slices are supported")
             first = max(lo, hi + 1 + j.start)
-            return [int(m.ring[r, b % m.ring_blocks]) for b in range(first, hi + 1)]
+            return m.ring[r, np.arange(first, hi + 1) % m.ring_blocks].tolist()
         return super().__getitem__(j)
 
 
@@ -108,7 +109,7 @@ class SwaCacheRunner:
         for sid, n_new in prompts:
             r = mgr.row_of(sid)
             ctx = int(mgr.n_tokens[r])
-            mgr.append_tokens(sid, n_new, True, store_all=chunked_prefill)
+            mgr.append_tokens(sid, n_new, True, store_all=chunked_prefill, want_slots=False)
             total = ctx + n_new
             first = int(mgr.lo[r]) * bs if mgr.hi[r] >= mgr.lo[r] else 0
             paged = chunked_prefill
@@ -125,7 +126,7 @@ class SwaCacheRunner:
             mgr.decode_step([sid for sid, _ in decodes])
         else:
             for sid, n in decodes:      # same policy, one sequence after the other in batch-row order
-                mgr.append_tokens(sid, n, False)
+                mgr.append_tokens(sid, n, False, want_slots=False)
         for sid, n in decodes:
             r = mgr.row_of(sid)
             total = int(mgr.n_tokens[r])
