@@ -135,6 +135,36 @@ def test_product_slot_mapping_functions_match(sb):
     assert a == [-1] * 5
 
 
+def test_slot_buffer_path_matches_list_path(sb):
+    """The builder's SlotBuffer (numpy pieces, vectorised table lookups through LogicalTable.blocks) gives the
+    slots of the list path and of the oracle, sequence after sequence into one buffer; a lookup outside the
+    resident range raises as the per-block path does."""
+    from spikingbrain_7b_amd.block_manager import LogicalTable, SlotBuffer
+    rng = np.random.default_rng(0)
+    bs, wl = 16, 64
+    mgr = sb.WindowBlockManager(512, bs, wl, max_seqs=4, max_chunk_tokens=400)
+    buf, ref = SlotBuffer(), []
+    for s in range(4):
+        mgr.add_seq(s)
+        n = int(rng.integers(1, 390))
+        mgr.append_tokens(s, n, True, store_all=bool(s & 1), want_slots=False)
+        r = mgr.row_of(s)
+        start = P.compute_slot_mapping_start_idx(True, n, 0, None if s & 1 else wl)
+        view = LogicalTable(mgr, r)
+        sb.compute_slot_mapping(False, buf, r, n, 0, start, bs, {r: view})
+        as_list = {r: {j: view[j] for j in range(int(mgr.lo[r]), int(mgr.hi[r]) + 1)}}
+        P.compute_slot_mapping(False, ref, r, n, 0, start, bs, as_list)
+        assert len(buf) == len(ref)
+    assert buf.tolist() == ref and buf.array().dtype == np.int64
+    buf.extend([-1] * 3)
+    assert buf.tolist() == ref + [-1] * 3
+    with pytest.raises(IndexError):
+        LogicalTable(mgr, 0).blocks(int(mgr.hi[0]), int(mgr.hi[0]) + 1)
+    empty = SlotBuffer()
+    sb.compute_slot_mapping(True, empty, 0, 4, 0, 0, bs, None)
+    assert empty.tolist() == [-1] * 4 and SlotBuffer().array().shape == (0,)
+
+
 def test_block_manager_errors(sb):
     with pytest.raises(ValueError, match="multiple of 16"):
         sb.WindowBlockManager(8, 24, 32, max_seqs=1)
