@@ -10,13 +10,16 @@
 //   (a wider GQA group takes several launches, 7 = 4 + 3). Every wavefront owns two "column blocks" of
 //   16 tokens x 1 head (32 score columns, no padding): a pair of heads is served by 4 wavefronts (one
 //   per 16-token sub-tile), an odd last head by 2 wavefronts (two sub-tiles each) - 8 wavefronts for 4
-//   heads, 6 for 3. At 256 registers per wavefront two of them share a SIMD, so one wavefront's
-//   softmax arithmetic overlaps the other's matrix instructions and LDS waits.
+//   heads, 6 for 3. At 256 registers per wavefront two of them share a SIMD.
 //   The workgroup walks the union of its tokens' windows in chunks of 32 keys. Each chunk of K and V
-//   (32 rows x 256 B each) is fetched from global memory ONCE per workgroup (the first four wavefronts
-//   fetch 8 rows each with whole-row 16-byte lanes) into a double-buffered LDS stage whose rows are
-//   padded to 272 B (K) and 288 B (V); all wavefronts then read their MFMA operands from LDS. Global loads run two chunks
-//   ahead of the arithmetic (two register sets used alternately, the loop written out for both).
+//   (32 rows x 256 B each) is fetched from global memory ONCE per workgroup (every wavefront of an
+//   8-wavefront workgroup fetches 4 rows with whole-row 16-byte lanes, else the first four fetch 8) into a
+//   ring of three LDS chunks whose rows are padded to 272 B (K) and 288 B (V); all wavefronts then read
+//   their MFMA operands from LDS. Global loads run three chunks ahead of the arithmetic (two register sets
+//   used alternately, the loop written out for both). The arithmetic is staggered over two chunks: an
+//   iteration issues the scores of chunk x+1 ahead of the numerators of chunk x, and the P V product of
+//   chunk x ahead of the masking and maxima of chunk x+1, so that a wavefront's matrix instructions have
+//   vector work of another chunk behind them.
 //   Per chunk and column block: S^T = K Q^T (8 MFMA 16x16x32, tokens on the N axis), softmax numerators
 //   per lane for token lane%16 in log2 units, O^T += V^T P^T (8 MFMA). P stays in the lane that produced
 //   it; V^T operands come out of the [key][dim] stage through the transposing LDS load, shared by the two
