@@ -61,7 +61,8 @@ struct PrefillParams {
   int Hq;
   int num_tiles;
   int block_size, window_left;
-  int bs_shift;               // log2(block_size) when it is a power of two, else -1
+  int tiles_per_block;        // block_size / 16
+  uint32_t tpb_magic;         // ceil(2^31 / tiles_per_block): tile -> block by one multiplication
   float scale_log2;
   int64_t q_sr, q_sh, o_sr, o_sh;  // elements
   int64_t kv_sb, kv_sr, kv_sh;     // bytes
@@ -140,7 +141,7 @@ __device__ __forceinline__ uint4 dequant8(uint2 w, float s) {
                     Mma<E>::pack(code_value<Q, 2>(w.y) * s, code_value<Q, 3>(w.y) * s));
 }
 
-template <typename E, int NHEADS, int KVQ>
+template <typename E, int NHEADS, int KVQ, bool PAGED>
 __global__ __attribute__((amdgpu_flat_work_group_size(64 * Shape<NHEADS>::kWaves, 64 * Shape<NHEADS>::kWaves),
                           amdgpu_waves_per_eu(2, 2)))
 void swa_prefill_kernel(const PrefillParams p) {
@@ -176,12 +177,8 @@ void swa_prefill_kernel(const PrefillParams p) {
   const int wg_lo = min(max(wl >= 0 ? shift + q0 - wl : 0, klo), wg_hi - 1);
   const int first_tile = wg_lo >> 4, last_tile = (wg_hi - 1) >> 4;
   const int ch_begin = wg_lo >> 5, ch_end = ((wg_hi - 1) >> 5) + 1;
-  // The walk: the meta rows' chunks first (walk index x < nm), then window chunk ch_begin + x - nm.
-  // (Over a byte-code cache the meta rows, which are elements, do not fit the registers a chunk of codes
-  // travels in: there they are taken in a loop of their own in front of the walk.)
+  const int n_walk = ch_end - ch_begin;  // the walk: index x is window chunk ch_begin + x
   const int meta_chunks = (p.meta_len + 31) >> 5;
-  const int nm = KVQ == SB_KV_NONE ? meta_chunks : 0;
-  const int n_walk = nm + ch_end - ch_begin;
 
   // this wavefront's two column blocks: 16-token sub-tile ts[b] of head hd[b]
   int ts[2], hd[2];
@@ -210,6 +207,11 @@ void swa_prefill_kernel(const PrefillParams p) {
       qb[b][s] = *reinterpret_cast<const uint4 *>(
           p.q + ((int64_t)(qrow0 + j_mine) * p.q_sr + (int64_t)(head0 + hd[b]) * p.q_sh + (4 * s + g) * 8) * 2);
   }
+  // Chunks wholly visible to every token of the wavefront (at or above every token's lower bound, at or below
+  // the first token) need no masking: walk indices [full_lo, full_lo + full_cnt).
+  const int vis_lo = max(wl >= 0 ? shift + jw_last - wl : 0, klo);
+  const int full_lo = ((vis_lo + 31) >> 5) - ch_begin;
+  const unsigned full_cnt = (unsigned)max(((shift + jw0 + 1) >> 5) - ch_begin - full_lo, 0);
 
   f32x4_t acc[2][8];
   float m[2], l[2];  // m: reference point of the numerators (log2 units), l: this lane's share of the sum
@@ -221,70 +223,74 @@ void swa_prefill_kernel(const PrefillParams p) {
     for (int mt = 0; mt < 8; ++mt) acc[b][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  const bool paged = p.block_table != nullptr;
-  const int64_t dense_row0 = (!paged && p.kv_start) ? p.kv_start[seq] : 0;
-  const int64_t head_off = (int64_t)kvh * p.kv_sh;
-  int64_t scale_base = 0;  // INT8: index of the tile's first row in the scale tensors (set by tile_base)
-  auto tile_base = [&](int t) __attribute__((always_inline)) -> int64_t {  // t inside [first_tile, last_tile], wave-uniform
-    const int i0 = t << 4;
-    if (paged) {
-      const int bi = p.bs_shift >= 0 ? i0 >> p.bs_shift : i0 / p.block_size;
-      const int64_t blk = p.block_table[(int64_t)seq * p.bt_stride + bi];
-      if constexpr (KVQ == SB_KV_INT8) scale_base = (blk * p.Hkv + kvh) * p.block_size + (i0 - bi * p.block_size);
-      return blk * p.kv_sb + (int64_t)(i0 - bi * p.block_size) * p.kv_sr + head_off;
-    }
-    return (dense_row0 + i0) * p.kv_sr + head_off;
-  };
-
   // ---- global -> registers -> LDS: the first kFetchWaves wavefronts move the chunk (32 K rows and
   // 32 V rows of 256 B); each of their loads covers 4 rows, all inside one 16-key tile of the table.
-  // rows outside [wg_lo, wg_hi) are clamped onto the nearest visible key (masked for every token)
-  const bool fetcher = wave < S::kFetchWaves;
-  const int rows_per_wave = 32 / S::kFetchWaves;                         // 8 or 16
-  const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the 16-key tile, +4 per load
+  // Rows outside [wg_lo, wg_hi) are clamped onto the nearest visible key (masked for every token).
+  // Everything that does not depend on the lane is kept in scalar registers: per chunk, the tile's byte offset
+  // (one block-table entry, looked up one call ahead of its use) added to the K and V bases; a lane adds its
+  // row and column as a 32-bit offset.
+  constexpr int kFetchAll = S::kFetchWaves == S::kWaves;
+  const bool fetcher = kFetchAll || wave < S::kFetchWaves;
+  constexpr int rows_per_wave = 32 / S::kFetchWaves;                     // 4, 8 or 16
+  const int tsel = (wave * rows_per_wave) >> 4;                          // which 16-key tile of a chunk this wavefront's rows are in
+  const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the tile, +4 per load
+  const uint32_t row_bytes = (uint32_t)p.kv_sr;                          // < 2^24 (host check)
+  const uint32_t lane_col = c * (KVQ == SB_KV_NONE ? 16 : 8);
+  const int64_t wg_off = (int64_t)kvh * p.kv_sh + ((!PAGED && p.kv_start) ? p.kv_start[seq] * p.kv_sr : 0);
+  const char *const kbase = p.k + wg_off, *const vbase = p.v + wg_off;
+  const int32_t *const table_row = PAGED ? p.block_table + (int64_t)seq * p.bt_stride : nullptr;
+  auto walk_tile = [&](int x) __attribute__((always_inline)) {  // (past the end of the walk: the last tile again)
+    return min(max(2 * (ch_begin + x) + tsel, first_tile), last_tile);
+  };
+  // block of 16-key tile t: t / tiles_per_block by multiplication (exact while t < 2^31 / tiles_per_block)
+  auto block_of = [&](int t) __attribute__((always_inline)) { return (int)__umulhi((uint32_t)t << 1, p.tpb_magic); };
+  int next_blk = 0;  // table entry of the tile the next fetch takes
+  if constexpr (PAGED) next_blk = table_row[block_of(walk_tile(0))];
+  int fx = 0;        // walk index the next fetch takes
   using Set = StageSet<KVQ, S::kLoads>;
   Set stage[2];  // walk index x travels in set x & 1
-  auto fetch = [&](int x, Set &st) __attribute__((always_inline)) {
-    if constexpr (KVQ == SB_KV_NONE) {
-      if (x < nm) {  // meta chunk: dense rows shared by every sequence, clamped to the last one
-        const int64_t moff = (int64_t)kvh * p.meta_sh + c * 16;
-#pragma unroll
-        for (int u = 0; u < S::kLoads; ++u) {
-          const int row = min((x << 5) + wave * rows_per_wave + (lane >> 4) + 4 * u, p.meta_len - 1);
-          st.k[u] = *reinterpret_cast<const uint4 *>(p.meta_k + moff + (int64_t)row * p.meta_sr);
-          st.v[u] = *reinterpret_cast<const uint4 *>(p.meta_v + moff + (int64_t)row * p.meta_sr);
-        }
-        return;
-      }
+  auto fetch = [&](Set &st) __attribute__((always_inline)) {
+    const int t = walk_tile(fx);
+    ++fx;
+    int64_t off;  // of the tile's first row from kbase / vbase
+    [[maybe_unused]] int64_t scale_row = 0;  // INT8: index of that row in the scale tensors
+    if constexpr (PAGED) {
+      const int bi = block_of(t);
+      const int64_t blk = next_blk;
+      next_blk = table_row[block_of(walk_tile(fx))];
+      const int in_block = (t - bi * p.tiles_per_block) << 4;
+      off = blk * p.kv_sb + (int64_t)((uint32_t)in_block * row_bytes);
+      if constexpr (KVQ == SB_KV_INT8) scale_row = (blk * p.Hkv + kvh) * p.block_size + in_block;
+    } else {
+      off = (int64_t)(t << 4) * p.kv_sr;
     }
-    const int ch = ch_begin + x - nm;
-    const int t = min(max(2 * ch + (wave * rows_per_wave) / 16, first_tile), last_tile);
-    const int64_t base = tile_base(t);
+    const char *const kp = kbase + off, *const vp = vbase + off;
+    const int lo = wg_lo - (t << 4), hi = wg_hi - 1 - (t << 4);
 #pragma unroll
     for (int u = 0; u < S::kLoads; ++u) {
-      const int row = min(max((t << 4) + lrow + 4 * u, wg_lo), wg_hi - 1) - (t << 4);
+      const int row = min(max(lrow + 4 * u, lo), hi);  // inside the tile: 0 .. 15
+      const uint32_t vo = __umul24((uint32_t)row, row_bytes) + lane_col;
       if constexpr (KVQ == SB_KV_NONE) {
-        const int64_t off = base + (int64_t)row * p.kv_sr + c * 16;
-        st.k[u] = load_stream16(p.k + off);
-        st.v[u] = load_stream16(p.v + off);
+        st.k[u] = load_stream16(kp + vo);
+        st.v[u] = load_stream16(vp + vo);
       } else {  // a row is 128 code bytes: 8 per lane
-        const int64_t off = base + (int64_t)row * p.kv_sr + c * 8;
-        const unsigned long long wk = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(p.k + off));
-        const unsigned long long wv = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(p.v + off));
+        const unsigned long long wk = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(kp + vo));
+        const unsigned long long wv = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(vp + vo));
         st.k[u] = make_uint2((uint32_t)wk, (uint32_t)(wk >> 32));
         st.v[u] = make_uint2((uint32_t)wv, (uint32_t)(wv >> 32));
         if constexpr (KVQ == SB_KV_INT8) {
-          st.ks[u] = p.k_scale[scale_base + row];
-          st.vs[u] = p.v_scale[scale_base + row];
+          st.ks[u] = (p.k_scale + scale_row)[(uint32_t)row];
+          st.vs[u] = (p.v_scale + scale_row)[(uint32_t)row];
         }
       }
     }
   };
+  const int stash_off = (wave * rows_per_wave + (lane >> 4)) * kRowPad + c * 16;   // of this lane's first row in a K chunk;
+  const int stash_off_v = (wave * rows_per_wave + (lane >> 4)) * kRowPadV + c * 16 + kStageK;  // in the V chunk behind it
   auto stash = [&](int slot, const Set &st) __attribute__((always_inline)) {  // slot = byte offset of a ring slot
-    char *sk = smem + slot, *sv = sk + kStageK;
+    char *sk = smem + slot + stash_off, *sv = smem + slot + stash_off_v;
 #pragma unroll
     for (int u = 0; u < S::kLoads; ++u) {
-      const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
       uint4 kq, vq;
       if constexpr (KVQ == SB_KV_NONE) {
         kq = st.k[u];
@@ -296,35 +302,37 @@ void swa_prefill_kernel(const PrefillParams p) {
         kq = dequant8<E, KVQ>(st.k[u], p.k_scale_tensor);
         vq = dequant8<E, KVQ>(st.v[u], p.v_scale_tensor);
       }
-      *reinterpret_cast<uint4 *>(sk + kk * kRowPad + c * 16) = kq;
-      *reinterpret_cast<uint4 *>(sv + kk * kRowPadV + c * 16) = vq;
+      *reinterpret_cast<uint4 *>(sk + 4 * u * kRowPad) = kq;
+      *reinterpret_cast<uint4 *>(sv + 4 * u * kRowPadV) = vq;
     }
   };
 
-  float sc[2][8];  // scores of the chunk whose softmax comes next (raw dot products; -inf where masked)
-  float mx[2];     // their row maxima, in log2 units
+  // Scores live in two register sets used alternately: while the numerators of one chunk are formed in one set,
+  // the matrix instructions write the next chunk's scores into the other. s[b][t][i]: block b, key 16 t + 4 g + i
+  // of the chunk (raw dot products; -inf where masked).
+  using Scores = f32x4_t[2][2];
+  Scores sa, sb2;
+  float mx[2];     // row maxima of the scores whose softmax comes next, in log2 units
   uint4 pb[2];     // probabilities of the chunk whose P V product comes next
 
-  // The two halves of an iteration. Each runs 16 matrix instructions and, BETWEEN them in issue order, the
-  // vector work of another chunk that does not depend on them, so that a wavefront keeps both pipes busy by
-  // itself (the two wavefronts of a SIMD run in step, from barrier to barrier, and do not fill each other's
-  // gaps). sched_barrier pins that order.
+  // The two halves of an iteration. Each runs 16 matrix instructions next to the vector work of another chunk
+  // that does not depend on them.
   //
-  // first half: S^T = K Q^T of walk index xn (kNext; K from ring slot `slot`) into `sn`, interleaved with the
+  // first half: S^T = K Q^T of the next chunk (kNext; K from ring slot `slot`) into `sn`, next to the
   // numerators of the chunk in `sc` against the current reference points (kCur) -> pb, l.
-  auto first_half = [&](int slot, float (&sn)[2][8], auto next_tag, auto cur_tag) __attribute__((always_inline)) {
+  auto first_half = [&](int slot, Scores &sn, Scores &sc, auto next_tag, auto cur_tag) __attribute__((always_inline)) {
     constexpr bool kNext = decltype(next_tag)::value, kCur = decltype(cur_tag)::value;
     const char *sk0 = smem + slot + c * kRowPad + g * 16, *sk1 = sk0 + 16 * kRowPad;
     uint4 k0[4], k1[4];  // operand loads run one step ahead of their use (two pairs live)
     if constexpr (kNext) {
       k0[0] = *reinterpret_cast<const uint4 *>(sk0);
       k1[0] = *reinterpret_cast<const uint4 *>(sk1);
+#pragma unroll
+      for (int b = 0; b < 2; ++b) sn[b][0] = sn[b][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
-    f32x4_t s0[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, s1[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     float m_safe[2], psum[2] = {0.f, 0.f};
 #pragma unroll
     for (int b = 0; b < 2; ++b) m_safe[b] = (m[b] == kNegInf) ? 0.f : m[b];
-    SB_FENCE;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       if constexpr (kNext) {  // four chains (block, tile), each four instructions deep, taken in turn
@@ -333,66 +341,52 @@ void swa_prefill_kernel(const PrefillParams p) {
           k0[s + 1] = *reinterpret_cast<const uint4 *>(sk0 + (s + 1) * 64);
           k1[s + 1] = *reinterpret_cast<const uint4 *>(sk1 + (s + 1) * 64);
         }
-        if (i & 1) s1[b] = Mma<E>::run(k1[s], qb[b][s], s1[b]);
-        else s0[b] = Mma<E>::run(k0[s], qb[b][s], s0[b]);
+        sn[b][i & 1] = Mma<E>::run((i & 1) ? k1[s] : k0[s], qb[b][s], sn[b][i & 1]);
       }
       if constexpr (kCur) {
         const int b = i >> 3, j = i & 7;
-        sc[b][j] = fast_exp2(fmaf(sc[b][j], p.scale_log2, -m_safe[b]));
-        psum[b] += sc[b][j];
+        const float e = fast_exp2(fmaf(sc[b][j >> 2][j & 3], p.scale_log2, -m_safe[b]));
+        sc[b][j >> 2][j & 3] = e;
+        psum[b] += e;
       }
-      SB_FENCE;
     }
     if constexpr (kCur) {
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
         l[b] += psum[b];
-        pb[b] = make_uint4(Mma<E>::pack(sc[b][0], sc[b][1]), Mma<E>::pack(sc[b][2], sc[b][3]),
-                           Mma<E>::pack(sc[b][4], sc[b][5]), Mma<E>::pack(sc[b][6], sc[b][7]));
+        pb[b] = make_uint4(Mma<E>::pack(sc[b][0][0], sc[b][0][1]), Mma<E>::pack(sc[b][0][2], sc[b][0][3]),
+                           Mma<E>::pack(sc[b][1][0], sc[b][1][1]), Mma<E>::pack(sc[b][1][2], sc[b][1][3]));
       }
-    }
-    if constexpr (kNext) {
-#pragma unroll
-      for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          sn[b][j] = s0[b][j];
-          sn[b][4 + j] = s1[b][j];
-        }
     }
   };
 
-  // second half: O^T += V^T P^T (kPV; V from ring slot `slot`, probabilities pb), interleaved with the row
-  // maxima of the (masked) scores `sn` of the next chunk (kPost), which become `sc`. True when some row of
-  // that chunk needs a higher reference point.
-  auto second_half = [&](int slot, const float (&sn)[2][8], auto pv_tag, auto post_tag) __attribute__((always_inline)) -> bool {
-    constexpr bool kPV = decltype(pv_tag)::value, kPost = decltype(post_tag)::value;
-    // V^T operand of dims 16 mt + c: this lane's 8 keys (4g .. 4g+3 of either 16-key tile, the order of its
-    // probabilities) by two transposing loads, one step ahead of their use; built once, used by both blocks
+  // second half: O^T += V^T P^T (kPV; probabilities pb), next to the row maxima of the (masked) scores `sn` of
+  // the next chunk (kPost). True when some row of that chunk needs a higher reference point.
+  // V^T operands of a chunk, dims 16 mt + c: this lane's 8 keys (4g .. 4g+3 of either 16-key tile, the order of
+  // its probabilities) by two transposing loads per mt; built once, used by both blocks. They are requested at
+  // the top of an iteration and arrive while the first half runs.
+  uint2 vlo[8], vhi[8];
+  auto load_v = [&](int slot) __attribute__((always_inline)) {
     const char *v0 = smem + slot + kStageK + (4 * g + (c >> 2)) * kRowPadV + (c & 3) * 8, *v1 = v0 + 16 * kRowPadV;
-    uint2 vlo[8], vhi[8];
-    if constexpr (kPV) {
-      vlo[0] = load_transposed(v0);
-      vhi[0] = load_transposed(v1);
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) {
+      vlo[mt] = load_transposed(v0 + mt * 32);
+      vhi[mt] = load_transposed(v1 + mt * 32);
     }
+  };
+  auto second_half = [&](const Scores &sn, auto pv_tag, auto post_tag) __attribute__((always_inline)) -> bool {
+    constexpr bool kPV = decltype(pv_tag)::value, kPost = decltype(post_tag)::value;
     float t[2] = {kNegInf, kNegInf};
-    SB_FENCE;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       if constexpr (kPV) {
         const int mt = i >> 1, b = i & 1;
-        if (b == 0 && mt + 1 < 8) {
-          vlo[mt + 1] = load_transposed(v0 + (mt + 1) * 32);
-          vhi[mt + 1] = load_transposed(v1 + (mt + 1) * 32);
-        }
         acc[b][mt] = Mma<E>::run(make_uint4(vlo[mt].x, vlo[mt].y, vhi[mt].x, vhi[mt].y), pb[b], acc[b][mt]);
       }
-      if constexpr (kPost) {
+      if constexpr (kPost) {  // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
         const int b = i >> 3, j = i & 7;
-        sc[b][j] = sn[b][j];
-        t[b] = fmaxf(t[b], sn[b][j]);  // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
+        t[b] = fmaxf(t[b], sn[b][j >> 2][j & 3]);
       }
-      SB_FENCE;
     }
     bool raise = false;
     if constexpr (kPost) {
@@ -404,31 +398,18 @@ void swa_prefill_kernel(const PrefillParams p) {
     }
     return __builtin_amdgcn_ballot_w64(raise) != 0;
   };
-  // Masking of the scores of walk index xn, in place. Most chunks are wholly visible to all tokens of the
-  // wavefront (above every lower bound, at or below the first token; a meta chunk: every row that exists is
-  // visible to every token) and skip it; the others pay for it outside the interleaved code.
-  auto mask_scores = [&](int xn, float (&sn)[2][8]) __attribute__((always_inline)) {
-    const bool is_meta = xn < nm;
-    const int c0 = (is_meta ? xn : ch_begin + xn - nm) << 5;
-    const bool full = is_meta ? c0 + 32 <= p.meta_len
-                              : (wl < 0 || c0 >= shift + jw_last - wl) && c0 >= klo && (c0 + 31 <= shift + jw0);
-    if (full) return;
-    // (selects, not branches: the comparison results are combined as bits)
-    if (is_meta) {
+  // Masking of the scores of walk index xn, in place (selects, not branches: the comparison results are
+  // combined as bits). Skipped for the chunks every token of the wavefront sees whole.
+  auto mask_scores = [&](int xn, Scores &sn) __attribute__((always_inline)) {
+    if ((unsigned)(xn - full_lo) < full_cnt) return;
+    const int c0 = (ch_begin + xn) << 5;
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < 2; ++b)
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          sn[b][j] = (c0 + ((j >> 2) << 4) + 4 * g + (j & 3) >= p.meta_len) ? kNegInf : sn[b][j];
-    } else {
-#pragma unroll
-      for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-          sn[b][j] = bool((key > my_pos[b]) | (key < my_lo[b])) ? kNegInf : sn[b][j];
-        }
-    }
+      for (int j = 0; j < 8; ++j) {
+        const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+        sn[b][j >> 2][j & 3] = bool((key > my_pos[b]) | (key < my_lo[b])) ? kNegInf : sn[b][j >> 2][j & 3];
+      }
   };
   const std::true_type kYes{};
   const std::false_type kNo{};
@@ -450,97 +431,114 @@ void swa_prefill_kernel(const PrefillParams p) {
     }
   };
 
+  if (fetcher) {
+    fetch(stage[0]);
+    fetch(stage[1]);
+  }
+  // ---- meta rows: global -> ring slot 0 -> scores, one chunk at a time, while the first two chunks of the
+  // window are on their way (every row that exists is visible to every token)
+  for (int mc = 0; mc < meta_chunks; ++mc) {
+    if (fetcher) {
+      const char *mk = p.meta_k + (int64_t)kvh * p.meta_sh + c * 16, *mv = p.meta_v + (int64_t)kvh * p.meta_sh + c * 16;
+#pragma unroll
+      for (int u = 0; u < S::kLoads; ++u) {
+        const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
+        const int64_t row = min((mc << 5) + kk, p.meta_len - 1);
+        *reinterpret_cast<uint4 *>(smem + kk * kRowPad + c * 16) = *reinterpret_cast<const uint4 *>(mk + row * p.meta_sr);
+        *reinterpret_cast<uint4 *>(smem + kStageK + kk * kRowPadV + c * 16) =
+            *reinterpret_cast<const uint4 *>(mv + row * p.meta_sr);
+      }
+    }
+    __syncthreads();
+    first_half(0, sa, sa, kYes, kNo);
+    {
+      const int c0 = mc << 5;
+      float t[2] = {kNegInf, kNegInf};
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+          sa[b][j >> 2][j & 3] = key >= p.meta_len ? kNegInf : sa[b][j >> 2][j & 3];
+          t[b] = fmaxf(t[b], sa[b][j >> 2][j & 3]);
+        }
+      bool raise = false;
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        mx[b] = t[b] * p.scale_log2;
+        raise |= mx[b] > m[b] + kRaise;
+      }
+      if (__builtin_amdgcn_ballot_w64(raise) != 0) rescale();
+    }
+    first_half(0, sa, sa, kNo, kYes);
+    load_v(0);
+    second_half(sa, kYes, kNo);
+    __syncthreads();
+  }
+
   // ---- chunk loop: one barrier per chunk, every wavefront visits every chunk -------------------
   // (chunks outside a wavefront's own band come out fully masked and add zero)
   // Iteration x: scores of chunk x+1 while the numerators of chunk x are formed, then P V of chunk x while the
   // scores of chunk x+1 are masked and searched for their maxima; chunk x+2 goes from registers into the ring
   // slot that chunk x-1 has left, and chunk x+3 is requested from global memory into the registers chunk x+1
-  // has left (two register sets used alternately; the loop is written out for both so that every register
-  // index is static). Loads are issued unconditionally (past the end they re-read the last rows), so the wait
-  // in front of each LDS store counts exactly the loads that may still be in flight.
+  // has left (two register sets and two score sets used alternately; the loop is written out for both so that
+  // every register index is static). Loads are issued unconditionally (past the end they re-read the last
+  // rows), so the wait in front of each LDS store counts exactly the loads that may still be in flight.
   int r0 = 0, r1 = kStage, r2 = 2 * kStage;  // ring slots of chunks x, x+1, x+2
-  float sn[2][8];
-  auto body = [&](int x, auto par) __attribute__((always_inline)) {
-    constexpr int P = decltype(par)::value;  // chunk y travels in register set y & 1
-    if (fetcher) fetch(x + 3, stage[P ^ 1]);
-    first_half(r1, sn, kYes, kYes);
+#ifdef SB_PREFILL_TIMING
+  long long tsum[6] = {0, 0, 0, 0, 0, 0};
+#define SB_TICK(i) { const long long now = __builtin_readcyclecounter(); tsum[i] += now - tprev; tprev = now; }
+#else
+#define SB_TICK(i)
+#endif
+  auto body = [&](int x, Scores &sc, Scores &sn, Set &arriving, Set &leaving) __attribute__((always_inline)) {
+#ifdef SB_PREFILL_TIMING
+    long long tprev = __builtin_readcyclecounter();
+#endif
+    load_v(r0);
+    if (fetcher) fetch(arriving);  // chunk x + 3
+    SB_TICK(0)
+    first_half(r1, sn, sc, kYes, kYes);
+    SB_TICK(1)
     mask_scores(x + 1, sn);
-    if (second_half(r0, sn, kYes, kYes)) rescale();
-    if (fetcher) stash(r2, stage[P]);
+    SB_TICK(2)
+    if (second_half(sn, kYes, kYes)) rescale();
+    SB_TICK(3)
+    if (fetcher) stash(r2, leaving);  // chunk x + 2
+    SB_TICK(4)
     __syncthreads();
+    SB_TICK(5)
     const int t = r0;
     r0 = r1;
     r1 = r2;
     r2 = t;
   };
   if (fetcher) {
-    fetch(0, stage[0]);
-    fetch(1, stage[1]);
-  }
-  if constexpr (KVQ != SB_KV_NONE) {
-    // meta rows over a byte-code cache: global -> ring slot 0 -> scores, one chunk at a time, while the
-    // first two chunks of codes are on their way
-    for (int mc = 0; mc < meta_chunks; ++mc) {
-      if (fetcher) {
-        const int64_t moff = (int64_t)kvh * p.meta_sh + c * 16;
-#pragma unroll
-        for (int u = 0; u < S::kLoads; ++u) {
-          const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
-          const int64_t row = min((mc << 5) + kk, p.meta_len - 1);
-          *reinterpret_cast<uint4 *>(smem + kk * kRowPad + c * 16) =
-              *reinterpret_cast<const uint4 *>(p.meta_k + moff + row * p.meta_sr);
-          *reinterpret_cast<uint4 *>(smem + kStageK + kk * kRowPadV + c * 16) =
-              *reinterpret_cast<const uint4 *>(p.meta_v + moff + row * p.meta_sr);
-        }
-      }
-      __syncthreads();
-      // (a meta chunk of its own: walk index -1 - mc never collides with the window's; masked by meta_len)
-      first_half(0, sn, kYes, kNo);
-      {
-        const int c0 = mc << 5;
-        float t[2] = {kNegInf, kNegInf};
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-            sc[b][j] = key >= p.meta_len ? kNegInf : sn[b][j];
-            t[b] = fmaxf(t[b], sc[b][j]);
-          }
-        bool raise = false;
-#pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          mx[b] = t[b] * p.scale_log2;
-          raise |= mx[b] > m[b] + kRaise;
-        }
-        if (__builtin_amdgcn_ballot_w64(raise) != 0) rescale();
-      }
-      first_half(0, sn, kNo, kYes);
-      second_half(0, sn, kYes, kNo);
-      __syncthreads();
-    }
-  }
-  if (fetcher) {
     stash(r0, stage[0]);
-    fetch(2, stage[0]);
+    fetch(stage[0]);  // chunk 2
     stash(r1, stage[1]);
   }
   __syncthreads();
-  first_half(r0, sn, kYes, kNo);
-  mask_scores(0, sn);
-  if (second_half(r0, sn, kNo, kYes)) rescale();
+  first_half(r0, sa, sa, kYes, kNo);
+  mask_scores(0, sa);
+  if (second_half(sa, kNo, kYes)) rescale();
   int x = 0;
   for (; x + 2 < n_walk; x += 2) {
-    body(x, std::integral_constant<int, 0>{});
-    body(x + 1, std::integral_constant<int, 1>{});
+    body(x, sa, sb2, stage[1], stage[0]);
+    body(x + 1, sb2, sa, stage[0], stage[1]);
   }
   if (x + 1 < n_walk) {
-    body(x, std::integral_constant<int, 0>{});
-    ++x;
+    body(x, sa, sb2, stage[1], stage[0]);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      sa[b][0] = sb2[b][0];
+      sa[b][1] = sb2[b][1];
+    }
   }
   // the last chunk: its numerators and its P V product
-  first_half(r1, sn, kNo, kYes);
-  second_half(r0, sn, kYes, kNo);
+  load_v(r0);
+  first_half(r1, sa, sa, kNo, kYes);
+  second_half(sa, kYes, kNo);
 
   // ---- epilogue: lane (g, c) owns token c of each block, dims 16 mt + 4g + i --------------------------
 #pragma unroll
@@ -556,27 +554,36 @@ void swa_prefill_kernel(const PrefillParams p) {
       for (int mt = 0; mt < 8; ++mt)
         *reinterpret_cast<uint2 *>(dst + 32 * mt) = make_uint2(E::pack(acc[b][mt][0] * inv, acc[b][mt][1] * inv),
                                                                E::pack(acc[b][mt][2] * inv, acc[b][mt][3] * inv));
+#ifndef SB_PREFILL_TIMING
       if (p.lse && g == 0)
         p.lse[(int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.Hq + head0 + hd[b]] =
             lt > 0.f ? (m[b] + log2f(lt)) * kLn2 : kNegInf;
+#endif
     }
   }
+#ifdef SB_PREFILL_TIMING
+  if (p.lse && tile == p.num_tiles / 2 + 100 && kvh == 0 && lane == 0) {
+    for (int i = 0; i < 6; ++i) p.lse[wave * 8 + i] = (float)tsum[i];
+    p.lse[wave * 8 + 6] = (float)n_walk;
+  }
+#endif
 }
 
-template <typename E, int KVQ>
+template <typename E, int KVQ, bool PAGED>
 void launch_prefill_q(int nh, dim3 grid, hipStream_t st, const PrefillParams &p) {
   switch (nh) {
-    case 1: hipLaunchKernelGGL((swa_prefill_kernel<E, 1, KVQ>), grid, dim3(64 * Shape<1>::kWaves), 0, st, p); break;
-    case 2: hipLaunchKernelGGL((swa_prefill_kernel<E, 2, KVQ>), grid, dim3(64 * Shape<2>::kWaves), 0, st, p); break;
-    case 3: hipLaunchKernelGGL((swa_prefill_kernel<E, 3, KVQ>), grid, dim3(64 * Shape<3>::kWaves), 0, st, p); break;
-    default: hipLaunchKernelGGL((swa_prefill_kernel<E, 4, KVQ>), grid, dim3(64 * Shape<4>::kWaves), 0, st, p); break;
+    case 1: hipLaunchKernelGGL((swa_prefill_kernel<E, 1, KVQ, PAGED>), grid, dim3(64 * Shape<1>::kWaves), 0, st, p); break;
+    case 2: hipLaunchKernelGGL((swa_prefill_kernel<E, 2, KVQ, PAGED>), grid, dim3(64 * Shape<2>::kWaves), 0, st, p); break;
+    case 3: hipLaunchKernelGGL((swa_prefill_kernel<E, 3, KVQ, PAGED>), grid, dim3(64 * Shape<3>::kWaves), 0, st, p); break;
+    default: hipLaunchKernelGGL((swa_prefill_kernel<E, 4, KVQ, PAGED>), grid, dim3(64 * Shape<4>::kWaves), 0, st, p); break;
   }
 }
 template <typename E>
 void launch_prefill(int kv_quant, int nh, dim3 grid, hipStream_t st, const PrefillParams &p) {
-  if (kv_quant == SB_KV_INT8) launch_prefill_q<E, SB_KV_INT8>(nh, grid, st, p);
-  else if (kv_quant == SB_KV_FP8) launch_prefill_q<E, SB_KV_FP8>(nh, grid, st, p);
-  else launch_prefill_q<E, SB_KV_NONE>(nh, grid, st, p);
+  if (kv_quant == SB_KV_INT8) launch_prefill_q<E, SB_KV_INT8, true>(nh, grid, st, p);
+  else if (kv_quant == SB_KV_FP8) launch_prefill_q<E, SB_KV_FP8, true>(nh, grid, st, p);
+  else if (p.block_table) launch_prefill_q<E, SB_KV_NONE, true>(nh, grid, st, p);
+  else launch_prefill_q<E, SB_KV_NONE, false>(nh, grid, st, p);
 }
 
 }  // namespace
@@ -616,6 +623,9 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   for (int64_t s : kes)
     if ((s * kv_esz) % 16 != 0)
       return fail(SB_ERR_INVALID, "sb_swa_prefill: cache stride %lld elements is not 16-byte aligned", (long long)s);
+  if (a->kv_stride_row <= 0 || a->kv_stride_row * kv_esz >= (1 << 24))
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: cache row stride %lld elements (must be positive and below 16 MiB)",
+                (long long)a->kv_stride_row);
   if ((reinterpret_cast<uintptr_t>(a->q) | reinterpret_cast<uintptr_t>(a->k) | reinterpret_cast<uintptr_t>(a->v) |
        reinterpret_cast<uintptr_t>(a->out)) & 15u)
     return fail(SB_ERR_INVALID, "sb_swa_prefill: q/k/v/out base not 16-byte aligned");
@@ -627,7 +637,8 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   p.cu_q = a->cu_seqlens_q; p.seq_lens_k = a->seq_lens_k; p.tile_seq = a->tile_seq; p.tile_q0 = a->tile_q0;
   p.G = a->num_q_heads / a->num_kv_heads; p.head_begin = 0;
   p.block_size = a->block_size > 0 ? a->block_size : 16; p.window_left = a->window_left;
-  p.bs_shift = (p.block_size & (p.block_size - 1)) == 0 ? __builtin_ctz((unsigned)p.block_size) : -1;
+  p.tiles_per_block = p.block_size / 16;
+  p.tpb_magic = (uint32_t)(((1ull << 31) + p.tiles_per_block - 1) / p.tiles_per_block);
   p.scale_log2 = a->scale * sb::kLog2e;
   p.q_sr = a->q_stride_row; p.q_sh = a->q_stride_head; p.o_sr = a->out_stride_row; p.o_sh = a->out_stride_head;
   p.kv_sb = a->kv_stride_block * kv_esz; p.kv_sr = a->kv_stride_row * kv_esz; p.kv_sh = a->kv_stride_head * kv_esz;

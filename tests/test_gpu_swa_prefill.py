@@ -60,7 +60,7 @@ def test_dense_context_offsets(sb, dev, wl):
     check(out, q, k, v, cu_q, cu_k, D ** -0.5, wl, 2e-2)
 
 
-@pytest.mark.parametrize("bs", [16, 32, 256])
+@pytest.mark.parametrize("bs", [16, 32, 48, 256])
 @pytest.mark.parametrize("wl", [-1, 40, 300])
 def test_paged_chunked_prefill_vs_oracle(sb, dev, bs, wl):
     """Chunked prefill: keys (context + the chunk) live in the paged cache in a shuffled block order."""
