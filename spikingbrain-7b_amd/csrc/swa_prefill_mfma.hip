@@ -80,10 +80,13 @@ struct PrefillParams {
 #else
 #define SB_FENCE
 #endif
+#ifndef SB_PREFILL_FETCH8
+#define SB_PREFILL_FETCH8 8
+#endif
 #ifndef SB_PREFILL_HEADS
 #define SB_PREFILL_HEADS 4
 #endif
-constexpr int kRowPad = 272;   // LDS row stride of a K chunk: 256 B of data + 16 B (16-byte operand loads, 16 rows at a time)
+constexpr int kRowPad = 288;   // LDS row stride of a K chunk: 256 B of data + 32 B (16-byte operand loads of 16 rows: measured 1.6 x the rate of a 272 B stride)
 constexpr int kRowPadV = 288;  // of a V chunk: 256 B + 32 B (transposing loads: 4 rows x 32 B at a time)
 constexpr int kStageK = 32 * kRowPad, kStageV = 32 * kRowPadV;
 constexpr int kStage = kStageK + kStageV;  // one chunk of K and V
@@ -106,7 +109,7 @@ template <int NHEADS>
 struct Shape {
   static constexpr int kPairs = NHEADS / 2;
   static constexpr int kWaves = 4 * kPairs + 2 * (NHEADS % 2);
-  static constexpr int kFetchWaves = kWaves == 8 ? 8 : (kWaves < 4 ? kWaves : 4);   // wavefronts that move K/V into LDS
+  static constexpr int kFetchWaves = kWaves == 8 ? SB_PREFILL_FETCH8 : (kWaves < 4 ? kWaves : 4);   // wavefronts that move K/V into LDS
   static constexpr int kLoads = 8 / kFetchWaves;                // 4-row loads per fetching lane, per K and per V
 };
 
@@ -271,11 +274,11 @@ void swa_prefill_kernel(const PrefillParams p) {
       const int row = min(max(lrow + 4 * u, lo), hi);  // inside the tile: 0 .. 15
       const uint32_t vo = __umul24((uint32_t)row, row_bytes) + lane_col;
       if constexpr (KVQ == SB_KV_NONE) {
-        st.k[u] = load_stream16(kp + vo);
-        st.v[u] = load_stream16(vp + vo);
+        st.k[u] = *reinterpret_cast<const uint4 *>(kp + vo);  // (cached: the neighbouring query tiles read the same rows)
+        st.v[u] = *reinterpret_cast<const uint4 *>(vp + vo);
       } else {  // a row is 128 code bytes: 8 per lane
-        const unsigned long long wk = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(kp + vo));
-        const unsigned long long wv = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long *>(vp + vo));
+        const unsigned long long wk = *reinterpret_cast<const unsigned long long *>(kp + vo);
+        const unsigned long long wv = *reinterpret_cast<const unsigned long long *>(vp + vo);
         st.k[u] = make_uint2((uint32_t)wk, (uint32_t)(wk >> 32));
         st.v[u] = make_uint2((uint32_t)wv, (uint32_t)(wv >> 32));
         if constexpr (KVQ == SB_KV_INT8) {
@@ -487,18 +490,28 @@ void swa_prefill_kernel(const PrefillParams p) {
   int r0 = 0, r1 = kStage, r2 = 2 * kStage;  // ring slots of chunks x, x+1, x+2
 #ifdef SB_PREFILL_TIMING
   long long tsum[6] = {0, 0, 0, 0, 0, 0};
-#define SB_TICK(i) { const long long now = __builtin_readcyclecounter(); tsum[i] += now - tprev; tprev = now; }
+  long long tabs[14] = {0};
+#define SB_TICK(i) { const long long now = __builtin_readcyclecounter(); tsum[i] += now - tprev; tprev = now; if (x == 60) tabs[1 + i] = now; if (x == 61) tabs[8 + i] = now; }
 #else
 #define SB_TICK(i)
 #endif
   auto body = [&](int x, Scores &sc, Scores &sn, Set &arriving, Set &leaving) __attribute__((always_inline)) {
 #ifdef SB_PREFILL_TIMING
     long long tprev = __builtin_readcyclecounter();
+    if (x == 60) tabs[0] = tprev;
+    if (x == 61) tabs[7] = tprev;
+#endif
+#ifdef SB_ABL_NO_VLOAD
+    if (x < 0)
 #endif
     load_v(r0);
     if (fetcher) fetch(arriving);  // chunk x + 3
     SB_TICK(0)
+#ifdef SB_ABL_NO_KLOAD
+    first_half(x < 0 ? r1 : 0, sn, sc, kYes, kYes);
+#else
     first_half(r1, sn, sc, kYes, kYes);
+#endif
     SB_TICK(1)
     mask_scores(x + 1, sn);
     SB_TICK(2)
@@ -565,6 +578,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   if (p.lse && tile == p.num_tiles / 2 + 100 && kvh == 0 && lane == 0) {
     for (int i = 0; i < 6; ++i) p.lse[wave * 8 + i] = (float)tsum[i];
     p.lse[wave * 8 + 6] = (float)n_walk;
+    for (int i = 0; i < 14; ++i) p.lse[64 + wave * 16 + i] = (float)(tabs[i] & 0xffffff);
   }
 #endif
 }
