@@ -14,12 +14,19 @@
 //   The workgroup walks the union of its tokens' windows in chunks of 32 keys. Each chunk of K and V
 //   (32 rows x 256 B each) is fetched from global memory ONCE per workgroup (every wavefront of an
 //   8-wavefront workgroup fetches 4 rows with whole-row 16-byte lanes, else the first four fetch 8) into a
-//   ring of three LDS chunks whose rows are padded to 272 B (K) and 288 B (V); all wavefronts then read
-//   their MFMA operands from LDS. Global loads run three chunks ahead of the arithmetic (two register sets
-//   used alternately, the loop written out for both). The arithmetic is staggered over two chunks: an
+//   ring of three LDS chunks whose rows are padded to 288 B; all wavefronts then read their MFMA operands
+//   from LDS. Global loads run three chunks ahead of the arithmetic (two register sets used alternately, the
+//   loop written out for both). They are ordinary cached loads: the neighbouring query tiles, which run at
+//   the same time on the same XCD, read the same rows. The arithmetic is staggered over two chunks: an
 //   iteration issues the scores of chunk x+1 ahead of the numerators of chunk x, and the P V product of
 //   chunk x ahead of the masking and maxima of chunk x+1, so that a wavefront's matrix instructions have
 //   vector work of another chunk behind them.
+//   A wavefront issues about one instruction per 5 cycles whatever its kind, and a scalar branch costs 15-25
+//   cycles, so the loop is kept short: everything that does not depend on the lane lives in scalar registers
+//   (a chunk's address is one block-table entry, read one iteration ahead, times the block stride, plus the
+//   K and V bases; a lane adds a 32-bit offset), the range of chunks that need no masking is computed once,
+//   and the rare paths (masking, raising the reference point) sit behind one branch each.
+//   Meta rows, when given, are taken in a loop of their own in front of the walk.
 //   Per chunk and column block: S^T = K Q^T (8 MFMA 16x16x32, tokens on the N axis), softmax numerators
 //   per lane for token lane%16 in log2 units, O^T += V^T P^T (8 MFMA). P stays in the lane that produced
 //   it; V^T operands come out of the [key][dim] stage through the transposing LDS load, shared by the two
@@ -75,14 +82,6 @@ struct PrefillParams {
   int64_t meta_sr, meta_sh;  // bytes
 };
 
-#ifdef SB_PREFILL_FENCES
-#define SB_FENCE __builtin_amdgcn_sched_barrier(0)
-#else
-#define SB_FENCE
-#endif
-#ifndef SB_PREFILL_FETCH8
-#define SB_PREFILL_FETCH8 8
-#endif
 #ifndef SB_PREFILL_HEADS
 #define SB_PREFILL_HEADS 4
 #endif
@@ -109,7 +108,7 @@ template <int NHEADS>
 struct Shape {
   static constexpr int kPairs = NHEADS / 2;
   static constexpr int kWaves = 4 * kPairs + 2 * (NHEADS % 2);
-  static constexpr int kFetchWaves = kWaves == 8 ? SB_PREFILL_FETCH8 : (kWaves < 4 ? kWaves : 4);   // wavefronts that move K/V into LDS
+  static constexpr int kFetchWaves = kWaves == 8 ? 8 : (kWaves < 4 ? kWaves : 4);   // wavefronts that move K/V into LDS
   static constexpr int kLoads = 8 / kFetchWaves;                // 4-row loads per fetching lane, per K and per V
 };
 
@@ -501,17 +500,10 @@ void swa_prefill_kernel(const PrefillParams p) {
     if (x == 60) tabs[0] = tprev;
     if (x == 61) tabs[7] = tprev;
 #endif
-#ifdef SB_ABL_NO_VLOAD
-    if (x < 0)
-#endif
     load_v(r0);
     if (fetcher) fetch(arriving);  // chunk x + 3
     SB_TICK(0)
-#ifdef SB_ABL_NO_KLOAD
-    first_half(x < 0 ? r1 : 0, sn, sc, kYes, kYes);
-#else
     first_half(r1, sn, sc, kYes, kYes);
-#endif
     SB_TICK(1)
     mask_scores(x + 1, sn);
     SB_TICK(2)
