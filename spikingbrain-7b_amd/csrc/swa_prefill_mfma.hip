@@ -107,7 +107,7 @@ constexpr float kRaise = 8.f;
 template <int NHEADS>
 struct Shape {
   static constexpr int kPairs = NHEADS / 2;
-  static constexpr int kWaves = 4 * kPairs + 2 * (NHEADS % 2);
+  static constexpr int kWaves = 4 * kPairs + 4 * (NHEADS % 2);
   static constexpr int kFetchWaves = kWaves == 8 ? 8 : (kWaves < 4 ? kWaves : 4);   // wavefronts that move K/V into LDS
   static constexpr int kLoads = 8 / kFetchWaves;                // 4-row loads per fetching lane, per K and per V
 };
@@ -182,25 +182,25 @@ void swa_prefill_kernel(const PrefillParams p) {
   const int n_walk = ch_end - ch_begin;  // the walk: index x is window chunk ch_begin + x
   const int meta_chunks = (p.meta_len + 31) >> 5;
 
-  // this wavefront's two column blocks: 16-token sub-tile ts[b] of head hd[b]
-  int ts[2], hd[2];
-  if (wave < 4 * S::kPairs) {
-    ts[0] = ts[1] = wave & 3;
-    hd[0] = 2 * (wave >> 2);
-    hd[1] = hd[0] + 1;
-  } else {
-    ts[0] = 2 * (wave - 4 * S::kPairs);
-    ts[1] = ts[0] + 1;
-    hd[0] = hd[1] = NHEADS - 1;
+  // Everything from here on is written for NB column blocks per wavefront: two for the wavefronts of a head
+  // pair, one for those of an odd last head (four wavefronts, one per 16-token sub-tile).
+  auto run = [&](auto nb_tag) __attribute__((always_inline)) {
+    constexpr int NB = decltype(nb_tag)::value;
+  // this wavefront's NB column blocks: 16-token sub-tile ts[b] of head hd[b]
+  int ts[NB], hd[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    ts[b] = wave & 3;
+    hd[b] = NB == 2 ? 2 * (wave >> 2) + b : NHEADS - 1;
   }
   const int head0 = kvh * p.G + p.head_begin;
   // (rows past the end of the sequence repeat its last token; they are never stored)
   const int jw0 = min(q0 + 16 * ts[0], Lq - 1);            // first and last token of the wavefront
-  const int jw_last = min(q0 + 16 * ts[1] + 15, Lq - 1);
-  int my_pos[2], my_lo[2];
-  uint4 qb[2][4];  // Q^T operands: token lane%16 of the block, dims of 16-byte piece 4s+g
+  const int jw_last = min(q0 + 16 * ts[NB - 1] + 15, Lq - 1);
+  int my_pos[NB], my_lo[NB];
+  uint4 qb[NB][4];  // Q^T operands: token lane%16 of the block, dims of 16-byte piece 4s+g
 #pragma unroll
-  for (int b = 0; b < 2; ++b) {
+  for (int b = 0; b < NB; ++b) {
     const int j_mine = min(q0 + 16 * ts[b] + c, Lq - 1);
     my_pos[b] = shift + j_mine;
     my_lo[b] = max(wl >= 0 ? my_pos[b] - wl : 0, klo);
@@ -215,10 +215,10 @@ void swa_prefill_kernel(const PrefillParams p) {
   const int full_lo = ((vis_lo + 31) >> 5) - ch_begin;
   const unsigned full_cnt = (unsigned)max(((shift + jw0 + 1) >> 5) - ch_begin - full_lo, 0);
 
-  f32x4_t acc[2][8];
-  float m[2], l[2];  // m: reference point of the numerators (log2 units), l: this lane's share of the sum
+  f32x4_t acc[NB][8];
+  float m[NB], l[NB];  // m: reference point of the numerators (log2 units), l: this lane's share of the sum
 #pragma unroll
-  for (int b = 0; b < 2; ++b) {
+  for (int b = 0; b < NB; ++b) {
     m[b] = kNegInf;
     l[b] = 0.f;
 #pragma unroll
@@ -312,10 +312,10 @@ void swa_prefill_kernel(const PrefillParams p) {
   // Scores live in two register sets used alternately: while the numerators of one chunk are formed in one set,
   // the matrix instructions write the next chunk's scores into the other. s[b][t][i]: block b, key 16 t + 4 g + i
   // of the chunk (raw dot products; -inf where masked).
-  using Scores = f32x4_t[2][2];
+  using Scores = f32x4_t[NB][2];
   Scores sa, sb2;
-  float mx[2];     // row maxima of the scores whose softmax comes next, in log2 units
-  uint4 pb[2];     // probabilities of the chunk whose P V product comes next
+  float mx[NB];    // row maxima of the scores whose softmax comes next, in log2 units
+  uint4 pb[NB];    // probabilities of the chunk whose P V product comes next
 
   // The two halves of an iteration. Each runs 16 matrix instructions next to the vector work of another chunk
   // that does not depend on them.
@@ -330,31 +330,40 @@ void swa_prefill_kernel(const PrefillParams p) {
       k0[0] = *reinterpret_cast<const uint4 *>(sk0);
       k1[0] = *reinterpret_cast<const uint4 *>(sk1);
 #pragma unroll
-      for (int b = 0; b < 2; ++b) sn[b][0] = sn[b][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int b = 0; b < NB; ++b) sn[b][0] = sn[b][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
-    float m_safe[2], psum[2] = {0.f, 0.f};
+    float m_safe[NB], psum[NB];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) m_safe[b] = (m[b] == kNegInf) ? 0.f : m[b];
+    for (int b = 0; b < NB; ++b) m_safe[b] = (m[b] == kNegInf) ? 0.f : m[b];
+    if constexpr (kNext) {  // 2 NB chains (block, tile), each four instructions deep, taken in turn
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if constexpr (kNext) {  // four chains (block, tile), each four instructions deep, taken in turn
-        const int s = i >> 2, b = (i >> 1) & 1;
-        if ((i & 3) == 0 && s + 1 < 4) {
+      for (int s = 0; s < 4; ++s) {
+        if (s + 1 < 4) {
           k0[s + 1] = *reinterpret_cast<const uint4 *>(sk0 + (s + 1) * 64);
           k1[s + 1] = *reinterpret_cast<const uint4 *>(sk1 + (s + 1) * 64);
         }
-        sn[b][i & 1] = Mma<E>::run((i & 1) ? k1[s] : k0[s], qb[b][s], sn[b][i & 1]);
-      }
-      if constexpr (kCur) {
-        const int b = i >> 3, j = i & 7;
-        const float e = fast_exp2(fmaf(sc[b][j >> 2][j & 3], p.scale_log2, -m_safe[b]));
-        sc[b][j >> 2][j & 3] = e;
-        psum[b] += e;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          sn[b][0] = Mma<E>::run(k0[s], qb[b][s], sn[b][0]);
+          sn[b][1] = Mma<E>::run(k1[s], qb[b][s], sn[b][1]);
+        }
       }
     }
     if constexpr (kCur) {
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
+      for (int b = 0; b < NB; ++b) {
+        psum[b] = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float e = fast_exp2(fmaf(sc[b][j >> 2][j & 3], p.scale_log2, -m_safe[b]));
+          sc[b][j >> 2][j & 3] = e;
+          psum[b] += e;
+        }
+      }
+    }
+    if constexpr (kCur) {
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
         l[b] += psum[b];
         pb[b] = make_uint4(Mma<E>::pack(sc[b][0][0], sc[b][0][1]), Mma<E>::pack(sc[b][0][2], sc[b][0][3]),
                            Mma<E>::pack(sc[b][1][0], sc[b][1][1]), Mma<E>::pack(sc[b][1][2], sc[b][1][3]));
@@ -378,22 +387,26 @@ void swa_prefill_kernel(const PrefillParams p) {
   };
   auto second_half = [&](const Scores &sn, auto pv_tag, auto post_tag) __attribute__((always_inline)) -> bool {
     constexpr bool kPV = decltype(pv_tag)::value, kPost = decltype(post_tag)::value;
-    float t[2] = {kNegInf, kNegInf};
+    float t[NB];
+    if constexpr (kPV) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if constexpr (kPV) {
-        const int mt = i >> 1, b = i & 1;
-        acc[b][mt] = Mma<E>::run(make_uint4(vlo[mt].x, vlo[mt].y, vhi[mt].x, vhi[mt].y), pb[b], acc[b][mt]);
-      }
-      if constexpr (kPost) {  // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
-        const int b = i >> 3, j = i & 7;
-        t[b] = fmaxf(t[b], sn[b][j >> 2][j & 3]);
+      for (int mt = 0; mt < 8; ++mt)
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+          acc[b][mt] = Mma<E>::run(make_uint4(vlo[mt].x, vlo[mt].y, vhi[mt].x, vhi[mt].y), pb[b], acc[b][mt]);
+    }
+    if constexpr (kPost) {  // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        t[b] = kNegInf;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[b] = fmaxf(t[b], sn[b][j >> 2][j & 3]);
       }
     }
     bool raise = false;
     if constexpr (kPost) {
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
+      for (int b = 0; b < NB; ++b) {
         mx[b] = t[b] * p.scale_log2;
         raise |= mx[b] > m[b] + kRaise;  // also true for the first finite score of a row (m = -inf)
       }
@@ -406,7 +419,7 @@ void swa_prefill_kernel(const PrefillParams p) {
     if ((unsigned)(xn - full_lo) < full_cnt) return;
     const int c0 = (ch_begin + xn) << 5;
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
@@ -419,7 +432,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   // lift the reference points to the running maxima and rescale what has been accumulated
   auto rescale = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
+    for (int b = 0; b < NB; ++b) {
       float t = mx[b];  // row maximum over the four lanes that share a token
       t = fmaxf(t, __shfl_xor(t, 16));
       t = fmaxf(t, __shfl_xor(t, 32));
@@ -455,18 +468,20 @@ void swa_prefill_kernel(const PrefillParams p) {
     first_half(0, sa, sa, kYes, kNo);
     {
       const int c0 = mc << 5;
-      float t[2] = {kNegInf, kNegInf};
+      float t[NB];
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
+      for (int b = 0; b < NB; ++b) {
+        t[b] = kNegInf;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
           sa[b][j >> 2][j & 3] = key >= p.meta_len ? kNegInf : sa[b][j >> 2][j & 3];
           t[b] = fmaxf(t[b], sa[b][j >> 2][j & 3]);
         }
+      }
       bool raise = false;
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
+      for (int b = 0; b < NB; ++b) {
         mx[b] = t[b] * p.scale_log2;
         raise |= mx[b] > m[b] + kRaise;
       }
@@ -535,7 +550,7 @@ void swa_prefill_kernel(const PrefillParams p) {
   if (x + 1 < n_walk) {
     body(x, sa, sb2, stage[1], stage[0]);
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
+    for (int b = 0; b < NB; ++b) {
       sa[b][0] = sb2[b][0];
       sa[b][1] = sb2[b][1];
     }
@@ -547,7 +562,7 @@ void swa_prefill_kernel(const PrefillParams p) {
 
   // ---- epilogue: lane (g, c) owns token c of each block, dims 16 mt + 4g + i --------------------------
 #pragma unroll
-  for (int b = 0; b < 2; ++b) {
+  for (int b = 0; b < NB; ++b) {
     float lt = l[b];
     lt += __shfl_xor(lt, 16);
     lt += __shfl_xor(lt, 32);
@@ -573,6 +588,13 @@ void swa_prefill_kernel(const PrefillParams p) {
     for (int i = 0; i < 14; ++i) p.lse[64 + wave * 16 + i] = (float)(tabs[i] & 0xffffff);
   }
 #endif
+  };
+  if constexpr (NHEADS % 2 == 1) {
+    if (wave >= 4 * S::kPairs) run(std::integral_constant<int, 1>{});
+    else if constexpr (NHEADS > 1) run(std::integral_constant<int, 2>{});
+  } else {
+    run(std::integral_constant<int, 2>{});
+  }
 }
 
 template <typename E, int KVQ, bool PAGED>
