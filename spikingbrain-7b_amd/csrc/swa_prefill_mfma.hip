@@ -186,408 +186,381 @@ void swa_prefill_kernel(const PrefillParams p) {
   // pair, one for those of an odd last head (four wavefronts, one per 16-token sub-tile).
   auto run = [&](auto nb_tag) __attribute__((always_inline)) {
     constexpr int NB = decltype(nb_tag)::value;
-  // this wavefront's NB column blocks: 16-token sub-tile ts[b] of head hd[b]
-  int ts[NB], hd[NB];
-#pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    ts[b] = wave & 3;
-    hd[b] = NB == 2 ? 2 * (wave >> 2) + b : NHEADS - 1;
-  }
-  const int head0 = kvh * p.G + p.head_begin;
-  // (rows past the end of the sequence repeat its last token; they are never stored)
-  const int jw0 = min(q0 + 16 * ts[0], Lq - 1);            // first and last token of the wavefront
-  const int jw_last = min(q0 + 16 * ts[NB - 1] + 15, Lq - 1);
-  int my_pos[NB], my_lo[NB];
-  uint4 qb[NB][4];  // Q^T operands: token lane%16 of the block, dims of 16-byte piece 4s+g
-#pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    const int j_mine = min(q0 + 16 * ts[b] + c, Lq - 1);
-    my_pos[b] = shift + j_mine;
-    my_lo[b] = max(wl >= 0 ? my_pos[b] - wl : 0, klo);
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-      qb[b][s] = *reinterpret_cast<const uint4 *>(
-          p.q + ((int64_t)(qrow0 + j_mine) * p.q_sr + (int64_t)(head0 + hd[b]) * p.q_sh + (4 * s + g) * 8) * 2);
-  }
-  // Chunks wholly visible to every token of the wavefront (at or above every token's lower bound, at or below
-  // the first token) need no masking: walk indices [full_lo, full_lo + full_cnt).
-  const int vis_lo = max(wl >= 0 ? shift + jw_last - wl : 0, klo);
-  const int full_lo = ((vis_lo + 31) >> 5) - ch_begin;
-  const unsigned full_cnt = (unsigned)max(((shift + jw0 + 1) >> 5) - ch_begin - full_lo, 0);
-
-  f32x4_t acc[NB][8];
-  float m[NB], l[NB];  // m: reference point of the numerators (log2 units), l: this lane's share of the sum
-#pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    m[b] = kNegInf;
-    l[b] = 0.f;
-#pragma unroll
-    for (int mt = 0; mt < 8; ++mt) acc[b][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  }
-
-  // ---- global -> registers -> LDS: the first kFetchWaves wavefronts move the chunk (32 K rows and
-  // 32 V rows of 256 B); each of their loads covers 4 rows, all inside one 16-key tile of the table.
-  // Rows outside [wg_lo, wg_hi) are clamped onto the nearest visible key (masked for every token).
-  // Everything that does not depend on the lane is kept in scalar registers: per chunk, the tile's byte offset
-  // (one block-table entry, looked up one call ahead of its use) added to the K and V bases; a lane adds its
-  // row and column as a 32-bit offset.
-  constexpr int kFetchAll = S::kFetchWaves == S::kWaves;
-  const bool fetcher = kFetchAll || wave < S::kFetchWaves;
-  constexpr int rows_per_wave = 32 / S::kFetchWaves;                     // 4, 8 or 16
-  const int tsel = (wave * rows_per_wave) >> 4;                          // which 16-key tile of a chunk this wavefront's rows are in
-  const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the tile, +4 per load
-  const uint32_t row_bytes = (uint32_t)p.kv_sr;                          // < 2^24 (host check)
-  const uint32_t lane_col = c * (KVQ == SB_KV_NONE ? 16 : 8);
-  const int64_t wg_off = (int64_t)kvh * p.kv_sh + ((!PAGED && p.kv_start) ? p.kv_start[seq] * p.kv_sr : 0);
-  const char *const kbase = p.k + wg_off, *const vbase = p.v + wg_off;
-  const int32_t *const table_row = PAGED ? p.block_table + (int64_t)seq * p.bt_stride : nullptr;
-  auto walk_tile = [&](int x) __attribute__((always_inline)) {  // (past the end of the walk: the last tile again)
-    return min(max(2 * (ch_begin + x) + tsel, first_tile), last_tile);
-  };
-  // block of 16-key tile t: t / tiles_per_block by multiplication (exact while t < 2^31 / tiles_per_block)
-  auto block_of = [&](int t) __attribute__((always_inline)) { return (int)__umulhi((uint32_t)t << 1, p.tpb_magic); };
-  int next_blk = 0;  // table entry of the tile the next fetch takes
-  if constexpr (PAGED) next_blk = table_row[block_of(walk_tile(0))];
-  int fx = 0;        // walk index the next fetch takes
-  using Set = StageSet<KVQ, S::kLoads>;
-  Set stage[2];  // walk index x travels in set x & 1
-  auto fetch = [&](Set &st) __attribute__((always_inline)) {
-    const int t = walk_tile(fx);
-    ++fx;
-    int64_t off;  // of the tile's first row from kbase / vbase
-    [[maybe_unused]] int64_t scale_row = 0;  // INT8: index of that row in the scale tensors
-    if constexpr (PAGED) {
-      const int bi = block_of(t);
-      const int64_t blk = next_blk;
-      next_blk = table_row[block_of(walk_tile(fx))];
-      const int in_block = (t - bi * p.tiles_per_block) << 4;
-      off = blk * p.kv_sb + (int64_t)((uint32_t)in_block * row_bytes);
-      if constexpr (KVQ == SB_KV_INT8) scale_row = (blk * p.Hkv + kvh) * p.block_size + in_block;
-    } else {
-      off = (int64_t)(t << 4) * p.kv_sr;
-    }
-    const char *const kp = kbase + off, *const vp = vbase + off;
-    const int lo = wg_lo - (t << 4), hi = wg_hi - 1 - (t << 4);
-#pragma unroll
-    for (int u = 0; u < S::kLoads; ++u) {
-      const int row = min(max(lrow + 4 * u, lo), hi);  // inside the tile: 0 .. 15
-      const uint32_t vo = __umul24((uint32_t)row, row_bytes) + lane_col;
-      if constexpr (KVQ == SB_KV_NONE) {
-        st.k[u] = *reinterpret_cast<const uint4 *>(kp + vo);  // (cached: the neighbouring query tiles read the same rows)
-        st.v[u] = *reinterpret_cast<const uint4 *>(vp + vo);
-      } else {  // a row is 128 code bytes: 8 per lane
-        const unsigned long long wk = *reinterpret_cast<const unsigned long long *>(kp + vo);
-        const unsigned long long wv = *reinterpret_cast<const unsigned long long *>(vp + vo);
-        st.k[u] = make_uint2((uint32_t)wk, (uint32_t)(wk >> 32));
-        st.v[u] = make_uint2((uint32_t)wv, (uint32_t)(wv >> 32));
-        if constexpr (KVQ == SB_KV_INT8) {
-          st.ks[u] = (p.k_scale + scale_row)[(uint32_t)row];
-          st.vs[u] = (p.v_scale + scale_row)[(uint32_t)row];
-        }
-      }
-    }
-  };
-  const int stash_off = (wave * rows_per_wave + (lane >> 4)) * kRowPad + c * 16;   // of this lane's first row in a K chunk;
-  const int stash_off_v = (wave * rows_per_wave + (lane >> 4)) * kRowPadV + c * 16 + kStageK;  // in the V chunk behind it
-  auto stash = [&](int slot, const Set &st) __attribute__((always_inline)) {  // slot = byte offset of a ring slot
-    char *sk = smem + slot + stash_off, *sv = smem + slot + stash_off_v;
-#pragma unroll
-    for (int u = 0; u < S::kLoads; ++u) {
-      uint4 kq, vq;
-      if constexpr (KVQ == SB_KV_NONE) {
-        kq = st.k[u];
-        vq = st.v[u];
-      } else if constexpr (KVQ == SB_KV_INT8) {
-        kq = dequant8<E, KVQ>(st.k[u], st.ks[u]);
-        vq = dequant8<E, KVQ>(st.v[u], st.vs[u]);
-      } else {
-        kq = dequant8<E, KVQ>(st.k[u], p.k_scale_tensor);
-        vq = dequant8<E, KVQ>(st.v[u], p.v_scale_tensor);
-      }
-      *reinterpret_cast<uint4 *>(sk + 4 * u * kRowPad) = kq;
-      *reinterpret_cast<uint4 *>(sv + 4 * u * kRowPadV) = vq;
-    }
-  };
-
-  // Scores live in two register sets used alternately: while the numerators of one chunk are formed in one set,
-  // the matrix instructions write the next chunk's scores into the other. s[b][t][i]: block b, key 16 t + 4 g + i
-  // of the chunk (raw dot products; -inf where masked).
-  using Scores = f32x4_t[NB][2];
-  Scores sa, sb2;
-  float mx[NB];    // row maxima of the scores whose softmax comes next, in log2 units
-  uint4 pb[NB];    // probabilities of the chunk whose P V product comes next
-
-  // The two halves of an iteration. Each runs 16 matrix instructions next to the vector work of another chunk
-  // that does not depend on them.
-  //
-  // first half: S^T = K Q^T of the next chunk (kNext; K from ring slot `slot`) into `sn`, next to the
-  // numerators of the chunk in `sc` against the current reference points (kCur) -> pb, l.
-  auto first_half = [&](int slot, Scores &sn, Scores &sc, auto next_tag, auto cur_tag) __attribute__((always_inline)) {
-    constexpr bool kNext = decltype(next_tag)::value, kCur = decltype(cur_tag)::value;
-    const char *sk0 = smem + slot + c * kRowPad + g * 16, *sk1 = sk0 + 16 * kRowPad;
-    uint4 k0[4], k1[4];  // operand loads run one step ahead of their use (two pairs live)
-    if constexpr (kNext) {
-      k0[0] = *reinterpret_cast<const uint4 *>(sk0);
-      k1[0] = *reinterpret_cast<const uint4 *>(sk1);
-#pragma unroll
-      for (int b = 0; b < NB; ++b) sn[b][0] = sn[b][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    }
-    float m_safe[NB], psum[NB];
-#pragma unroll
-    for (int b = 0; b < NB; ++b) m_safe[b] = (m[b] == kNegInf) ? 0.f : m[b];
-    if constexpr (kNext) {  // 2 NB chains (block, tile), each four instructions deep, taken in turn
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        if (s + 1 < 4) {
-          k0[s + 1] = *reinterpret_cast<const uint4 *>(sk0 + (s + 1) * 64);
-          k1[s + 1] = *reinterpret_cast<const uint4 *>(sk1 + (s + 1) * 64);
-        }
-#pragma unroll
-        for (int b = 0; b < NB; ++b) {
-          sn[b][0] = Mma<E>::run(k0[s], qb[b][s], sn[b][0]);
-          sn[b][1] = Mma<E>::run(k1[s], qb[b][s], sn[b][1]);
-        }
-      }
-    }
-    if constexpr (kCur) {
-#pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        psum[b] = 0.f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float e = fast_exp2(fmaf(sc[b][j >> 2][j & 3], p.scale_log2, -m_safe[b]));
-          sc[b][j >> 2][j & 3] = e;
-          psum[b] += e;
-        }
-      }
-    }
-    if constexpr (kCur) {
-#pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        l[b] += psum[b];
-        pb[b] = make_uint4(Mma<E>::pack(sc[b][0][0], sc[b][0][1]), Mma<E>::pack(sc[b][0][2], sc[b][0][3]),
-                           Mma<E>::pack(sc[b][1][0], sc[b][1][1]), Mma<E>::pack(sc[b][1][2], sc[b][1][3]));
-      }
-    }
-  };
-
-  // second half: O^T += V^T P^T (kPV; probabilities pb), next to the row maxima of the (masked) scores `sn` of
-  // the next chunk (kPost). True when some row of that chunk needs a higher reference point.
-  // V^T operands of a chunk, dims 16 mt + c: this lane's 8 keys (4g .. 4g+3 of either 16-key tile, the order of
-  // its probabilities) by two transposing loads per mt; built once, used by both blocks. They are requested at
-  // the top of an iteration and arrive while the first half runs.
-  uint2 vlo[8], vhi[8];
-  auto load_v = [&](int slot) __attribute__((always_inline)) {
-    const char *v0 = smem + slot + kStageK + (4 * g + (c >> 2)) * kRowPadV + (c & 3) * 8, *v1 = v0 + 16 * kRowPadV;
-#pragma unroll
-    for (int mt = 0; mt < 8; ++mt) {
-      vlo[mt] = load_transposed(v0 + mt * 32);
-      vhi[mt] = load_transposed(v1 + mt * 32);
-    }
-  };
-  auto second_half = [&](const Scores &sn, auto pv_tag, auto post_tag) __attribute__((always_inline)) -> bool {
-    constexpr bool kPV = decltype(pv_tag)::value, kPost = decltype(post_tag)::value;
-    float t[NB];
-    if constexpr (kPV) {
-#pragma unroll
-      for (int mt = 0; mt < 8; ++mt)
-#pragma unroll
-        for (int b = 0; b < NB; ++b)
-          acc[b][mt] = Mma<E>::run(make_uint4(vlo[mt].x, vlo[mt].y, vhi[mt].x, vhi[mt].y), pb[b], acc[b][mt]);
-    }
-    if constexpr (kPost) {  // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
-#pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        t[b] = kNegInf;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) t[b] = fmaxf(t[b], sn[b][j >> 2][j & 3]);
-      }
-    }
-    bool raise = false;
-    if constexpr (kPost) {
-#pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        mx[b] = t[b] * p.scale_log2;
-        raise |= mx[b] > m[b] + kRaise;  // also true for the first finite score of a row (m = -inf)
-      }
-    }
-    return __builtin_amdgcn_ballot_w64(raise) != 0;
-  };
-  // Masking of the scores of walk index xn, in place (selects, not branches: the comparison results are
-  // combined as bits). Skipped for the chunks every token of the wavefront sees whole.
-  auto mask_scores = [&](int xn, Scores &sn) __attribute__((always_inline)) {
-    if ((unsigned)(xn - full_lo) < full_cnt) return;
-    const int c0 = (ch_begin + xn) << 5;
-#pragma unroll
-    for (int b = 0; b < NB; ++b)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-        sn[b][j >> 2][j & 3] = bool((key > my_pos[b]) | (key < my_lo[b])) ? kNegInf : sn[b][j >> 2][j & 3];
-      }
-  };
-  const std::true_type kYes{};
-  const std::false_type kNo{};
-
-  // lift the reference points to the running maxima and rescale what has been accumulated
-  auto rescale = [&]() __attribute__((always_inline)) {
+    // this wavefront's NB column blocks: 16-token sub-tile ts[b] of head hd[b]
+    int ts[NB], hd[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      float t = mx[b];  // row maximum over the four lanes that share a token
-      t = fmaxf(t, __shfl_xor(t, 16));
-      t = fmaxf(t, __shfl_xor(t, 32));
-      const float m_new = fmaxf(m[b], t);
-      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
-      const float alpha = fast_exp2(m[b] - m_safe);
-      m[b] = m_new;
-      l[b] *= alpha;
-#pragma unroll
-      for (int mt = 0; mt < 8; ++mt) acc[b][mt] *= alpha;
+      ts[b] = wave & 3;
+      hd[b] = NB == 2 ? 2 * (wave >> 2) + b : NHEADS - 1;
     }
-  };
+    const int head0 = kvh * p.G + p.head_begin;
+    // (rows past the end of the sequence repeat its last token; they are never stored)
+    const int jw0 = min(q0 + 16 * ts[0], Lq - 1);            // first and last token of the wavefront
+    const int jw_last = min(q0 + 16 * ts[NB - 1] + 15, Lq - 1);
+    int my_pos[NB], my_lo[NB];
+    uint4 qb[NB][4];  // Q^T operands: token lane%16 of the block, dims of 16-byte piece 4s+g
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int j_mine = min(q0 + 16 * ts[b] + c, Lq - 1);
+      my_pos[b] = shift + j_mine;
+      my_lo[b] = max(wl >= 0 ? my_pos[b] - wl : 0, klo);
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        qb[b][s] = *reinterpret_cast<const uint4 *>(
+            p.q + ((int64_t)(qrow0 + j_mine) * p.q_sr + (int64_t)(head0 + hd[b]) * p.q_sh + (4 * s + g) * 8) * 2);
+    }
+    // Chunks wholly visible to every token of the wavefront (at or above every token's lower bound, at or below
+    // the first token) need no masking: walk indices [full_lo, full_lo + full_cnt).
+    const int vis_lo = max(wl >= 0 ? shift + jw_last - wl : 0, klo);
+    const int full_lo = ((vis_lo + 31) >> 5) - ch_begin;
+    const unsigned full_cnt = (unsigned)max(((shift + jw0 + 1) >> 5) - ch_begin - full_lo, 0);
 
-  if (fetcher) {
-    fetch(stage[0]);
-    fetch(stage[1]);
-  }
-  // ---- meta rows: global -> ring slot 0 -> scores, one chunk at a time, while the first two chunks of the
-  // window are on their way (every row that exists is visible to every token)
-  for (int mc = 0; mc < meta_chunks; ++mc) {
-    if (fetcher) {
-      const char *mk = p.meta_k + (int64_t)kvh * p.meta_sh + c * 16, *mv = p.meta_v + (int64_t)kvh * p.meta_sh + c * 16;
+    f32x4_t acc[NB][8];
+    float m[NB], l[NB];  // m: reference point of the numerators (log2 units), l: this lane's share of the sum
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      m[b] = kNegInf;
+      l[b] = 0.f;
+#pragma unroll
+      for (int mt = 0; mt < 8; ++mt) acc[b][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- global -> registers -> LDS: the first kFetchWaves wavefronts move the chunk (32 K rows and
+    // 32 V rows of 256 B); each of their loads covers 4 rows, all inside one 16-key tile of the table.
+    // Rows outside [wg_lo, wg_hi) are clamped onto the nearest visible key (masked for every token).
+    // Everything that does not depend on the lane is kept in scalar registers: per chunk, the tile's byte offset
+    // (one block-table entry, looked up one call ahead of its use) added to the K and V bases; a lane adds its
+    // row and column as a 32-bit offset.
+    constexpr int kFetchAll = S::kFetchWaves == S::kWaves;
+    const bool fetcher = kFetchAll || wave < S::kFetchWaves;
+    constexpr int rows_per_wave = 32 / S::kFetchWaves;                     // 4, 8 or 16
+    const int tsel = (wave * rows_per_wave) >> 4;                          // which 16-key tile of a chunk this wavefront's rows are in
+    const int lrow = (wave * rows_per_wave) % 16 + (lane >> 4);            // row inside the tile, +4 per load
+    const uint32_t row_bytes = (uint32_t)p.kv_sr;                          // < 2^24 (host check)
+    const uint32_t lane_col = c * (KVQ == SB_KV_NONE ? 16 : 8);
+    const int64_t wg_off = (int64_t)kvh * p.kv_sh + ((!PAGED && p.kv_start) ? p.kv_start[seq] * p.kv_sr : 0);
+    const char *const kbase = p.k + wg_off, *const vbase = p.v + wg_off;
+    const int32_t *const table_row = PAGED ? p.block_table + (int64_t)seq * p.bt_stride : nullptr;
+    auto walk_tile = [&](int x) __attribute__((always_inline)) {  // (past the end of the walk: the last tile again)
+      return min(max(2 * (ch_begin + x) + tsel, first_tile), last_tile);
+    };
+    // block of 16-key tile t: t / tiles_per_block by multiplication (exact while t < 2^31 / tiles_per_block)
+    auto block_of = [&](int t) __attribute__((always_inline)) { return (int)__umulhi((uint32_t)t << 1, p.tpb_magic); };
+    int next_blk = 0;  // table entry of the tile the next fetch takes
+    if constexpr (PAGED) next_blk = table_row[block_of(walk_tile(0))];
+    int fx = 0;        // walk index the next fetch takes
+    using Set = StageSet<KVQ, S::kLoads>;
+    Set stage[2];  // walk index x travels in set x & 1
+    auto fetch = [&](Set &st) __attribute__((always_inline)) {
+      const int t = walk_tile(fx);
+      ++fx;
+      int64_t off;  // of the tile's first row from kbase / vbase
+      [[maybe_unused]] int64_t scale_row = 0;  // INT8: index of that row in the scale tensors
+      if constexpr (PAGED) {
+        const int bi = block_of(t);
+        const int64_t blk = next_blk;
+        next_blk = table_row[block_of(walk_tile(fx))];
+        const int in_block = (t - bi * p.tiles_per_block) << 4;
+        off = blk * p.kv_sb + (int64_t)((uint32_t)in_block * row_bytes);
+        if constexpr (KVQ == SB_KV_INT8) scale_row = (blk * p.Hkv + kvh) * p.block_size + in_block;
+      } else {
+        off = (int64_t)(t << 4) * p.kv_sr;
+      }
+      const char *const kp = kbase + off, *const vp = vbase + off;
+      const int lo = wg_lo - (t << 4), hi = wg_hi - 1 - (t << 4);
 #pragma unroll
       for (int u = 0; u < S::kLoads; ++u) {
-        const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
-        const int64_t row = min((mc << 5) + kk, p.meta_len - 1);
-        *reinterpret_cast<uint4 *>(smem + kk * kRowPad + c * 16) = *reinterpret_cast<const uint4 *>(mk + row * p.meta_sr);
-        *reinterpret_cast<uint4 *>(smem + kStageK + kk * kRowPadV + c * 16) =
-            *reinterpret_cast<const uint4 *>(mv + row * p.meta_sr);
+        const int row = min(max(lrow + 4 * u, lo), hi);  // inside the tile: 0 .. 15
+        const uint32_t vo = __umul24((uint32_t)row, row_bytes) + lane_col;
+        if constexpr (KVQ == SB_KV_NONE) {
+          st.k[u] = *reinterpret_cast<const uint4 *>(kp + vo);  // (cached: the neighbouring query tiles read the same rows)
+          st.v[u] = *reinterpret_cast<const uint4 *>(vp + vo);
+        } else {  // a row is 128 code bytes: 8 per lane
+          const unsigned long long wk = *reinterpret_cast<const unsigned long long *>(kp + vo);
+          const unsigned long long wv = *reinterpret_cast<const unsigned long long *>(vp + vo);
+          st.k[u] = make_uint2((uint32_t)wk, (uint32_t)(wk >> 32));
+          st.v[u] = make_uint2((uint32_t)wv, (uint32_t)(wv >> 32));
+          if constexpr (KVQ == SB_KV_INT8) {
+            st.ks[u] = (p.k_scale + scale_row)[(uint32_t)row];
+            st.vs[u] = (p.v_scale + scale_row)[(uint32_t)row];
+          }
+        }
       }
-    }
-    __syncthreads();
-    first_half(0, sa, sa, kYes, kNo);
-    {
-      const int c0 = mc << 5;
+    };
+    const int stash_off = (wave * rows_per_wave + (lane >> 4)) * kRowPad + c * 16;   // of this lane's first row in a K chunk;
+    const int stash_off_v = (wave * rows_per_wave + (lane >> 4)) * kRowPadV + c * 16 + kStageK;  // in the V chunk behind it
+    auto stash = [&](int slot, const Set &st) __attribute__((always_inline)) {  // slot = byte offset of a ring slot
+      char *sk = smem + slot + stash_off, *sv = smem + slot + stash_off_v;
+#pragma unroll
+      for (int u = 0; u < S::kLoads; ++u) {
+        uint4 kq, vq;
+        if constexpr (KVQ == SB_KV_NONE) {
+          kq = st.k[u];
+          vq = st.v[u];
+        } else if constexpr (KVQ == SB_KV_INT8) {
+          kq = dequant8<E, KVQ>(st.k[u], st.ks[u]);
+          vq = dequant8<E, KVQ>(st.v[u], st.vs[u]);
+        } else {
+          kq = dequant8<E, KVQ>(st.k[u], p.k_scale_tensor);
+          vq = dequant8<E, KVQ>(st.v[u], p.v_scale_tensor);
+        }
+        *reinterpret_cast<uint4 *>(sk + 4 * u * kRowPad) = kq;
+        *reinterpret_cast<uint4 *>(sv + 4 * u * kRowPadV) = vq;
+      }
+    };
+
+    // Scores live in two register sets used alternately: while the numerators of one chunk are formed in one set,
+    // the matrix instructions write the next chunk's scores into the other. s[b][t][i]: block b, key 16 t + 4 g + i
+    // of the chunk (raw dot products; -inf where masked).
+    using Scores = f32x4_t[NB][2];
+    Scores sa, sb2;
+    float mx[NB];    // row maxima of the scores whose softmax comes next, in log2 units
+    uint4 pb[NB];    // probabilities of the chunk whose P V product comes next
+
+    // The two halves of an iteration. Each runs 16 matrix instructions next to the vector work of another chunk
+    // that does not depend on them.
+    //
+    // first half: S^T = K Q^T of the next chunk (kNext; K from ring slot `slot`) into `sn`, next to the
+    // numerators of the chunk in `sc` against the current reference points (kCur) -> pb, l.
+    auto first_half = [&](int slot, Scores &sn, Scores &sc, auto next_tag, auto cur_tag) __attribute__((always_inline)) {
+      constexpr bool kNext = decltype(next_tag)::value, kCur = decltype(cur_tag)::value;
+      const char *sk0 = smem + slot + c * kRowPad + g * 16, *sk1 = sk0 + 16 * kRowPad;
+      uint4 k0[4], k1[4];  // operand loads run one step ahead of their use (two pairs live)
+      if constexpr (kNext) {
+        k0[0] = *reinterpret_cast<const uint4 *>(sk0);
+        k1[0] = *reinterpret_cast<const uint4 *>(sk1);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) sn[b][0] = sn[b][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      }
+      float m_safe[NB], psum[NB];
+#pragma unroll
+      for (int b = 0; b < NB; ++b) m_safe[b] = (m[b] == kNegInf) ? 0.f : m[b];
+      if constexpr (kNext) {  // 2 NB chains (block, tile), each four instructions deep, taken in turn
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          if (s + 1 < 4) {
+            k0[s + 1] = *reinterpret_cast<const uint4 *>(sk0 + (s + 1) * 64);
+            k1[s + 1] = *reinterpret_cast<const uint4 *>(sk1 + (s + 1) * 64);
+          }
+#pragma unroll
+          for (int b = 0; b < NB; ++b) {
+            sn[b][0] = Mma<E>::run(k0[s], qb[b][s], sn[b][0]);
+            sn[b][1] = Mma<E>::run(k1[s], qb[b][s], sn[b][1]);
+          }
+        }
+      }
+      if constexpr (kCur) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          psum[b] = 0.f;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float e = fast_exp2(fmaf(sc[b][j >> 2][j & 3], p.scale_log2, -m_safe[b]));
+            sc[b][j >> 2][j & 3] = e;
+            psum[b] += e;
+          }
+        }
+      }
+      if constexpr (kCur) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          l[b] += psum[b];
+          pb[b] = make_uint4(Mma<E>::pack(sc[b][0][0], sc[b][0][1]), Mma<E>::pack(sc[b][0][2], sc[b][0][3]),
+                             Mma<E>::pack(sc[b][1][0], sc[b][1][1]), Mma<E>::pack(sc[b][1][2], sc[b][1][3]));
+        }
+      }
+    };
+
+    // second half: O^T += V^T P^T (kPV; probabilities pb), next to the row maxima of the (masked) scores `sn` of
+    // the next chunk (kPost). True when some row of that chunk needs a higher reference point.
+    // V^T operands of a chunk, dims 16 mt + c: this lane's 8 keys (4g .. 4g+3 of either 16-key tile, the order of
+    // its probabilities) by two transposing loads per mt; built once, used by both blocks. They are requested at
+    // the top of an iteration and arrive while the first half runs.
+    uint2 vlo[8], vhi[8];
+    auto load_v = [&](int slot) __attribute__((always_inline)) {
+      const char *v0 = smem + slot + kStageK + (4 * g + (c >> 2)) * kRowPadV + (c & 3) * 8, *v1 = v0 + 16 * kRowPadV;
+#pragma unroll
+      for (int mt = 0; mt < 8; ++mt) {
+        vlo[mt] = load_transposed(v0 + mt * 32);
+        vhi[mt] = load_transposed(v1 + mt * 32);
+      }
+    };
+    auto second_half = [&](const Scores &sn, auto pv_tag, auto post_tag) __attribute__((always_inline)) -> bool {
+      constexpr bool kPV = decltype(pv_tag)::value, kPost = decltype(post_tag)::value;
       float t[NB];
+      if constexpr (kPV) {
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        t[b] = kNegInf;
+        for (int mt = 0; mt < 8; ++mt)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
-          sa[b][j >> 2][j & 3] = key >= p.meta_len ? kNegInf : sa[b][j >> 2][j & 3];
-          t[b] = fmaxf(t[b], sa[b][j >> 2][j & 3]);
+          for (int b = 0; b < NB; ++b)
+            acc[b][mt] = Mma<E>::run(make_uint4(vlo[mt].x, vlo[mt].y, vhi[mt].x, vhi[mt].y), pb[b], acc[b][mt]);
+      }
+      if constexpr (kPost) {  // each lane checks its own 8 keys: no cross-lane traffic unless the reference point must move
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          t[b] = kNegInf;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) t[b] = fmaxf(t[b], sn[b][j >> 2][j & 3]);
         }
       }
       bool raise = false;
+      if constexpr (kPost) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          mx[b] = t[b] * p.scale_log2;
+          raise |= mx[b] > m[b] + kRaise;  // also true for the first finite score of a row (m = -inf)
+        }
+      }
+      return __builtin_amdgcn_ballot_w64(raise) != 0;
+    };
+    // Masking of the scores of walk index xn, in place (selects, not branches: the comparison results are
+    // combined as bits). Skipped for the chunks every token of the wavefront sees whole.
+    auto mask_scores = [&](int xn, Scores &sn) __attribute__((always_inline)) {
+      if ((unsigned)(xn - full_lo) < full_cnt) return;
+      const int c0 = (ch_begin + xn) << 5;
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+          sn[b][j >> 2][j & 3] = bool((key > my_pos[b]) | (key < my_lo[b])) ? kNegInf : sn[b][j >> 2][j & 3];
+        }
+    };
+    const std::true_type kYes{};
+    const std::false_type kNo{};
+
+    // lift the reference points to the running maxima and rescale what has been accumulated
+    auto rescale = [&]() __attribute__((always_inline)) {
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
-        mx[b] = t[b] * p.scale_log2;
-        raise |= mx[b] > m[b] + kRaise;
+        float t = mx[b];  // row maximum over the four lanes that share a token
+        t = fmaxf(t, __shfl_xor(t, 16));
+        t = fmaxf(t, __shfl_xor(t, 32));
+        const float m_new = fmaxf(m[b], t);
+        const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+        const float alpha = fast_exp2(m[b] - m_safe);
+        m[b] = m_new;
+        l[b] *= alpha;
+#pragma unroll
+        for (int mt = 0; mt < 8; ++mt) acc[b][mt] *= alpha;
       }
-      if (__builtin_amdgcn_ballot_w64(raise) != 0) rescale();
-    }
-    first_half(0, sa, sa, kNo, kYes);
-    load_v(0);
-    second_half(sa, kYes, kNo);
-    __syncthreads();
-  }
+    };
 
-  // ---- chunk loop: one barrier per chunk, every wavefront visits every chunk -------------------
-  // (chunks outside a wavefront's own band come out fully masked and add zero)
-  // Iteration x: scores of chunk x+1 while the numerators of chunk x are formed, then P V of chunk x while the
-  // scores of chunk x+1 are masked and searched for their maxima; chunk x+2 goes from registers into the ring
-  // slot that chunk x-1 has left, and chunk x+3 is requested from global memory into the registers chunk x+1
-  // has left (two register sets and two score sets used alternately; the loop is written out for both so that
-  // every register index is static). Loads are issued unconditionally (past the end they re-read the last
-  // rows), so the wait in front of each LDS store counts exactly the loads that may still be in flight.
-  int r0 = 0, r1 = kStage, r2 = 2 * kStage;  // ring slots of chunks x, x+1, x+2
-#ifdef SB_PREFILL_TIMING
-  long long tsum[6] = {0, 0, 0, 0, 0, 0};
-  long long tabs[14] = {0};
-#define SB_TICK(i) { const long long now = __builtin_readcyclecounter(); tsum[i] += now - tprev; tprev = now; if (x == 60) tabs[1 + i] = now; if (x == 61) tabs[8 + i] = now; }
-#else
-#define SB_TICK(i)
-#endif
-  auto body = [&](int x, Scores &sc, Scores &sn, Set &arriving, Set &leaving) __attribute__((always_inline)) {
-#ifdef SB_PREFILL_TIMING
-    long long tprev = __builtin_readcyclecounter();
-    if (x == 60) tabs[0] = tprev;
-    if (x == 61) tabs[7] = tprev;
-#endif
-    load_v(r0);
-    if (fetcher) fetch(arriving);  // chunk x + 3
-    SB_TICK(0)
-    first_half(r1, sn, sc, kYes, kYes);
-    SB_TICK(1)
-    mask_scores(x + 1, sn);
-    SB_TICK(2)
-    if (second_half(sn, kYes, kYes)) rescale();
-    SB_TICK(3)
-    if (fetcher) stash(r2, leaving);  // chunk x + 2
-    SB_TICK(4)
+    if (fetcher) {
+      fetch(stage[0]);
+      fetch(stage[1]);
+    }
+    // ---- meta rows: global -> ring slot 0 -> scores, one chunk at a time, while the first two chunks of the
+    // window are on their way (every row that exists is visible to every token)
+    for (int mc = 0; mc < meta_chunks; ++mc) {
+      if (fetcher) {
+        const char *mk = p.meta_k + (int64_t)kvh * p.meta_sh + c * 16, *mv = p.meta_v + (int64_t)kvh * p.meta_sh + c * 16;
+#pragma unroll
+        for (int u = 0; u < S::kLoads; ++u) {
+          const int kk = wave * rows_per_wave + (lane >> 4) + 4 * u;
+          const int64_t row = min((mc << 5) + kk, p.meta_len - 1);
+          *reinterpret_cast<uint4 *>(smem + kk * kRowPad + c * 16) = *reinterpret_cast<const uint4 *>(mk + row * p.meta_sr);
+          *reinterpret_cast<uint4 *>(smem + kStageK + kk * kRowPadV + c * 16) =
+              *reinterpret_cast<const uint4 *>(mv + row * p.meta_sr);
+        }
+      }
+      __syncthreads();
+      first_half(0, sa, sa, kYes, kNo);
+      {
+        const int c0 = mc << 5;
+        float t[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          t[b] = kNegInf;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int key = c0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+            sa[b][j >> 2][j & 3] = key >= p.meta_len ? kNegInf : sa[b][j >> 2][j & 3];
+            t[b] = fmaxf(t[b], sa[b][j >> 2][j & 3]);
+          }
+        }
+        bool raise = false;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          mx[b] = t[b] * p.scale_log2;
+          raise |= mx[b] > m[b] + kRaise;
+        }
+        if (__builtin_amdgcn_ballot_w64(raise) != 0) rescale();
+      }
+      first_half(0, sa, sa, kNo, kYes);
+      load_v(0);
+      second_half(sa, kYes, kNo);
+      __syncthreads();
+    }
+
+    // ---- chunk loop: one barrier per chunk, every wavefront visits every chunk -------------------
+    // (chunks outside a wavefront's own band come out fully masked and add zero)
+    // Iteration x: scores of chunk x+1 while the numerators of chunk x are formed, then P V of chunk x while the
+    // scores of chunk x+1 are masked and searched for their maxima; chunk x+2 goes from registers into the ring
+    // slot that chunk x-1 has left, and chunk x+3 is requested from global memory into the registers chunk x+1
+    // has left (two register sets and two score sets used alternately; the loop is written out for both so that
+    // every register index is static). Loads are issued unconditionally (past the end they re-read the last
+    // rows), so the wait in front of each LDS store counts exactly the loads that may still be in flight.
+    int r0 = 0, r1 = kStage, r2 = 2 * kStage;  // ring slots of chunks x, x+1, x+2
+    auto body = [&](int x, Scores &sc, Scores &sn, Set &arriving, Set &leaving) __attribute__((always_inline)) {
+      load_v(r0);
+      if (fetcher) fetch(arriving);  // chunk x + 3
+      first_half(r1, sn, sc, kYes, kYes);
+      mask_scores(x + 1, sn);
+      if (second_half(sn, kYes, kYes)) rescale();
+      if (fetcher) stash(r2, leaving);  // chunk x + 2
+      __syncthreads();
+      const int t = r0;
+      r0 = r1;
+      r1 = r2;
+      r2 = t;
+    };
+    if (fetcher) {
+      stash(r0, stage[0]);
+      fetch(stage[0]);  // chunk 2
+      stash(r1, stage[1]);
+    }
     __syncthreads();
-    SB_TICK(5)
-    const int t = r0;
-    r0 = r1;
-    r1 = r2;
-    r2 = t;
-  };
-  if (fetcher) {
-    stash(r0, stage[0]);
-    fetch(stage[0]);  // chunk 2
-    stash(r1, stage[1]);
-  }
-  __syncthreads();
-  first_half(r0, sa, sa, kYes, kNo);
-  mask_scores(0, sa);
-  if (second_half(sa, kNo, kYes)) rescale();
-  int x = 0;
-  for (; x + 2 < n_walk; x += 2) {
-    body(x, sa, sb2, stage[1], stage[0]);
-    body(x + 1, sb2, sa, stage[0], stage[1]);
-  }
-  if (x + 1 < n_walk) {
-    body(x, sa, sb2, stage[1], stage[0]);
+    first_half(r0, sa, sa, kYes, kNo);
+    mask_scores(0, sa);
+    if (second_half(sa, kNo, kYes)) rescale();
+    int x = 0;
+    for (; x + 2 < n_walk; x += 2) {
+      body(x, sa, sb2, stage[1], stage[0]);
+      body(x + 1, sb2, sa, stage[0], stage[1]);
+    }
+    if (x + 1 < n_walk) {
+      body(x, sa, sb2, stage[1], stage[0]);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        sa[b][0] = sb2[b][0];
+        sa[b][1] = sb2[b][1];
+      }
+    }
+    // the last chunk: its numerators and its P V product
+    load_v(r0);
+    first_half(r1, sa, sa, kNo, kYes);
+    second_half(sa, kYes, kNo);
+
+    // ---- epilogue: lane (g, c) owns token c of each block, dims 16 mt + 4g + i --------------------------
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      sa[b][0] = sb2[b][0];
-      sa[b][1] = sb2[b][1];
-    }
-  }
-  // the last chunk: its numerators and its P V product
-  load_v(r0);
-  first_half(r1, sa, sa, kNo, kYes);
-  second_half(sa, kYes, kNo);
-
-  // ---- epilogue: lane (g, c) owns token c of each block, dims 16 mt + 4g + i --------------------------
+      float lt = l[b];
+      lt += __shfl_xor(lt, 16);
+      lt += __shfl_xor(lt, 32);
+      if (q0 + 16 * ts[b] + c < Lq) {
+        const float inv = lt > 0.f ? 1.f / lt : 0.f;
+        char *dst = p.out + ((int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.o_sr + (int64_t)(head0 + hd[b]) * p.o_sh +
+                             4 * g) * 2;
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    float lt = l[b];
-    lt += __shfl_xor(lt, 16);
-    lt += __shfl_xor(lt, 32);
-    if (q0 + 16 * ts[b] + c < Lq) {
-      const float inv = lt > 0.f ? 1.f / lt : 0.f;
-      char *dst = p.out + ((int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.o_sr + (int64_t)(head0 + hd[b]) * p.o_sh +
-                           4 * g) * 2;
-#pragma unroll
-      for (int mt = 0; mt < 8; ++mt)
-        *reinterpret_cast<uint2 *>(dst + 32 * mt) = make_uint2(E::pack(acc[b][mt][0] * inv, acc[b][mt][1] * inv),
-                                                               E::pack(acc[b][mt][2] * inv, acc[b][mt][3] * inv));
-#ifndef SB_PREFILL_TIMING
-      if (p.lse && g == 0)
-        p.lse[(int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.Hq + head0 + hd[b]] =
-            lt > 0.f ? (m[b] + log2f(lt)) * kLn2 : kNegInf;
-#endif
+        for (int mt = 0; mt < 8; ++mt)
+          *reinterpret_cast<uint2 *>(dst + 32 * mt) = make_uint2(E::pack(acc[b][mt][0] * inv, acc[b][mt][1] * inv),
+                                                                 E::pack(acc[b][mt][2] * inv, acc[b][mt][3] * inv));
+        if (p.lse && g == 0)
+          p.lse[(int64_t)(qrow0 + q0 + 16 * ts[b] + c) * p.Hq + head0 + hd[b]] =
+              lt > 0.f ? (m[b] + log2f(lt)) * kLn2 : kNegInf;
+      }
     }
-  }
-#ifdef SB_PREFILL_TIMING
-  if (p.lse && tile == p.num_tiles / 2 + 100 && kvh == 0 && lane == 0) {
-    for (int i = 0; i < 6; ++i) p.lse[wave * 8 + i] = (float)tsum[i];
-    p.lse[wave * 8 + 6] = (float)n_walk;
-    for (int i = 0; i < 14; ++i) p.lse[64 + wave * 16 + i] = (float)(tabs[i] & 0xffffff);
-  }
-#endif
   };
   if constexpr (NHEADS % 2 == 1) {
     if (wave >= 4 * S::kPairs) run(std::integral_constant<int, 1>{});
