@@ -377,7 +377,8 @@ typedef struct sb_swa_prefill_args {
   float scale;
   int64_t q_stride_row, q_stride_head;     /* elements */
   int64_t out_stride_row, out_stride_head;
-  int64_t kv_stride_block, kv_stride_row, kv_stride_head; /* elements; block stride unused when dense */
+  int64_t kv_stride_block, kv_stride_row, kv_stride_head; /* elements; block stride unused when dense;
+                                                             a row stride of 16 MiB or more is rejected */
   int64_t block_table_stride;
   void *stream;
   float *lse;      /* optional, fp32 [total_q, Hq], natural log: log-sum-exp of each query's scaled scores,
