@@ -205,6 +205,13 @@ typedef struct sb_swa_decode_args {
    * bf16/fp16 caches; ignored elsewhere. */
   void *profile_start_event;
   void *profile_stop_event;
+  /* The two score options the backend passes on to flash-attn (meta_attention.py:665-690, :965-981
+   * alibi_slopes=..., softcap=...): softcap > 0 turns every scaled score x into softcap * tanh(x / softcap);
+   * alibi_slopes ([num_q_heads] fp32, NULL = off) adds -slope[h] * (query position - key index), the query
+   * sitting at key index seq_lens[r]-1. Both are applied in front of the mask, the cap first. bf16/fp16
+   * queries on the matrix-core kernels (element, INT8 and fp8 caches); not together with meta tokens. */
+  float softcap;
+  const float *alibi_slopes;
 } sb_swa_decode_args;
 
 /* Split count the auto rule (n_split = 0) would use for these shapes: the one with the lowest estimated
@@ -400,6 +407,10 @@ typedef struct sb_swa_prefill_args {
   const void *meta_v;
   int32_t meta_len;
   int64_t meta_stride_row, meta_stride_head;
+  /* Score options as for sb_swa_decode (fa_kernel_metatoken.py:235-253 alibi_slopes=..., softcap=...): query j
+   * of a sequence sits at key index seq_lens_k - query_len + j. Not together with meta tokens. */
+  float softcap;
+  const float *alibi_slopes;
 } sb_swa_prefill_args;
 
 int sb_swa_prefill(const sb_swa_prefill_args *args);

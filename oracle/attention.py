@@ -29,16 +29,26 @@ def sliding_causal_mask(q_len: int, k_len: int, window_size: int) -> np.ndarray:
 
 
 def masked_softmax_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, masked: np.ndarray,
-                             scale: Optional[float] = None, return_lse: bool = False):
+                             scale: Optional[float] = None, return_lse: bool = False,
+                             softcap: float = 0.0, bias: Optional[np.ndarray] = None):
     """softmax(q k^T * scale + (-inf where masked)) v with fully-masked rows -> 0
     (window_attention_sdpa.py:205-214: additive -inf mask, SDPA default scale D^-0.5,
-    nan_to_num(nan=0)). q [..., Q, D], k/v [..., K, D], masked broadcastable to [..., Q, K]."""
+    nan_to_num(nan=0)). q [..., Q, D], k/v [..., K, D], masked broadcastable to [..., Q, K].
+    softcap > 0 and bias are the two options the backend hands to flash-attn
+    (vllm_hymeta/attention/meta_attention.py:686-690 logits_soft_cap, :665-670 alibi_slopes;
+    fa_kernel_metatoken.py:157-168, 235-253 pass them on as softcap / alibi_slopes): the scaled
+    scores become softcap * tanh(scores / softcap), then the bias (broadcastable to [..., Q, K]) is
+    added, then the mask."""
     q = np.asarray(q, np.float64)
     k = np.asarray(k, np.float64)
     v = np.asarray(v, np.float64)
     if scale is None:
         scale = q.shape[-1] ** -0.5
     s = np.einsum("...qd,...kd->...qk", q, k) * scale
+    if softcap > 0:
+        s = softcap * np.tanh(s / softcap)
+    if bias is not None:
+        s = s + np.asarray(bias, np.float64)
     s = np.where(masked, -np.inf, s)
     mx = s.max(axis=-1, keepdims=True)
     mx_safe = np.where(np.isfinite(mx), mx, 0.0)
@@ -104,9 +114,16 @@ def gather_paged(cache: np.ndarray, block_table_row: Sequence[int], n: int) -> n
     return cache[blocks].reshape(nb * bs, cache.shape[2], cache.shape[3])[:n]
 
 
+def alibi_bias(slope: float, query_pos: np.ndarray, n_keys: int) -> np.ndarray:
+    """The ALiBi term flash-attn adds for a query at key position query_pos: -slope * |query_pos - key|
+    for every key index (the causal mask removes the keys to the right). Returns [len(query_pos), n_keys]."""
+    return -float(slope) * np.abs(np.asarray(query_pos)[:, None] - np.arange(n_keys)[None, :])
+
+
 def paged_decode_attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray,
                            block_tables: np.ndarray, cache_seqlens: Sequence[int], scale: float,
-                           window_left: int, return_lse: bool = False):
+                           window_left: int, return_lse: bool = False, softcap: float = 0.0,
+                           alibi_slopes: Optional[Sequence[float]] = None):
     """Semantics of flash_attn_with_kvcache as called at
     vllm_hymeta/attention/fa_kernel_metatoken.py:157-168: one query per sequence placed at key
     index cache_seqlens-1, causal, window_size=(window_left, -1): key i visible iff
@@ -126,15 +143,17 @@ def paged_decode_attention(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarr
         i = np.arange(n)
         masked = np.zeros(n, bool) if window_left < 0 else (i < n - 1 - window_left)
         for h in range(Hq):
+            bias = None if alibi_slopes is None else alibi_bias(alibi_slopes[h], np.array([n - 1]), n)
             o, ls = masked_softmax_attention(np.asarray(q[b, h], np.float64)[None], kk[:, h // G], vv[:, h // G],
-                                             masked[None], scale, return_lse=True)
+                                             masked[None], scale, return_lse=True, softcap=softcap, bias=bias)
             out[b, h] = o[0]
             lse[b, h] = ls[0]
     return (out, lse) if return_lse else out
 
 
 def varlen_window_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, cu_seqlens_q: Sequence[int],
-                            cu_seqlens_k: Sequence[int], scale: float, window_left: int) -> np.ndarray:
+                            cu_seqlens_k: Sequence[int], scale: float, window_left: int, softcap: float = 0.0,
+                            alibi_slopes: Optional[Sequence[float]] = None) -> np.ndarray:
     """Semantics of the varlen causal sliding-window call at
     vllm_hymeta/attention/fa_kernel_metatoken.py:235-253 (bottom-right aligned causal mask):
     query j of a sequence with Lq queries and Lk keys sits at key position Lk-Lq+j and sees keys
@@ -155,7 +174,9 @@ def varlen_window_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, cu_seql
         if window_left >= 0:
             masked |= kp[None, :] < (pos[:, None] - window_left)
         for h in range(Hq):
-            out[q0:q1, h] = masked_softmax_attention(q[q0:q1, h], k[k0:k1, h // G], v[k0:k1, h // G], masked, scale)
+            bias = None if alibi_slopes is None else alibi_bias(alibi_slopes[h], pos, Lk)
+            out[q0:q1, h] = masked_softmax_attention(q[q0:q1, h], k[k0:k1, h // G], v[k0:k1, h // G], masked, scale,
+                                                     softcap=softcap, bias=bias)
     return out
 
 

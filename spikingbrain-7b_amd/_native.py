@@ -61,6 +61,7 @@ class SwaDecodeArgs(C.Structure):
         ("k_scale_tensor", f32), ("v_scale_tensor", f32),
         ("meta_k", vp), ("meta_v", vp), ("meta_len", i32), ("meta_stride_row", i64), ("meta_stride_head", i64),
         ("profile_start_event", vp), ("profile_stop_event", vp),
+        ("softcap", f32), ("alibi_slopes", vp),
     ]
 
 
@@ -104,6 +105,7 @@ class SwaPrefillArgs(C.Structure):
         ("stream", vp), ("lse", vp), ("k_scale", vp), ("v_scale", vp), ("kv_quant", i32),
         ("k_scale_tensor", f32), ("v_scale_tensor", f32),
         ("meta_k", vp), ("meta_v", vp), ("meta_len", i32), ("meta_stride_row", i64), ("meta_stride_head", i64),
+        ("softcap", f32), ("alibi_slopes", vp),
     ]
 
 

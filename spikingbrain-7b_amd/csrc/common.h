@@ -87,6 +87,25 @@ __device__ __forceinline__ float row16_allreduce_sum(float v) {
 // exp2 with the hardware instruction (inputs here are <= 0 or -inf).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The two score options flash-attn takes from the backend (vllm_hymeta/attention/meta_attention.py:665-690:
+// alibi_slopes, logits_soft_cap). A raw dot product s becomes, in the units the kernels keep their scores in,
+//   (cap * tanh(s * mult / cap) + slope * dist) / mult,     mult = softmax scale (times a cache's K scale),
+// dist = key index - query position (<= 0 for visible keys), cap = 0: no cap. tanh(y) = 1 - 2 / (exp(2y) + 1)
+// holds at both ends (exp -> inf gives 1, exp -> 0 gives -1).
+struct ScoreOptions {
+  float mult, inv_mult, cap, inv_cap2_log2e;  // inv_cap2_log2e = 2 log2(e) / cap
+  const float *slopes;                        // [Hq] or null
+  int on;                                     // 0: scores stay as they are
+};
+__device__ __forceinline__ float adjust_score(const ScoreOptions &o, float s, float slope, float dist) {
+  float x = s * o.mult;
+  if (o.cap > 0.f) {
+    const float e = fast_exp2(x * o.inv_cap2_log2e);
+    x = o.cap * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
+  }
+  return fmaf(slope, dist, x) * o.inv_mult;
+}
+
 }  // namespace sb
 
 // Host-side error plumbing shared by the entry points.

@@ -761,6 +761,24 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
       p.meta_v_mult = 1.f / a->v_scale_tensor;
     }
   }
+  // optional soft cap / ALiBi slopes on the scores
+  p.opt.on = 0;
+  p.opt.slopes = nullptr;
+  p.opt.cap = p.opt.inv_cap2_log2e = 0.f;
+  p.opt.mult = p.scale_log2 / sb::kLog2e;  // what turns a raw dot product into the scaled score (K tensor scale included)
+  p.opt.inv_mult = 1.f / p.opt.mult;
+  if (a->softcap < 0.f || a->softcap != a->softcap) return fail(SB_ERR_INVALID, "sb_swa_decode: softcap must be >= 0");
+  if (a->softcap > 0.f || a->alibi_slopes) {
+    if (!mfma)
+      return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: soft cap / ALiBi need bf16/fp16 queries on the matrix-core kernels");
+    if (a->meta_len > 0) return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: soft cap / ALiBi together with meta tokens");
+    p.opt.on = 1;
+    p.opt.slopes = a->alibi_slopes;
+    if (a->softcap > 0.f) {
+      p.opt.cap = a->softcap;
+      p.opt.inv_cap2_log2e = 2.f * sb::kLog2e / a->softcap;
+    }
+  }
   if (mfma && !int8_kv && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
     p.n_wg = (int)balanced_workgroups(a->num_rows, n_split);
   // On request the fixed split of the matrix-core kernel merges in the same launch (the last wavefront of a

@@ -99,6 +99,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           p.q + (r * p.q_sr + (int64_t)(kvh * G + c) * p.q_sh + 32 * g + 8 * s) * 2);
   }
 
+  const float my_slope = (p.opt.slopes && c < G) ? p.opt.slopes[kvh * G + c] : 0.f;  // ALiBi slope of this lane's head
+
   f32x4_t acc[8];
 #pragma unroll
   for (int mt = 0; mt < 8; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -156,6 +158,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     bool vis[8];
     const int i0 = ch << 5;
+    if (p.opt.on) {  // soft cap / ALiBi (wave-uniform; the query sits at key index hi - 1)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        sc[j] = adjust_score(p.opt, sc[j], my_slope, (float)(i0 + ((j >> 2) << 4) + 4 * g + (j & 3) - (hi - 1)));
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int i = i0 + ((j >> 2) << 4) + 4 * g + (j & 3);

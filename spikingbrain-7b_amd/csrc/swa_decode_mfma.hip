@@ -91,6 +91,8 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
           p.q + (r * p.q_sr + (int64_t)(kvh * G + c) * p.q_sh + (4 * s + g) * 8) * 2);
   }
 
+  const float my_slope = (p.opt.slopes && c < G) ? p.opt.slopes[kvh * G + c] : 0.f;  // ALiBi slope of this lane's head
+
   f32x4_t acc[8];
 #pragma unroll
   for (int mt = 0; mt < 8; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -254,6 +256,11 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
       s1 = Mma<E>::run(ck.k1[s], qb[s], s1);
     }
     float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+    if (p.opt.on) {  // soft cap / ALiBi (wave-uniform; the query sits at key index hi - 1)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        sc[j] = adjust_score(p.opt, sc[j], my_slope, (float)((ch << 5) + ((j >> 2) << 4) + 4 * g + (j & 3) - (hi - 1)));
+    }
     if constexpr (kMask) {
       const int i0 = ch << 5;
 #pragma unroll

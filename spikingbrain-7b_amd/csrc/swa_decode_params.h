@@ -1,6 +1,7 @@
 // Kernel parameter block shared by the two split kernels (VALU and matrix-core) and the merge.
 #pragma once
 #include <stdint.h>
+#include "common.h"
 #ifndef SB_BALANCED_T
 #define SB_BALANCED_T 3
 #endif
@@ -60,6 +61,8 @@ struct DecodeParams {
   // Over a byte-code cache the meta rows are still elements: their scores and probabilities are multiplied by
   // these so that the scales folded into scale_log2 and kv_out_scale (fp8 cache) cancel for them; else 1.
   float meta_k_mult, meta_v_mult;
+  // soft cap / ALiBi (matrix-core kernels): applied to every raw score in front of the mask
+  ScoreOptions opt;
 };
 
 }  // namespace sb

@@ -80,6 +80,7 @@ struct PrefillParams {
   const char *meta_v;
   int meta_len;
   int64_t meta_sr, meta_sh;  // bytes
+  ScoreOptions opt;          // soft cap / ALiBi slopes, applied to every raw score in front of the mask
 };
 
 #ifndef SB_PREFILL_HEADS
@@ -413,6 +414,20 @@ void swa_prefill_kernel(const PrefillParams p) {
       }
       return __builtin_amdgcn_ballot_w64(raise) != 0;
     };
+    // Soft cap / ALiBi on the scores of walk index xn, in place (only when asked for: one uniform branch).
+    float my_slope[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) my_slope[b] = p.opt.slopes ? p.opt.slopes[head0 + hd[b]] : 0.f;
+    auto adjust_scores = [&](int xn, Scores &sn) __attribute__((always_inline)) {
+      if (!p.opt.on) return;
+      const int c0 = (ch_begin + xn) << 5;
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          sn[b][j >> 2][j & 3] = adjust_score(p.opt, sn[b][j >> 2][j & 3], my_slope[b],
+                                              (float)(c0 + ((j >> 2) << 4) + 4 * g + (j & 3) - my_pos[b]));
+    };
     // Masking of the scores of walk index xn, in place (selects, not branches: the comparison results are
     // combined as bits). Skipped for the chunks every token of the wavefront sees whole.
     auto mask_scores = [&](int xn, Scores &sn) __attribute__((always_inline)) {
@@ -506,6 +521,7 @@ void swa_prefill_kernel(const PrefillParams p) {
       load_v(r0);
       if (fetcher) fetch(arriving);  // chunk x + 3
       first_half(r1, sn, sc, kYes, kYes);
+      adjust_scores(x + 1, sn);
       mask_scores(x + 1, sn);
       if (second_half(sn, kYes, kYes)) rescale();
       if (fetcher) stash(r2, leaving);  // chunk x + 2
@@ -522,6 +538,7 @@ void swa_prefill_kernel(const PrefillParams p) {
     }
     __syncthreads();
     first_half(r0, sa, sa, kYes, kNo);
+    adjust_scores(0, sa);
     mask_scores(0, sa);
     if (second_half(sa, kNo, kYes)) rescale();
     int x = 0;
@@ -650,6 +667,21 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   p.meta_k = p.meta_v = nullptr;
   p.meta_len = 0;
   p.meta_sr = p.meta_sh = 0;
+  p.opt.on = 0;
+  p.opt.slopes = nullptr;
+  p.opt.cap = p.opt.inv_cap2_log2e = 0.f;
+  p.opt.mult = a->scale;  // (byte-code rows are dequantised on their way into LDS: the scores are those of elements)
+  p.opt.inv_mult = 1.f / p.opt.mult;
+  if (a->softcap < 0.f || a->softcap != a->softcap) return fail(SB_ERR_INVALID, "sb_swa_prefill: softcap must be >= 0");
+  if (a->softcap > 0.f || a->alibi_slopes) {
+    if (a->meta_len > 0) return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: soft cap / ALiBi together with meta tokens");
+    p.opt.on = 1;
+    p.opt.slopes = a->alibi_slopes;
+    if (a->softcap > 0.f) {
+      p.opt.cap = a->softcap;
+      p.opt.inv_cap2_log2e = 2.f * sb::kLog2e / a->softcap;
+    }
+  }
   if (a->meta_len < 0) return fail(SB_ERR_INVALID, "sb_swa_prefill: negative meta_len");
   if (a->meta_len > 0) {
     if (!a->meta_k || !a->meta_v) return fail(SB_ERR_INVALID, "sb_swa_prefill: meta_len without meta_k / meta_v");

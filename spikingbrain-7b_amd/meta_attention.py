@@ -412,9 +412,12 @@ class MetaAttentionImpl:
         self.head_size = head_size
         self.scale = float(scale)
         self.num_kv_heads = num_kv_heads
+        # (:665-670) one slope per query head, kept as an fp32 tensor and handed to the kernels as it is
         if alibi_slopes is not None:
-            raise NotImplementedError("ALiBi slopes are not supported by the gfx950 window-attention kernels.")
-        self.alibi_slopes = None
+            alibi_slopes = torch.tensor(alibi_slopes, dtype=torch.float32)
+            if alibi_slopes.shape != (num_heads,):
+                raise ValueError(f"alibi_slopes must hold one slope per query head ({num_heads})")
+        self.alibi_slopes = alibi_slopes
         self.sliding_window = ((sliding_window - 1, 0) if sliding_window is not None else (-1, -1))
         self.kv_cache_dtype = kv_cache_dtype
         self.num_meta_tokens = num_meta_tokens
@@ -427,10 +430,11 @@ class MetaAttentionImpl:
                 f"MetaAttention does not support {self.kv_cache_dtype} kv-cache on this device "
                 "(fp8 means e4m3fn here).")
         if logits_soft_cap is None:
+            # (:686-690) in flash-attn a soft cap of 0 means no soft cap; the kernels here read it the same way
             logits_soft_cap = 0
-        if logits_soft_cap != 0:
-            raise NotImplementedError("logits_soft_cap is not supported by the gfx950 window-attention kernels.")
-        self.logits_soft_cap = logits_soft_cap
+        if logits_soft_cap < 0:
+            raise ValueError("logits_soft_cap must be >= 0")
+        self.logits_soft_cap = float(logits_soft_cap)
         self.num_queries_per_kv = self.num_heads // self.num_kv_heads
         support_head_sizes = MetaAttentionBackend.get_supported_head_sizes()
         if self.head_size not in support_head_sizes:
@@ -541,6 +545,14 @@ class MetaAttentionImpl:
         meta_inside = with_meta and query.dtype in (torch.bfloat16, torch.float16)
         meta_kv = dict(meta_k=key2, meta_v=value2) if meta_inside else {}
         want_lse = with_meta and not meta_inside
+        # The two score options (:758-759, handed to every flash-attn call of the step) travel with the
+        # meta rows' arguments to whichever kernel takes a piece of the step.
+        if self.logits_soft_cap > 0 or self.alibi_slopes is not None:
+            if with_meta:
+                raise NotImplementedError("meta tokens together with logits_soft_cap / alibi_slopes")
+            if self.alibi_slopes is not None and self.alibi_slopes.device != query.device:
+                self.alibi_slopes = self.alibi_slopes.to(query.device)
+            meta_kv = dict(softcap=self.logits_soft_cap, alibi_slopes=self.alibi_slopes)
 
         def merge_meta(q_part, out_part, lse_part):
             """out_part (attention over the window, log-sum-exp lse_part) takes in the meta tokens."""

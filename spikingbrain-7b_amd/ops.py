@@ -125,8 +125,15 @@ def swa_decode_attention(
     meta_k: Optional[torch.Tensor] = None,
     meta_v: Optional[torch.Tensor] = None,
     profile_events=None,
+    softcap: float = 0.0,
+    alibi_slopes: Optional[torch.Tensor] = None,
 ):
     """Single-query window attention for each row of q [R, Hq, D].
+
+    softcap > 0: every scaled score x becomes softcap * tanh(x / softcap); alibi_slopes [Hq] fp32 (device):
+    -slope[h] * (query position - key index) is added, the query sitting at the row's last key. Both in front
+    of the mask, the cap first (what flash-attn does with the backend's logits_soft_cap / alibi_slopes);
+    bf16/fp16 queries only, not together with meta tokens.
 
     profile_events: (start, stop) torch.cuda.Event pair made by `timing_events()`: attached to the split
     kernel's own dispatch, so start.elapsed_time(stop) is that kernel's duration alone (fixed-split
@@ -303,9 +310,20 @@ def swa_decode_attention(
         k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale),
         kv_quant=N.SB_KV_FP8 if fp8_kv else (N.SB_KV_INT8 if int8_kv else N.SB_KV_NONE),
         k_scale_tensor=float(fp8_scales[0]) if fp8_kv else 0.0, v_scale_tensor=float(fp8_scales[1]) if fp8_kv else 0.0,
+        softcap=float(softcap), alibi_slopes=N.ptr(_slopes(alibi_slopes, Hq, dev)),
         **fused, **_event_args(profile_events))
     N.check(L.sb_swa_decode(C.byref(a)), "swa_decode")
     return (out, lse) if return_lse else out
+
+
+def _slopes(alibi_slopes, num_q_heads: int, device) -> Optional[torch.Tensor]:
+    """ALiBi slopes as the kernels read them: fp32 [Hq], contiguous, on the queries' device."""
+    if alibi_slopes is None:
+        return None
+    t = torch.as_tensor(alibi_slopes, dtype=torch.float32, device=device).contiguous()
+    if t.shape != (num_q_heads,):
+        raise ValueError(f"alibi_slopes must have one slope per query head ({num_q_heads}), got {tuple(t.shape)}")
+    return t
 
 
 def timing_events(device) -> Tuple[torch.cuda.Event, torch.cuda.Event]:
@@ -507,8 +525,12 @@ def swa_prefill_attention(
     fp8_scales: Optional[Tuple[float, float]] = None,
     meta_k: Optional[torch.Tensor] = None,
     meta_v: Optional[torch.Tensor] = None,
+    softcap: float = 0.0,
+    alibi_slopes: Optional[torch.Tensor] = None,
 ):
     """Causal sliding-window attention for q [total_q, Hq, D] packed sequence after sequence.
+    softcap / alibi_slopes: as for swa_decode_attention; query j of a sequence sits at key position
+    seq_len_k - query_len + j.
     With return_lse also the fp32 [total_q, Hq] natural-log log-sum-exp of each query's scores.
     meta_k/meta_v [M, Hkv, D]: meta (sink) tokens every query also attends to, unmasked, in the same
     softmax (not over byte-code caches).
@@ -627,7 +649,8 @@ def swa_prefill_attention(
         block_table_stride=bt_stride, stream=N.stream_ptr(dev), lse=N.ptr(lse),
         k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale), kv_quant=kv_quant,
         k_scale_tensor=float(fp8_scales[0]) if fp8_scales is not None else 0.0,
-        v_scale_tensor=float(fp8_scales[1]) if fp8_scales is not None else 0.0, **meta)
+        v_scale_tensor=float(fp8_scales[1]) if fp8_scales is not None else 0.0,
+        softcap=float(softcap), alibi_slopes=N.ptr(_slopes(alibi_slopes, Hq, dev)), **meta)
     N.check(N.lib().sb_swa_prefill(C.byref(a)), "swa_prefill")
     return (out, lse) if return_lse else out
 

@@ -1,0 +1,186 @@
+"""Soft cap and ALiBi slopes on the attention scores: the two options the backend hands to every flash-attn call
+(vllm_hymeta/attention/meta_attention.py:665-690, :758-759, :882-883, :916-918, :950-952, :978-980), in the
+decode kernels (element, INT8 and fp8 caches; fixed and balanced split), the many-query kernel (in-flight and
+paged keys) and through MetaAttentionImpl.forward, against the float64 oracle.
+Tolerance: max-abs 2e-2 (bf16), 5e-3 (fp16), against fp64 mathematics on the same (for byte-code caches:
+dequantised) rows."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as A
+from oracle import quant as Q
+
+pytestmark = pytest.mark.gpu
+
+D = 128
+TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3}
+OPTIONS = [dict(softcap=0.0, alibi=True), dict(softcap=3.0, alibi=False), dict(softcap=1.5, alibi=True)]
+
+
+def slopes_for(Hq):
+    return [2.0 ** (-8.0 * (h + 1) / Hq) for h in range(Hq)]           # the usual geometric ALiBi slopes
+
+
+def paged_problem(lens, bs, Hkv, dtype, seed, slack=4):
+    g = torch.Generator().manual_seed(seed)
+    need = [(n + bs - 1) // bs for n in lens]
+    nb = sum(need) + slack
+    perm = torch.randperm(nb, generator=g)
+    kv = torch.randn(2, nb, bs, Hkv, D, generator=g).to(dtype)
+    tables = torch.zeros(len(lens), max(need), dtype=torch.int32)
+    p = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[p:p + n]; p += n
+    return kv, tables
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Hq,Hkv", [(28, 4), (8, 2), (5, 1)])
+@pytest.mark.parametrize("opt", OPTIONS)
+@pytest.mark.parametrize("wl,n_split,balanced", [(64, 1, False), (100, 3, False), (-1, 2, False), (80, 2, True)])
+def test_decode_with_soft_cap_and_alibi(sb, dev, dtype, Hq, Hkv, opt, wl, n_split, balanced):
+    bs = 16
+    lens = [1, 16, 17, 65, 129, 300]
+    kv, tables = paged_problem(lens, bs, Hkv, dtype, seed=Hq + n_split)
+    q = (2.0 * torch.randn(len(lens), Hq, D, generator=torch.Generator().manual_seed(3))).to(dtype)  # scores large enough for the cap to bite
+    slopes = slopes_for(Hq) if opt["alibi"] else None
+    scale = D ** -0.5
+    out, lse = sb.ops.swa_decode_attention(
+        q.to(dev), kv[0].to(dev), kv[1].to(dev), torch.tensor(lens, dtype=torch.int32, device=dev),
+        block_table=tables.to(dev), window_left=wl, scale=scale, n_split=n_split, balanced=balanced, return_lse=True,
+        softcap=opt["softcap"], alibi_slopes=None if slopes is None else torch.tensor(slopes, device=dev))
+    ref, ref_lse = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(), tables.numpy(),
+                                            lens, scale, wl, return_lse=True, softcap=opt["softcap"], alibi_slopes=slopes)
+    assert np.abs(out.float().cpu().numpy() - ref).max() <= TOL[dtype]
+    assert np.abs(lse.cpu().numpy() - ref_lse).max() <= 2e-3
+    plain = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(), tables.numpy(),
+                                     lens, scale, wl)
+    assert np.abs(plain - ref).max() > 5 * TOL[dtype]                   # the options do change the result here
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+@pytest.mark.parametrize("opt", OPTIONS)
+def test_decode_over_byte_code_cache_with_soft_cap_and_alibi(sb, dev, kind, opt):
+    Hq, Hkv, bs, wl = 28, 4, 16, 150
+    lens = [1, 33, 150, 151, 400]
+    g = torch.Generator().manual_seed(5)
+    nblk = [(n + bs - 1) // bs for n in lens]
+    nb = sum(nblk) + 2
+    perm = torch.randperm(nb, generator=g)
+    tables = torch.zeros(len(lens), max(nblk), dtype=torch.int32)
+    p0 = 0
+    for r, n in enumerate(nblk):
+        tables[r, :n] = perm[p0:p0 + n]; p0 += n
+    T = sum(lens)
+    k = (torch.randn(T, Hkv, D, generator=g) * (0.5 + torch.rand(T, Hkv, 1, generator=g))).bfloat16()
+    v = torch.randn(T, Hkv, D, generator=g).bfloat16()
+    slots = torch.cat([torch.tensor([int(tables[r, i // bs]) * bs + i % bs for i in range(n)], dtype=torch.int64)
+                       for r, n in enumerate(lens)])
+    if kind == "int8":
+        kvc, sc = sb.ops.alloc_int8_kv_cache(nb, bs, Hkv, D, dev)
+        sb.ops.kv_append_int8(k.to(dev), v.to(dev), kvc[0], kvc[1], sc[0], sc[1], slots.to(dev))
+        kw = dict(k_scale=sc[0], v_scale=sc[1])
+        kd, vd = Q.quantize_sym(k.float().numpy(), "bf16"), Q.quantize_sym(v.float().numpy(), "bf16")
+    else:
+        kvc = torch.zeros(2, nb, bs, Hkv, D, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+        sb.ops.kv_append_fp8(k.to(dev), v.to(dev), kvc[0], kvc[1], slots.to(dev), 0.25, 0.5)
+        kw = dict(fp8_scales=(0.25, 0.5))
+        kd, vd = Q.fp8_round(k.float().numpy(), 0.25, "bf16"), Q.fp8_round(v.float().numpy(), 0.5, "bf16")
+    q = (2.0 * torch.randn(len(lens), Hq, D, generator=g)).bfloat16()
+    slopes = slopes_for(Hq) if opt["alibi"] else None
+    out = sb.ops.swa_decode_attention(
+        q.to(dev), kvc[0], kvc[1], torch.tensor(lens, dtype=torch.int32, device=dev), block_table=tables.to(dev),
+        window_left=wl, scale=D ** -0.5, n_split=2, softcap=opt["softcap"],
+        alibi_slopes=None if slopes is None else torch.tensor(slopes, device=dev), **kw)
+    # the oracle attends to the dequantised rows, laid out as one block per sequence
+    off = np.cumsum([0] + lens)
+    for r, n in enumerate(lens):
+        ref = A.paged_decode_attention(q[r:r + 1].float().numpy(), kd[off[r]:off[r + 1]][None], vd[off[r]:off[r + 1]][None],
+                                       np.zeros((1, 1), np.int32), [n], D ** -0.5, wl, softcap=opt["softcap"], alibi_slopes=slopes)
+        assert np.abs(out[r].float().cpu().numpy() - ref[0]).max() <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Hq,Hkv", [(28, 4), (6, 2), (5, 1)])
+@pytest.mark.parametrize("opt", OPTIONS)
+@pytest.mark.parametrize("paged", [False, True])
+def test_many_query_kernel_with_soft_cap_and_alibi(sb, dev, dtype, Hq, Hkv, opt, paged):
+    """Prompts and chunked prefill: query j of a sequence sits at key position Lk - Lq + j."""
+    wl, bs = 70, 16
+    query_lens = [1, 17, 64, 130] if not paged else [40, 3, 130, 1]
+    ctx = [0, 0, 0, 0] if not paged else [60, 0, 200, 33]
+    lens_k = [a + b for a, b in zip(query_lens, ctx)]
+    g = torch.Generator().manual_seed(Hq + (7 if paged else 0))
+    cu_q = np.cumsum([0] + query_lens); cu_k = np.cumsum([0] + lens_k)
+    q = (2.0 * torch.randn(int(cu_q[-1]), Hq, D, generator=g)).to(dtype)
+    k = torch.randn(int(cu_k[-1]), Hkv, D, generator=g).to(dtype)
+    v = torch.randn(int(cu_k[-1]), Hkv, D, generator=g).to(dtype)
+    slopes = slopes_for(Hq) if opt["alibi"] else None
+    kw = dict(softcap=opt["softcap"], alibi_slopes=None if slopes is None else torch.tensor(slopes, device=dev))
+    if paged:
+        need = [(n + bs - 1) // bs for n in lens_k]
+        nb = sum(need) + 3
+        perm = torch.randperm(nb, generator=g)
+        kc = torch.randn(nb, bs, Hkv, D, generator=g).to(dtype); vc = torch.randn(nb, bs, Hkv, D, generator=g).to(dtype)
+        tables = torch.zeros(len(lens_k), max(need), dtype=torch.int32)
+        p = 0
+        for s, n in enumerate(need):
+            tables[s, :n] = perm[p:p + n]; p += n
+            for i in range(lens_k[s]):
+                kc[int(tables[s, i // bs]), i % bs] = k[cu_k[s] + i]
+                vc[int(tables[s, i // bs]), i % bs] = v[cu_k[s] + i]
+        out = sb.ops.swa_prefill_attention(q.to(dev), kc.to(dev), vc.to(dev), query_lens=query_lens, seq_lens_k=lens_k,
+                                           block_table=tables.to(dev), window_left=wl, scale=D ** -0.5, **kw)
+    else:
+        out = sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), query_lens=query_lens, window_left=wl,
+                                           scale=D ** -0.5, **kw)
+    ref = A.varlen_window_attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), cu_q, cu_k, D ** -0.5, wl,
+                                    softcap=opt["softcap"], alibi_slopes=slopes)
+    assert np.abs(out.float().cpu().numpy() - ref).max() <= TOL[dtype]
+    plain = A.varlen_window_attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), cu_q, cu_k, D ** -0.5, wl)
+    assert np.abs(plain - ref).max() > 5 * TOL[dtype]
+
+
+def test_backend_passes_the_options_on_and_rejects_what_no_kernel_takes(sb, dev):
+    """MetaAttentionImpl(alibi_slopes=..., logits_soft_cap=...): a prompt step over the in-flight keys, then
+    decode steps through the paged cache, against the oracle with the same options."""
+    Hq, Hkv, bs, wl, nb = 28, 4, 16, 40, 32
+    slopes = slopes_for(Hq)
+    impl = sb.MetaAttentionImpl(Hq, D, D ** -0.5, Hkv, slopes, wl + 1, "auto", logits_soft_cap=2.5)
+    assert impl.logits_soft_cap == 2.5 and impl.alibi_slopes.shape == (Hq,)
+    runner = sb.runner.SwaCacheRunner(1, nb, bs, wl, Hkv, D, torch.bfloat16, dev, max_seqs=2, max_chunk_tokens=128)
+    g = torch.Generator().manual_seed(1)
+    hist_k = {0: [], 1: []}; hist_v = {0: [], 1: []}
+    for sid in (0, 1):
+        runner.add_seq(sid)
+
+    def step(prompts, decodes):
+        T = sum(n for _, n in prompts) + len(decodes)
+        q = (2.0 * torch.randn(T, Hq, D, generator=g)).bfloat16()
+        k = torch.randn(T, Hkv, D, generator=g).bfloat16(); v = torch.randn(T, Hkv, D, generator=g).bfloat16()
+        meta = runner.build_step(prompts, decodes)
+        out = torch.empty(T, Hq, D, dtype=torch.bfloat16, device=dev)
+        impl.forward(None, q.to(dev), k.to(dev), v.to(dev), None, None, None, runner.kv_caches[0], meta, output=out)
+        t = 0
+        for sid, n in prompts + [(d, 1) for d in decodes]:
+            hist_k[sid] += list(k[t:t + n].float().numpy()); hist_v[sid] += list(v[t:t + n].float().numpy())
+            L = len(hist_k[sid])
+            ref = A.varlen_window_attention(q[t:t + n].float().numpy(), np.stack(hist_k[sid]), np.stack(hist_v[sid]),
+                                            [0, n], [0, L], D ** -0.5, wl, softcap=2.5, alibi_slopes=slopes)
+            assert np.abs(out[t:t + n].float().cpu().numpy() - ref).max() <= 2e-2
+            t += n
+
+    step([(0, 30), (1, 75)], [])
+    for _ in range(20):
+        step([], [0, 1])
+    with pytest.raises(ValueError, match="one slope per query head"):
+        sb.MetaAttentionImpl(Hq, D, 1.0, Hkv, [0.5] * 3, wl + 1, "auto")
+    with pytest.raises(ValueError, match="logits_soft_cap"):
+        sb.MetaAttentionImpl(Hq, D, 1.0, Hkv, None, wl + 1, "auto", logits_soft_cap=-1.0)
+    # fp32 queries run on the vector-ALU kernel, which takes neither option: refused, not ignored
+    q32 = torch.randn(2, Hq, D, device=dev)
+    kv32 = torch.randn(2, 4, bs, Hkv, D, device=dev)
+    with pytest.raises(NotImplementedError, match="soft cap"):
+        sb.ops.swa_decode_attention(q32, kv32[0], kv32[1], torch.tensor([5, 9], dtype=torch.int32, device=dev),
+                                    block_table=torch.zeros(2, 2, dtype=torch.int32, device=dev), softcap=2.0)

@@ -121,6 +121,57 @@ def test_varlen_vs_torch_sdpa_and_decode_consistency():
             np.testing.assert_allclose(out[cu_q[s] + j], ref, rtol=1e-10, atol=1e-12)
 
 
+def test_soft_cap_and_alibi_vs_torch_and_limits():
+    """The two flash-attn options of the backend (meta_attention.py:665-690). ALiBi against torch SDPA with
+    the bias written out as an additive mask; the soft cap against its limits (a huge cap changes nothing,
+    a vanishing cap flattens the scores: the output is the mean of the visible V rows) and against the
+    formula evaluated by torch on explicit scores."""
+    B, Hq, Hkv, D, bs, wl = 3, 6, 2, 16, 16, 20
+    lens = [1, 30, 50]
+    kc, vc, tables = make_paged(B, lens, bs, Hkv, D, 12)
+    q = rng(13).standard_normal((B, Hq, D))
+    slopes = [2.0 ** -(i + 1) for i in range(Hq)]
+    G = Hq // Hkv
+    out = A.paged_decode_attention(q, kc, vc, tables, lens, 0.3, wl, alibi_slopes=slopes)
+    capped = A.paged_decode_attention(q, kc, vc, tables, lens, 0.3, wl, softcap=1.5)
+    both = A.paged_decode_attention(q, kc, vc, tables, lens, 0.3, wl, softcap=1.5, alibi_slopes=slopes)
+    for b, n in enumerate(lens):
+        kk = np.concatenate([kc[t] for t in tables[b]])[:n]
+        vv = np.concatenate([vc[t] for t in tables[b]])[:n]
+        i = np.arange(n)
+        vis = i >= n - 1 - wl
+        kr = torch.from_numpy(np.repeat(kk.transpose(1, 0, 2), G, 0))      # [Hq, n, D]
+        vr = torch.from_numpy(np.repeat(vv.transpose(1, 0, 2), G, 0))
+        dist = torch.from_numpy((n - 1 - i).astype(np.float64))
+        add = torch.where(torch.from_numpy(vis), 0.0, -torch.inf).double()[None, :] - torch.tensor(slopes).double()[:, None] * dist[None, :]
+        ref = F.scaled_dot_product_attention(torch.from_numpy(q[b])[None, :, None, :], kr[None], vr[None],
+                                             attn_mask=add[None, :, None, :], scale=0.3)[0, :, 0].numpy()
+        np.testing.assert_allclose(out[b], ref, rtol=1e-10, atol=1e-12)
+        sc = torch.einsum("hd,hnd->hn", torch.from_numpy(q[b]), kr) * 0.3
+        for cap, bias, got in ((1.5, 0.0, capped[b]), (1.5, 1.0, both[b])):
+            logits = cap * torch.tanh(sc / cap) - bias * torch.tensor(slopes).double()[:, None] * dist[None, :]
+            logits = torch.where(torch.from_numpy(vis)[None, :], logits, -torch.inf)
+            ref2 = torch.einsum("hn,hnd->hd", torch.softmax(logits, -1), vr).numpy()
+            np.testing.assert_allclose(got, ref2, rtol=1e-10, atol=1e-12)
+        flat = A.paged_decode_attention(q, kc, vc, tables, lens, 0.3, wl, softcap=1e-9)[b]
+        np.testing.assert_allclose(flat, np.repeat(vv[vis].mean(0), G, 0), rtol=1e-6)
+    np.testing.assert_allclose(A.paged_decode_attention(q, kc, vc, tables, lens, 0.3, wl, softcap=1e9),
+                               A.paged_decode_attention(q, kc, vc, tables, lens, 0.3, wl), rtol=1e-9)
+    # the varlen form: every query is a decode over the keys up to its own position, options included
+    cu_q = [0, 5, 9]; cu_k = [0, 5, 17]
+    r = rng(14)
+    qv = r.standard_normal((9, Hq, D)); kv = r.standard_normal((17, Hkv, D)); vv_ = r.standard_normal((17, Hkv, D))
+    got = A.varlen_window_attention(qv, kv, vv_, cu_q, cu_k, 0.4, 6, softcap=2.0, alibi_slopes=slopes)
+    for s_ in range(2):
+        Lq, Lk = cu_q[s_ + 1] - cu_q[s_], cu_k[s_ + 1] - cu_k[s_]
+        for j in range(Lq):
+            n = Lk - Lq + j + 1
+            kc1 = kv[cu_k[s_]:cu_k[s_] + n][None]; vc1 = vv_[cu_k[s_]:cu_k[s_] + n][None]   # one block of n rows
+            one = A.paged_decode_attention(qv[cu_q[s_] + j][None], kc1, vc1, np.zeros((1, 1), np.int32), [n], 0.4, 6,
+                                           softcap=2.0, alibi_slopes=slopes)
+            np.testing.assert_allclose(got[cu_q[s_] + j], one[0], rtol=1e-10, atol=1e-12)
+
+
 def test_lse_merge_equals_attention_over_union():
     D, nA, nB = 8, 5, 7
     r = rng(8)
