@@ -194,3 +194,74 @@ def test_prefill_argument_errors(sb, dev):
         sb.ops.swa_prefill_attention(q64, kv64, kv64, query_lens=[4])
     out = sb.ops.swa_prefill_attention(q[:0], kv, kv, query_lens=[])       # empty step
     assert out.shape == (0, 8, 128)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_vs_oracle(sb, dev, seed):
+    """Seeded random cases across what the kernel specialises on: GQA group (1..9: launches of 4, 3, 2 and 1 heads,
+    double- and single-block wavefronts), dtype, paged (block sizes 16/32/48/64/128, shuffled tables, garbage in
+    stale rows) or in-flight keys, window, ragged query and context lengths around the 16/32/64 boundaries,
+    optional meta rows, optional soft cap / ALiBi."""
+    r = np.random.default_rng(1000 + seed)
+    D = 128
+    Hkv = int(r.choice([1, 2, 4]))
+    G = int(r.integers(1, 10))
+    Hq = Hkv * G
+    dtype = torch.bfloat16 if r.random() < 0.7 else torch.float16
+    S = int(r.integers(1, 6))
+    query_lens = [int(r.choice([1, 2, 15, 16, 17, 31, 33, 63, 64, 65, 100, 129, 200])) for _ in range(S)]
+    paged = r.random() < 0.6
+    ctx = [int(r.choice([0, 1, 31, 32, 77, 300])) if paged else 0 for _ in range(S)]
+    wl = int(r.choice([-1, 0, 5, 31, 32, 63, 64, 100, 257]))
+    use_meta = r.random() < 0.25
+    use_opts = (not use_meta) and r.random() < 0.3
+    q, k, v, lens_k, cu_q, cu_k = dense_problem(query_lens, ctx, Hq, Hkv, D, dtype, seed=seed, spread=1.5 if use_opts else 1.0)
+    g = torch.Generator().manual_seed(seed)
+    kw = {}
+    slopes = None
+    softcap = 0.0
+    if use_opts:
+        slopes = [float(2.0 ** (-8.0 * (h + 1) / Hq)) for h in range(Hq)]
+        softcap = 2.0
+        kw.update(softcap=softcap, alibi_slopes=torch.tensor(slopes, device=dev))
+    M = 0
+    if use_meta:
+        M = int(r.choice([1, 31, 32, 100]))
+        mk = torch.randn(M, Hkv, D, generator=g).to(dtype); mv = torch.randn(M, Hkv, D, generator=g).to(dtype)
+        kw.update(meta_k=mk.to(dev), meta_v=mv.to(dev))
+    scale = D ** -0.5
+    if paged:
+        bs = int(r.choice([16, 32, 48, 64, 128]))
+        need = [(n + bs - 1) // bs for n in lens_k]
+        nb = sum(need) + 2
+        perm = torch.randperm(nb, generator=g)
+        kc = torch.randn(nb, bs, Hkv, D, generator=g).to(dtype); vc = torch.randn(nb, bs, Hkv, D, generator=g).to(dtype)
+        tables = torch.zeros(S, max(need), dtype=torch.int32)
+        p = 0
+        for s, n in enumerate(need):
+            tables[s, :n] = perm[p:p + n]; p += n
+            for i in range(lens_k[s]):
+                kc[int(tables[s, i // bs]), i % bs] = k[cu_k[s] + i]
+                vc[int(tables[s, i // bs]), i % bs] = v[cu_k[s] + i]
+        out = sb.ops.swa_prefill_attention(q.to(dev), kc.to(dev), vc.to(dev), query_lens=query_lens, seq_lens_k=lens_k,
+                                           block_table=tables.to(dev), window_left=wl, scale=scale, **kw)
+    else:
+        out = sb.ops.swa_prefill_attention(q.to(dev), k.to(dev), v.to(dev), query_lens=query_lens, window_left=wl,
+                                           scale=scale, **kw)
+    qn, kn, vn = q.float().numpy(), k.float().numpy(), v.float().numpy()
+    if use_meta:   # one softmax over [meta rows | window]: the oracle's merged form, query by query
+        ref = np.zeros((qn.shape[0], Hq, D))
+        for s in range(S):
+            Lq, Lk = query_lens[s], lens_k[s]
+            for j in range(Lq):
+                pos = Lk - Lq + j
+                lo = 0 if wl < 0 else max(0, pos - wl)
+                for h in range(Hq):
+                    kk = np.concatenate([mk.float().numpy()[:, h // G], kn[cu_k[s] + lo:cu_k[s] + pos + 1, h // G]])
+                    vv = np.concatenate([mv.float().numpy()[:, h // G], vn[cu_k[s] + lo:cu_k[s] + pos + 1, h // G]])
+                    ref[cu_q[s] + j, h] = A.masked_softmax_attention(qn[cu_q[s] + j, h][None], kk, vv,
+                                                                     np.zeros((1, len(kk)), bool), scale)[0]
+    else:
+        ref = A.varlen_window_attention(qn, kn, vn, cu_q, cu_k, scale, wl, softcap=softcap, alibi_slopes=slopes)
+    err = np.abs(out.float().cpu().numpy() - ref).max()
+    assert err <= TOL[dtype], (err, dict(Hq=Hq, Hkv=Hkv, dtype=dtype, query_lens=query_lens, ctx=ctx, wl=wl, paged=paged, M=M, opts=use_opts))
