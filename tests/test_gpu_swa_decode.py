@@ -388,3 +388,101 @@ def test_merge_inside_the_split_kernel_many_launches_back_to_back(sb, dev):
     torch.cuda.synchronize()
     for i, o in enumerate(got):
         assert torch.equal(o, want[i % 4]), f"launch {i}"
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_shapes_vs_oracle(sb, dev, seed):
+    """Seeded random cases across what the decode kernels specialise on: GQA group (1..16 on the matrix cores),
+    dtype, block size, window, split count and kind (fixed / balanced / merged inside the kernel), prefetch
+    depth, ragged lengths around the 16/32-key boundaries (empty rows included), key_lo, several query rows per
+    sequence, the fused append, meta rows, soft cap / ALiBi. Stale cache rows hold NaN."""
+    r = np.random.default_rng(2000 + seed)
+    D = 128
+    Hkv = int(r.choice([1, 2, 4]))
+    G = int(r.integers(1, 17))
+    Hq = Hkv * G
+    dtype = torch.bfloat16 if r.random() < 0.7 else torch.float16
+    bs = int(r.choice([16, 32, 48, 64, 128]))
+    wl = int(r.choice([-1, 0, 7, 31, 32, 100, 257, 1000]))
+    B = int(r.integers(1, 9))
+    lens = [int(r.choice([0, 1, 15, 16, 17, 31, 32, 33, 64, 100, 129, 300, 700])) for _ in range(B)]
+    n_split = int(r.choice([0, 1, 2, 3, 5]))
+    mode = r.choice(["fixed", "balanced", "merge_in_kernel", "fused", "meta", "options", "rows"])
+    g = torch.Generator().manual_seed(seed)
+    need = [(n + bs - 1) // bs for n in lens]
+    nb = sum(need) + 2
+    perm = torch.randperm(nb, generator=g)
+    kc = torch.full((nb, bs, Hkv, D), float("nan")).to(dtype); vc = torch.full((nb, bs, Hkv, D), float("nan")).to(dtype)
+    tables = torch.zeros(B, max(max(need), 1), dtype=torch.int32)
+    ks, vs = [], []
+    p = 0
+    for b, n in enumerate(need):
+        tables[b, :n] = perm[p:p + n]; p += n
+        k = torch.randn(lens[b], Hkv, D, generator=g).to(dtype); v = torch.randn(lens[b], Hkv, D, generator=g).to(dtype)
+        ks.append(k); vs.append(v)
+        for i in range(lens[b]):
+            kc[int(tables[b, i // bs]), i % bs] = k[i]; vc[int(tables[b, i // bs]), i % bs] = v[i]
+    scale = D ** -0.5
+    kw = dict(n_split=n_split, pipeline_depth=int(r.choice([0, 1, 2, 3])))
+    rows = list(range(B))                      # sequence of each query row
+    row_len = list(lens)                       # keys visible to each row
+    key_lo = None
+    slopes, softcap, meta = None, 0.0, None
+    if mode == "balanced":
+        kw["balanced"] = True
+    elif mode == "merge_in_kernel":
+        kw.update(balanced=False, merge_in_kernel=True)
+    elif mode == "options":
+        slopes = [float(2.0 ** (-8.0 * (h + 1) / Hq)) for h in range(Hq)]
+        softcap = float(r.choice([0.0, 2.0]))
+        kw.update(softcap=softcap, alibi_slopes=torch.tensor(slopes, device=dev))
+    elif mode == "meta":
+        M = int(r.choice([1, 32, 100]))
+        meta = (torch.randn(M, Hkv, D, generator=g).to(dtype), torch.randn(M, Hkv, D, generator=g).to(dtype))
+        kw.update(meta_k=meta[0].to(dev), meta_v=meta[1].to(dev), balanced=False)
+    elif mode == "rows":                       # several rows per sequence, each with its own length and key_lo
+        rows = [int(r.integers(0, B)) for _ in range(B + 3)]
+        row_len = [int(r.integers(0, lens[s] + 1)) for s in rows]
+        key_lo = [int(r.integers(0, 40)) if r.random() < 0.5 else 0 for _ in rows]
+        kw.update(row_seq=torch.tensor(rows, dtype=torch.int32, device=dev),
+                  key_lo=torch.tensor(key_lo, dtype=torch.int32, device=dev), max_seq_len=max(lens + [1]))
+    R = len(rows)
+    q = torch.randn(R, Hq, D, generator=g).to(dtype)
+    kc_d, vc_d = kc.to(dev), vc.to(dev)
+    if mode == "fused":                        # the newest key of every non-empty row arrives with the call
+        newk = torch.zeros(B, Hkv, D, dtype=dtype); newv = torch.zeros(B, Hkv, D, dtype=dtype)
+        slots = torch.full((B,), -1, dtype=torch.int64)
+        for b, n in enumerate(lens):
+            if n > 0:
+                newk[b], newv[b] = ks[b][n - 1], vs[b][n - 1]
+                blk, off = int(tables[b, (n - 1) // bs]), (n - 1) % bs
+                slots[b] = blk * bs + off
+                kc_d[blk, off] = float("nan"); vc_d[blk, off] = float("nan")
+        kw.update(new_key=newk.to(dev), new_value=newv.to(dev), new_slot_mapping=slots.to(dev))
+        if min(lens) == 0:                     # (a row without keys has no newest key to append)
+            pytest.skip("fused append needs a key in every row")
+    out = sb.ops.swa_decode_attention(q.to(dev), kc_d, vc_d, torch.tensor(row_len, dtype=torch.int32, device=dev),
+                                      block_table=tables.to(dev), window_left=wl, scale=scale, **kw).float().cpu().numpy()
+    assert np.isfinite(out).all()
+    for i, s in enumerate(rows):
+        n = row_len[i]
+        lo = max(0 if wl < 0 else max(0, n - 1 - wl), key_lo[i] if key_lo else 0)
+        kk, vv = ks[s][lo:n].float().numpy(), vs[s][lo:n].float().numpy()
+        for h in range(Hq):
+            kh, vh = kk[:, h // G], vv[:, h // G]
+            bias = None
+            if slopes is not None:
+                bias = -slopes[h] * (n - 1 - np.arange(lo, n))[None]
+            if meta is not None:
+                kh = np.concatenate([meta[0].float().numpy()[:, h // G], kh]); vh = np.concatenate([meta[1].float().numpy()[:, h // G], vh])
+            if len(kh) == 0:
+                assert (out[i, h] == 0).all()
+                continue
+            ref = A.masked_softmax_attention(q[i, h].float().numpy()[None], kh, vh, np.zeros((1, len(kh)), bool), scale,
+                                             softcap=softcap, bias=bias)[0]
+            err = np.abs(out[i, h] - ref).max()
+            assert err <= TOL[dtype], (err, dict(seed=seed, mode=str(mode), Hq=Hq, Hkv=Hkv, bs=bs, wl=wl, lens=lens, n_split=n_split))
+    if mode == "fused":                        # and the cache now holds them
+        for b, n in enumerate(lens):
+            blk, off = int(tables[b, (n - 1) // bs]), (n - 1) % bs
+            assert torch.equal(kc_d[blk, off].cpu(), ks[b][n - 1]) and torch.equal(vc_d[blk, off].cpu(), vs[b][n - 1])
