@@ -16,6 +16,10 @@ this path, so nothing here is pinned by a reference fixture):
                               routine) on the gathered dense K/V; single-key and constant-V
                               special cases; block-table permutation invariance; split merge
                               == attention over the union (tests/test_oracle_attention.py)
+  attention.* softcap / alibi_slopes   torch SDPA with the ALiBi term written out as an additive
+                              mask; the cap's formula evaluated by torch on explicit scores and its
+                              two limits (huge cap = none, vanishing cap = mean of the visible V
+                              rows); varlen form == decode per query (tests/test_oracle_attention.py)
   gla.*                       closed form S_T = sum_t diag(exp(sum_{u>t} g_u)) k_t^T v_t in
                               float64; g=0, k=0 and q=e_i special cases; slot -1 no-op
                               (tests/test_oracle_gla.py)
