@@ -467,26 +467,47 @@ def main():
         attend(c, 0, profile_events=events, **kw)
 
     n_split = args.n_split or sb._native.lib().sb_swa_decode_auto_split(prob["B"], HKV, prob["max_seq_len"], WL)
-    # ONE timed region: the split kernel of every 16th step carries a pair of HIP events on its own dispatch,
-    # on the stream it is launched on (torch's current stream), so the kernel time and the step time come
-    # from the same K steps. Not every step: a launch that carries events delays the launch behind it by about
-    # 6 us on this runtime (94.4 against 88.0 us per step with events on all of them), which would be charged
-    # to `value`; the kernel's own interval is not affected.
+    # How the step is timed.
+    #  * ramp: whatever --warmup says, RAMP_STEPS more untimed steps (>= 50 ms of the same GPU work) run right
+    #    before the timed region, so the clocks are where a serving loop holds them (the CPU baseline and the
+    #    set-up leave the GPU idle for seconds).
+    #  * the timed region is `steps` steps, back to back, with nothing else in the stream: no events ride on its
+    #    launches. It runs REGIONS times in a row; each run is timed by one pair of HIP events recorded on the
+    #    stream around it (the start marker delays the first of its launches by a few us: charged to the
+    #    region) and, independently, by the host clock from the first launch to the end of synchronize(). The
+    #    line reports the median region of the event timing; the host-clock median is given beside it.
+    #  * the split kernel's own duration comes from a separate pass right after: KERNEL_SAMPLES steps whose
+    #    split kernel carries a pair of HIP events on its own dispatch (hipExtLaunchKernel; the
+    #    profile_*_event fields of sb_swa_decode_args). Such a launch delays the one behind it by about 6 us,
+    #    which is why the pass is kept out of the timed region; the kernel's own interval is not affected.
+    RAMP_STEPS, REGIONS, KERNEL_SAMPLES = 640, 11, 64
     timed = not args.force_valu
-    EVERY = 16
-    evs = [sb.ops.timing_events(dev) for _ in range((args.steps + EVERY - 1) // EVERY)] if timed else []
     for i in range(args.warmup):
-        step(i, evs[0] if timed and i % EVERY == 0 else None)
+        step(i)
+    for i in range(RAMP_STEPS):
+        step(i)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i, evs[i // EVERY] if timed and i % EVERY == 0 else None)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    region_ev, region_host = [], []
+    marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(REGIONS)]
+    for a, b in marks:
+        t0 = time.perf_counter()
+        a.record()
+        for i in range(args.steps):
+            step(i)
+        b.record()
+        torch.cuda.synchronize()
+        region_host.append(time.perf_counter() - t0)
+        region_ev.append(a.elapsed_time(b) * 1e-3)
+    wall = statistics.median(region_ev)
     ms_per_step = wall / args.steps * 1e3
     value = prob["bytes_step"] / (wall / args.steps) / 1e9
-    if not timed:  # the vector-ALU comparison kernel has no timed launch: bracket its launches in a loop of their own
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    if timed:
+        evs = [sb.ops.timing_events(dev) for _ in range(KERNEL_SAMPLES)]
+        for i, pair in enumerate(evs):
+            step(i, pair)
+        torch.cuda.synchronize()
+    else:  # the vector-ALU comparison kernel has no timed launch: bracket its launches in a loop of their own
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(KERNEL_SAMPLES)]
         for i, (a, b) in enumerate(evs):
             a.record()
             attend(kv[i % n_copies], 1, **({} if args.unfused else new_kv))
@@ -507,12 +528,17 @@ def main():
                    "batch": prob["B"], "q_heads": HQ, "kv_heads": HKV, "head_dim": D, "block_size": BS,
                    "window_left": WL, "context_lens": "U[1024,32768] seed 0", "n_split": int(n_split),
                    "kv_cache_copies_rotated": n_copies, "bytes_per_step": prob["bytes_step"]},
+        "timing": {"ramp_steps": RAMP_STEPS, "regions": REGIONS, "region": f"{args.steps} steps back to back, no events on its launches",
+                   "reported": "median region, one HIP event pair on the stream around each region",
+                   "ms_per_step_regions_events": [round(t / args.steps * 1e3, 4) for t in region_ev],
+                   "ms_per_step_median_host_clock": round(statistics.median(region_host) / args.steps * 1e3, 4)},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "decode_tok_per_s_layer_step": round(prob["B"] / (wall / args.steps), 1),
         "roofline": {"bound": "hbm", "kernel": "swa_decode_split_kernel<BF16,7> (vector ALU)" if args.force_valu else "swa_decode_split_mfma_kernel<BF16>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_source": traffic_source, "kernel_ms": round(k_ms, 4),
-                     "kernel_ms_measured": f"HIP events on the kernel's own dispatch, every {EVERY}th launch of the timed region ({len(evs)} samples)" if timed
+                     "kernel_ms_measured": f"HIP events on the kernel's own dispatch, mean of {len(evs)} consecutive steps run right after the "
+                                           "timed region (an event-carrying launch delays the next one by ~6 us, the kernel's own interval is unaffected)" if timed
                      else "HIP events around the launches of a second loop (kernel + dispatch latency)",
                      "bytes_per_launch": prob["bytes_split_kernel"]},
     }

@@ -296,7 +296,13 @@ typedef struct sb_gla_recurrent_args {
   /* SB_GLA_* bits. Calls of 32 steps or more, and every packed call, with bf16 q/k/v run the
    * recurrence 16 tokens at a time on the matrix cores (its exact block form; fp32 state, gate
    * scan and accumulation; bf16 operand rounding on the output path as in any bf16 GEMM).
-   * SB_GLA_VECTOR_ONLY keeps such calls on the step-by-step fp32 kernel. */
+   * SB_GLA_VECTOR_ONLY keeps such calls on the step-by-step fp32 kernel.
+   * Gate range of the block form: inside a pair of blocks it forms exp(-(g_1 + .. + g_s)) per key dim, with
+   * the exponent clamped at 80, so it is exact only while the gates of any 32 consecutive tokens sum to
+   * more than -80 per key dim (|g| up to 2.5 per token, sustained; the model's log-sigmoid(x) / 16 gates
+   * reach that only for x < -40). Beyond it near-diagonal q.k terms are under-weighted without an error;
+   * callers whose gates can be that negative set SB_GLA_VECTOR_ONLY, which has no such limit (fla's
+   * fused_chunk_gla, which this path replaces, divides by the same cumulative decays inside its chunks). */
   int32_t flags;
   /* Shared states, 0 or 1 = off. The reference computes k, v and the gate for the 4 kv heads and
    * repeats them to the 28 query heads (hf_7B_model/gla_attention.py:147-149,

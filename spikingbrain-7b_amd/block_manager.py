@@ -175,16 +175,15 @@ class WindowBlockManager:
         return int(self._stack[self._top])
 
     # -- one engine step ------------------------------------------------------------
-    def _advance_row(self, r: int, count: int, is_prompt: bool, store_all: bool = False) -> Tuple[int, int]:
-        """Evict + allocate for `count` new tokens of row r; returns (p0, first stored position)."""
+    def _plan_row(self, r: int, count: int, is_prompt: bool, store_all: bool = False):
+        """What `count` new tokens of row r evict and allocate, without touching any state (raises on a
+        ring overflow): (p0, first stored position, n_evict, lo, hi after eviction, j0, n_new, new lo, new hi)."""
         bs, wl, R = self.block_size, self.window_left, self.ring_blocks
         p0 = int(self.n_tokens[r])
         lo_new = max(0, (p0 - wl) // bs)
         lo, hi = int(self.lo[r]), int(self.hi[r])
-        n_evict = min(lo_new, hi + 1) - lo
-        if n_evict > 0:  # pushed in order of logical block, as one slice
-            self._stack[self._top:self._top + n_evict] = self.ring[r, np.arange(lo, lo + n_evict) % R]
-            self._top += n_evict
+        ev_lo = lo
+        n_evict = max(0, min(lo_new, hi + 1) - lo)
         if hi >= lo:
             lo = max(lo, lo_new)
             if lo > hi:  # everything evicted
@@ -192,6 +191,7 @@ class WindowBlockManager:
         start_idx = compute_slot_mapping_start_idx(is_prompt, count, p0, None if store_all else wl)
         first = max(p0, start_idx)
         end = p0 + count
+        j0 = n_new = 0
         if end > first:
             jb, je = first // bs, (end - 1) // bs
             if hi < lo:
@@ -199,16 +199,32 @@ class WindowBlockManager:
             if je - lo + 1 > R:
                 raise RuntimeError(f"{je - lo + 1} resident blocks exceed the ring of {R}; raise max_chunk_tokens")
             j0 = max(jb, hi + 1)
-            n_new = je + 1 - j0
-            if n_new > 0:  # popped one after the other from the top of the stack, as one reversed slice
-                if n_new > self._top:
-                    raise RuntimeError("out of KV cache blocks")
-                self.ring[r, np.arange(j0, je + 1) % R] = self._stack[self._top - n_new:self._top][::-1]
-                self._top -= n_new
+            n_new = max(0, je + 1 - j0)
             hi = max(hi, je)
+        return p0, first, ev_lo, n_evict, j0, n_new, lo, hi, end
+
+    def _apply_plan(self, r: int, plan) -> Tuple[int, int]:
+        """Carries a plan of `_plan_row` out; the caller has checked that the free stack covers it."""
+        R = self.ring_blocks
+        p0, first, ev_lo, n_evict, j0, n_new, lo, hi, end = plan
+        if n_evict > 0:  # pushed in order of logical block, as one slice
+            self._stack[self._top:self._top + n_evict] = self.ring[r, np.arange(ev_lo, ev_lo + n_evict) % R]
+            self._top += n_evict
+        if n_new > 0:  # popped one after the other from the top of the stack, as one reversed slice
+            self.ring[r, np.arange(j0, j0 + n_new) % R] = self._stack[self._top - n_new:self._top][::-1]
+            self._top -= n_new
         self.lo[r], self.hi[r] = lo, hi
         self.n_tokens[r] = end
         return p0, first
+
+    def _advance_row(self, r: int, count: int, is_prompt: bool, store_all: bool = False) -> Tuple[int, int]:
+        """Evict + allocate for `count` new tokens of row r; returns (p0, first stored position).
+        All or nothing: when the blocks do not suffice (or the ring would overflow) it raises with the
+        row, the ring and the free stack exactly as they were, so the caller may free sequences and retry."""
+        plan = self._plan_row(r, count, is_prompt, store_all)
+        if plan[5] > self._top + plan[3]:
+            raise RuntimeError("out of KV cache blocks")
+        return self._apply_plan(r, plan)
 
     def append_tokens(self, seq_id, count: int, is_prompt: bool, store_all: bool = False,
                       want_slots: bool = True) -> List[int]:
@@ -231,8 +247,18 @@ class WindowBlockManager:
         p = self.n_tokens[rows]
         need_evict = (np.maximum(0, (p - wl) // bs) > self.lo[rows]) & (self.hi[rows] >= self.lo[rows])
         need_alloc = (p // bs) > self.hi[rows]
-        for i in np.nonzero(need_evict | need_alloc)[0]:
-            self._advance_row(int(rows[i]), 1, False)
+        # all or nothing over the batch: plan every row that evicts or allocates, replay the free count in
+        # batch-row order, and only then touch anything
+        busy = [int(rows[i]) for i in np.nonzero(need_evict | need_alloc)[0]]
+        plans = [self._plan_row(r, 1, False) for r in busy]
+        top = self._top
+        for plan in plans:
+            top += plan[3]
+            if plan[5] > top:
+                raise RuntimeError("out of KV cache blocks")
+            top -= plan[5]
+        for r, plan in zip(busy, plans):
+            self._apply_plan(r, plan)
         quiet = ~(need_evict | need_alloc)
         self.n_tokens[rows[quiet]] += 1
         return self.ring[rows, (p // bs) % R].astype(np.int64) * bs + p % bs

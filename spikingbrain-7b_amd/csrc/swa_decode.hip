@@ -704,41 +704,6 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
                (a->out_stride_head * esz) % 16))
     return fail(SB_ERR_INVALID, "sb_swa_decode: out rows must be 16-byte aligned");
 
-  // optional fused append of the step's newest key/value row
-  p.new_k = p.new_v = nullptr;
-  p.slot_mapping = nullptr;
-  p.nk_st = p.nk_sh = p.nv_st = p.nv_sh = 0;
-  const bool want_append = a->new_key || a->new_value || a->new_slot_mapping;
-  if (want_append) {
-    if (!a->new_key || !a->new_value || !a->new_slot_mapping)
-      return fail(SB_ERR_INVALID, "sb_swa_decode: new_key, new_value and new_slot_mapping go together");
-    if (!a->block_table || a->row_seq)
-      return fail(SB_ERR_INVALID, "sb_swa_decode: fused append needs paged mode and one query row per sequence");
-    if (((reinterpret_cast<uintptr_t>(a->new_key) | reinterpret_cast<uintptr_t>(a->new_value)) & 15u) ||
-        (a->new_key_stride_row * esz) % 16 || (a->new_key_stride_head * esz) % 16 ||
-        (a->new_value_stride_row * esz) % 16 || (a->new_value_stride_head * esz) % 16)
-      return fail(SB_ERR_INVALID, "sb_swa_decode: new key/value rows must be 16-byte aligned");
-    if (mfma && a->phases != 2) {
-      p.new_k = (const char *)a->new_key; p.new_v = (const char *)a->new_value;
-      p.slot_mapping = a->new_slot_mapping;
-      p.nk_st = a->new_key_stride_row * esz; p.nk_sh = a->new_key_stride_head * esz;
-      p.nv_st = a->new_value_stride_row * esz; p.nv_sh = a->new_value_stride_head * esz;
-    } else if (a->phases != 2) {
-      // vector-ALU path: same semantics as two launches
-      sb_kv_append_args ap;
-      ap.key = a->new_key; ap.value = a->new_value;
-      ap.k_cache = const_cast<void *>(a->k_cache); ap.v_cache = const_cast<void *>(a->v_cache);
-      ap.slot_mapping = a->new_slot_mapping; ap.num_tokens = a->num_rows;
-      ap.num_kv_heads = a->num_kv_heads; ap.head_size = a->head_size; ap.block_size = a->block_size;
-      ap.dtype = a->dtype;
-      ap.key_stride_token = a->new_key_stride_row; ap.key_stride_head = a->new_key_stride_head;
-      ap.value_stride_token = a->new_value_stride_row; ap.value_stride_head = a->new_value_stride_head;
-      ap.cache_stride_block = a->kv_stride_block; ap.cache_stride_row = a->kv_stride_row;
-      ap.cache_stride_head = a->kv_stride_head; ap.num_blocks = 0; ap.stream = a->stream;
-      const int arc = sb_kv_append(&ap);
-      if (arc != SB_OK) return arc;
-    }
-  }
   // optional meta tokens: shared rows every query also attends to, inside the same softmax
   p.meta_k = p.meta_v = nullptr;
   p.meta_len = 0;
@@ -779,6 +744,42 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
       p.opt.inv_cap2_log2e = 2.f * sb::kLog2e / a->softcap;
     }
   }
+  // (every rejection above happens before the first launch: the append below may already write the cache)
+  // optional fused append of the step's newest key/value row
+  p.new_k = p.new_v = nullptr;
+  p.slot_mapping = nullptr;
+  p.nk_st = p.nk_sh = p.nv_st = p.nv_sh = 0;
+  const bool want_append = a->new_key || a->new_value || a->new_slot_mapping;
+  if (want_append) {
+    if (!a->new_key || !a->new_value || !a->new_slot_mapping)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: new_key, new_value and new_slot_mapping go together");
+    if (!a->block_table || a->row_seq)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: fused append needs paged mode and one query row per sequence");
+    if (((reinterpret_cast<uintptr_t>(a->new_key) | reinterpret_cast<uintptr_t>(a->new_value)) & 15u) ||
+        (a->new_key_stride_row * esz) % 16 || (a->new_key_stride_head * esz) % 16 ||
+        (a->new_value_stride_row * esz) % 16 || (a->new_value_stride_head * esz) % 16)
+      return fail(SB_ERR_INVALID, "sb_swa_decode: new key/value rows must be 16-byte aligned");
+    if (mfma && a->phases != 2) {
+      p.new_k = (const char *)a->new_key; p.new_v = (const char *)a->new_value;
+      p.slot_mapping = a->new_slot_mapping;
+      p.nk_st = a->new_key_stride_row * esz; p.nk_sh = a->new_key_stride_head * esz;
+      p.nv_st = a->new_value_stride_row * esz; p.nv_sh = a->new_value_stride_head * esz;
+    } else if (a->phases != 2) {
+      // vector-ALU path: same semantics as two launches
+      sb_kv_append_args ap;
+      ap.key = a->new_key; ap.value = a->new_value;
+      ap.k_cache = const_cast<void *>(a->k_cache); ap.v_cache = const_cast<void *>(a->v_cache);
+      ap.slot_mapping = a->new_slot_mapping; ap.num_tokens = a->num_rows;
+      ap.num_kv_heads = a->num_kv_heads; ap.head_size = a->head_size; ap.block_size = a->block_size;
+      ap.dtype = a->dtype;
+      ap.key_stride_token = a->new_key_stride_row; ap.key_stride_head = a->new_key_stride_head;
+      ap.value_stride_token = a->new_value_stride_row; ap.value_stride_head = a->new_value_stride_head;
+      ap.cache_stride_block = a->kv_stride_block; ap.cache_stride_row = a->kv_stride_row;
+      ap.cache_stride_head = a->kv_stride_head; ap.num_blocks = 0; ap.stream = a->stream;
+      const int arc = sb_kv_append(&ap);
+      if (arc != SB_OK) return arc;
+    }
+  }
   if (mfma && !int8_kv && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
     p.n_wg = (int)balanced_workgroups(a->num_rows, n_split);
   // On request the fixed split of the matrix-core kernel merges in the same launch (the last wavefront of a
@@ -795,7 +796,7 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
     else if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
     else if (a->dtype == SB_F16) rc = launch_for_group<F16>(G, grid, st, p);
     else rc = launch_for_group<F32>(G, grid, st, p);
-    rc = check_launch("swa_decode_split_kernel");
+    if (rc == SB_OK) rc = check_launch("swa_decode_split_kernel");
   }
   if (rc != SB_OK || n_split == 1 || a->phases == 1 || p.merge_counter) return rc;
 

@@ -457,7 +457,12 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
   // rows either. The variant is therefore opt-in (SB_DECODE_MERGE_IN_KERNEL); it is an instantiation of its
   // own so that its 160 extra live registers do not weigh on the default kernel.
   if constexpr (kMergeHere) if (!direct && p.merge_counter != nullptr) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt vmcnt(0): this wavefront's partial is in the L2
+    // this wavefront's partial stores must have been acknowledged by the L2 before the counter moves: an
+    // explicit wait (a workgroup-scope release fence alone need not wait for vector stores), with the fence
+    // kept as a barrier for the compiler's own reordering
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), expcnt and lgkmcnt left alone (gfx9 encoding)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     int *counter = p.merge_counter + r * p.Hkv + kvh;
     const int xcc = (int)__builtin_amdgcn_s_getreg(20 | (3 << 11));  // HW_REG_XCC_ID, bits 3:0
     int arrived = 0;

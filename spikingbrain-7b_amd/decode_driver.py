@@ -147,10 +147,22 @@ class HybridDecodeCache:
             run_layers(meta)
         torch.cuda.current_stream(self.device).wait_stream(side)
         graph = torch.cuda.CUDAGraph()
+        before = set(ops.graph_workspace_ids(self.device))
         with torch.cuda.graph(graph):
             self.advance_device()
             run_layers(meta)
+        # split-K workspaces this capture allocated belong to the graph: `release_step_graph` frees them
+        graph.sb_workspace_ids = [c for c in ops.graph_workspace_ids(self.device) if c not in before]
         return graph
+
+    def release_step_graph(self, graph) -> int:
+        """Call when a graph from `capture_step` is dropped (re-capture for another batch size): hands the
+        split-K workspaces it owned back to the allocator. The graph must not be replayed afterwards."""
+        freed = 0
+        for cid in getattr(graph, "sb_workspace_ids", []):
+            freed += ops.release_graph_workspace(cid, self.device)
+        graph.sb_workspace_ids = []
+        return freed
 
     def gla_layer(self, layer_idx: int, q, k, v, g, out=None) -> torch.Tensor:
         """q [B, H, 1, D]; k, v, g [B, H, 1, D], or [B, Hkv, 1, D] with shared states; the layer's state is

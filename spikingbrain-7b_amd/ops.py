@@ -14,8 +14,9 @@ PAD_SLOT_ID = -1
 
 # Split-K scratch of the decode kernel. Outside stream capture: one buffer per (device, stream), grown on
 # demand (calls on one stream are ordered, so they can share it; calls on different streams must not).
-# Under stream capture: one buffer per capture, kept for the life of the process. A captured graph replays
-# into the addresses recorded at capture time, so such a buffer must never be replaced, shrunk or handed
+# Under stream capture: one buffer per capture, kept until `release_graph_workspace` is told that the graph
+# is gone (an engine that re-captures per batch size calls it when it drops the old graph). A captured graph
+# replays into the addresses recorded at capture time, so such a buffer must never be replaced, shrunk or handed
 # back to the allocator by a later, larger request (the allocator could give the block to another tensor
 # while every replay still writes and merges partials there).
 _workspaces: Dict[Tuple[torch.device, int], torch.Tensor] = {}
@@ -29,22 +30,49 @@ def _capture_id(dev: torch.device) -> int:
     return cid.value
 
 
+_COUNTER_BYTES = 64 << 10   # arrival counters of the in-kernel merge at the head of a workspace: zero between launches
+
+
+def _new_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+    ws[:_COUNTER_BYTES].zero_()   # only the counters need a known start; partials are written before they are read
+    return ws
+
+
 def _workspace(dev: torch.device, nbytes: int) -> Optional[torch.Tensor]:
     if nbytes == 0:
         return None
     cap = _capture_id(dev)
     if cap:
+        # (allocated inside the capture: the 64 KiB counter fill becomes a node of the graph and runs at every
+        # replay, which is harmless: the counters are zero between launches anyway)
         owned = _graph_workspaces.setdefault((dev, cap), [])
         if not owned or owned[-1].numel() < nbytes:
             # (a smaller buffer handed out earlier in this capture stays in the list: earlier nodes use it)
-            owned.append(torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev))
+            owned.append(_new_workspace(dev, nbytes))
         return owned[-1]
     key = (dev, N.stream_ptr(dev))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)   # (its merge counters start at zero)
+        ws = _new_workspace(dev, nbytes)
         _workspaces[key] = ws
     return ws
+
+
+def graph_workspace_ids(device=None):
+    """Capture ids that still own split-K workspaces (one id per stream capture that ran a split decode call)."""
+    return sorted(c for d, c in _graph_workspaces if device is None or d == torch.device(device))
+
+
+def release_graph_workspace(capture_id: Optional[int] = None, device=None) -> int:
+    """Drop the workspaces captured graphs own: those of one capture (`capture_id`, from
+    `graph_workspace_ids()`), or all of them. Call it when the graph is destroyed, never while it may still be
+    replayed: every replay writes its partial results there. Returns the bytes handed back to the allocator."""
+    freed = 0
+    for key in [k for k in _graph_workspaces
+                if (capture_id is None or k[1] == capture_id) and (device is None or k[0] == torch.device(device))]:
+        freed += sum(t.numel() for t in _graph_workspaces.pop(key))
+    return freed
 
 
 def _inner_contiguous(t: torch.Tensor, name: str) -> None:

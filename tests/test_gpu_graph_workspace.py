@@ -61,6 +61,13 @@ def test_graph_replays_keep_their_workspace(sb, dev):
         # eager work between the replays, through the same entry point
         again = sb.ops.swa_decode_attention(q2, kv2[0], kv2[1], sl2, block_table=t2, window_left=-1, n_split=16)
         assert torch.equal(again, big)
+    # the graph is dropped: its workspace goes back to the allocator through the release hook, once
+    ids = sb.ops.graph_workspace_ids(dev)
+    assert ids, "the capture should own a workspace"
+    del graph
+    assert sb.ops.release_graph_workspace(ids[-1], dev) >= 1 << 20
+    assert ids[-1] not in sb.ops.graph_workspace_ids(dev)
+    assert sb.ops.release_graph_workspace(ids[-1], dev) == 0
 
 
 def test_streams_do_not_share_a_workspace(sb, dev):

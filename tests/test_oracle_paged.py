@@ -174,3 +174,45 @@ def test_block_manager_errors(sb):
         m.append_tokens(0, 64, True)
     with pytest.raises(KeyError):
         m.add_seq(0)
+
+
+def _manager_state(m):
+    return (m.free_stack(), m.ring.copy(), m.lo.copy(), m.hi.copy(), m.n_tokens.copy())
+
+
+def _same_state(a, b):
+    return a[0] == b[0] and all(np.array_equal(x, y) for x, y in zip(a[1:], b[1:]))
+
+
+def test_exhausted_pool_leaves_the_manager_untouched(sb):
+    """A step that runs out of blocks raises with nothing changed: no block is both free and resident, so
+    freeing a sequence afterwards cannot hand one block to two sequences (prompt chunk with evictions,
+    and a decode batch that fails at its second row)."""
+    M = sb.block_manager.WindowBlockManager
+    m = M(num_blocks=12, block_size=16, window_left=64, max_seqs=4, max_chunk_tokens=128)
+    m.add_seq("a")
+    m.add_seq("b")
+    m.append_tokens("a", 96, True, store_all=True)      # 6 blocks
+    m.append_tokens("b", 80, True, store_all=True)      # 5 blocks, 1 left
+    before = _manager_state(m)
+    with pytest.raises(RuntimeError, match="out of KV cache blocks"):
+        m.append_tokens("a", 128, True, store_all=True)  # evicts 2, needs 8: 3 free in all
+    assert _same_state(before, _manager_state(m))
+    m.free_seq("a")
+    free = m.free_stack()
+    assert len(free) == len(set(free)) == 7
+    resident_b = {int(m.ring[m.row_of("b"), j % m.ring_blocks]) for j in range(int(m.lo[m.row_of("b")]), int(m.hi[m.row_of("b")]) + 1)}
+    assert not (resident_b & set(free))
+
+    # decode batch: the first row's allocation succeeds on its own, the second finds the stack empty
+    m = M(num_blocks=5, block_size=16, window_left=1024, max_seqs=4)
+    for s in ("a", "b"):
+        m.add_seq(s)
+        m.append_tokens(s, 32, True)                     # 2 blocks each, both full: the next token allocates
+    before = _manager_state(m)
+    with pytest.raises(RuntimeError, match="out of KV cache blocks"):
+        m.decode_step(["a", "b"])
+    assert _same_state(before, _manager_state(m))
+    m.free_seq("b")
+    slots = m.decode_step(["a"])
+    assert slots.shape == (1,) and len(set(m.free_stack())) == m.num_free_blocks == 2
