@@ -132,6 +132,14 @@ int sb_kv_append(const sb_kv_append_args *args);
  * workspace's first 64 KiB zeroed before its first use (see below). */
 #define SB_DECODE_MERGE_IN_KERNEL 4
 
+/* bf16/fp16 queries over a paged element cache with one query row per sequence, no key_lo and no meta rows
+ * (the serving path) run the split as ONE stream of chunks per wavefront (swa_decode_stream.hip): a row
+ * boundary inside a balanced run costs no pipeline restart, and nothing is fetched twice. This flag keeps such
+ * calls on the per-segment kernels (swa_decode_mfma.hip), which serve every other case anyway (dense K/V,
+ * row_seq, key_lo, meta rows, prefetch depths 2 and 3, the merge inside the kernel). Same results up to fp32
+ * summation order. */
+#define SB_DECODE_PER_SEGMENT 8
+
 typedef struct sb_swa_decode_args {
   const void *q;   /* [num_rows, num_q_heads, head_size] */
   const void *k_cache;

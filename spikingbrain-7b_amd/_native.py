@@ -19,6 +19,7 @@ SB_ERR_INVALID, SB_ERR_UNSUPPORTED, SB_ERR_WORKSPACE = -1, -2, -3
 SB_DECODE_FORCE_VALU = 1
 SB_DECODE_BALANCED = 2
 SB_DECODE_MERGE_IN_KERNEL = 4
+SB_DECODE_PER_SEGMENT = 8
 SB_KV_NONE, SB_KV_INT8, SB_KV_FP8 = 0, 1, 2
 SB_GLA_VECTOR_ONLY = 1
 SB_SWA_DECODE_STATIC_SCRATCH_BYTES = 8 << 20

@@ -26,6 +26,8 @@
 namespace sb_host {
 void launch_swa_decode_split_mfma(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, int depth,
                                   hipStream_t st, const sb::DecodeParams &p, hipEvent_t ev_start, hipEvent_t ev_stop);
+void launch_swa_decode_stream(int dtype, int G, int Hkv, unsigned rows, unsigned n_split, hipStream_t st,
+                              const sb::DecodeParams &p, hipEvent_t ev_start, hipEvent_t ev_stop);
 void launch_swa_decode_split_i8(int dtype, int kv_quant, int G, int Hkv, unsigned rows, unsigned n_split, hipStream_t st,
                                 const sb::DecodeParams &p);
 }
@@ -790,6 +792,11 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
     p.merge_counter = (int *)a->workspace;
   if (a->phases != 2) {
     if (int8_kv) launch_swa_decode_split_i8(a->dtype, a->kv_quant, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p);
+    else if (mfma && !(a->flags & SB_DECODE_PER_SEGMENT) && a->block_table && !a->row_seq && !a->key_lo && a->meta_len == 0 &&
+             !p.merge_counter && ((a->flags >> 4) & 7) <= 1 &&
+             (int64_t)a->num_q_heads * a->q_stride_head * esz < (1LL << 31))
+      launch_swa_decode_stream(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p,
+                               (hipEvent_t)a->profile_start_event, (hipEvent_t)a->profile_stop_event);
     else if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
                                            (a->flags >> 4) & 7, st, p, (hipEvent_t)a->profile_start_event,
                                            (hipEvent_t)a->profile_stop_event);

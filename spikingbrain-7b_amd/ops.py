@@ -141,6 +141,7 @@ def swa_decode_attention(
     phases: int = 0,
     force_valu: bool = False,
     merge_in_kernel: bool = False,
+    per_segment: bool = False,
     balanced: Optional[bool] = None,
     host_seq_lens=None,
     k_scale: Optional[torch.Tensor] = None,
@@ -329,7 +330,8 @@ def swa_decode_attention(
         window_left=int(window_left), max_seq_len=int(min(max_seq_len, 2**31 - 1)), n_split=int(n_split),
         dtype=N.dtype_code(q.dtype), phases=int(phases),
         flags=(N.SB_DECODE_FORCE_VALU if force_valu else 0) | (N.SB_DECODE_BALANCED if balanced else 0)
-        | (N.SB_DECODE_MERGE_IN_KERNEL if merge_in_kernel else 0) | ((int(pipeline_depth) & 7) << 4),
+        | (N.SB_DECODE_MERGE_IN_KERNEL if merge_in_kernel else 0) | (N.SB_DECODE_PER_SEGMENT if per_segment else 0)
+        | ((int(pipeline_depth) & 7) << 4),
         scale=float(scale),
         q_stride_row=q.stride(0), q_stride_head=q.stride(1),
         out_stride_row=out.stride(0), out_stride_head=out.stride(1),
