@@ -33,8 +33,8 @@ HBM_PEAK_GBPS = 8000.0
 # FETCH_SIZE / WRITE_SIZE runs (counters cannot be read from inside this script). The profile summary records
 # them together with a hash of the kernel sources it was taken with; the figure is attached to the bench line
 # only while the sources still hash to that value.
-PROFILE_FILE = os.path.join(ROOT, "profiles", "swa_decode_split_mfma_config2.md")
-KERNEL_SOURCES = ("swa_decode_mfma.hip", "swa_decode.hip", "swa_decode_params.h", "mfma_util.h", "common.h")
+PROFILE_FILE = os.path.join(ROOT, "profiles", "swa_decode_stream_config2.md")
+KERNEL_SOURCES = ("swa_decode_stream.hip", "swa_decode.hip", "swa_decode_params.h", "mfma_util.h", "common.h")
 
 
 def kernel_sources_hash():
@@ -57,8 +57,8 @@ def recorded_traffic():
     if not m:
         return None, "profile summary holds no traffic record"
     if m.group(2) != kernel_sources_hash():
-        return None, "profiles/swa_decode_split_mfma_config2.md was recorded with older kernel sources"
-    return int(m.group(1)), "rocprofv3 FETCH_SIZE + WRITE_SIZE recorded in profiles/swa_decode_split_mfma_config2.md (same kernel sources)"
+        return None, "profiles/swa_decode_stream_config2.md was recorded with older kernel sources"
+    return int(m.group(1)), "rocprofv3 FETCH_SIZE + WRITE_SIZE recorded in profiles/swa_decode_stream_config2.md (same kernel sources)"
 
 
 HQ, HKV, D, BS, WL = 28, 4, 128, 16, 4096
@@ -387,6 +387,8 @@ def main():
     ap.add_argument("--unfused", action="store_true", help="append with a separate kv_append launch")
     ap.add_argument("--force-valu", action="store_true",
                     help="run the vector-ALU split kernel instead of the matrix-core one (for comparison profiles)")
+    ap.add_argument("--per-segment", action="store_true",
+                    help="run the per-segment matrix-core split kernel instead of the stream kernel (for comparison profiles)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hybrid", action="store_true", help="skip the 28-layer hybrid decode step (config 5) section")
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
@@ -451,7 +453,8 @@ def main():
     def attend(c, phases, **kw):
         sb.ops.swa_decode_attention(prob["q"], c[0], c[1], prob["seqlens"], block_table=prob["tables"],
                                     window_left=WL, out=prob["out"], max_seq_len=prob["max_seq_len"],
-                                    n_split=args.n_split, phases=phases, force_valu=args.force_valu, balanced=False, **kw)
+                                    n_split=args.n_split, phases=phases, force_valu=args.force_valu, balanced=False,
+                                    per_segment=args.per_segment, **kw)
 
     def step(i, events=None):
         """One layer-step as MetaAttentionImpl.forward runs a pure decode batch: the split kernel
@@ -517,7 +520,7 @@ def main():
     k_ms = statistics.mean(a.elapsed_time(b) for a, b in evs)
     achieved = prob["bytes_split_kernel"] / (k_ms * 1e-3) / 1e9
 
-    default_workload = not (args.force_valu or args.unfused or args.n_split)
+    default_workload = not (args.force_valu or args.unfused or args.n_split or args.per_segment)
     traffic, traffic_source = recorded_traffic() if default_workload else (None, "not the default workload")
     line = {
         "metric": "SWA decode-attn+append GB/s (% of HBM peak) and decode tok/s, 7B shapes, 1 GPU",
@@ -534,7 +537,8 @@ def main():
                    "ms_per_step_median_host_clock": round(statistics.median(region_host) / args.steps * 1e3, 4)},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "decode_tok_per_s_layer_step": round(prob["B"] / (wall / args.steps), 1),
-        "roofline": {"bound": "hbm", "kernel": "swa_decode_split_kernel<BF16,7> (vector ALU)" if args.force_valu else "swa_decode_split_mfma_kernel<BF16>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": "swa_decode_split_kernel<BF16,7> (vector ALU)" if args.force_valu
+                     else ("swa_decode_split_mfma_kernel<BF16>" if args.per_segment else "swa_decode_stream_kernel<BF16, fixed split>"), "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_source": traffic_source, "kernel_ms": round(k_ms, 4),
                      "kernel_ms_measured": f"HIP events on the kernel's own dispatch, mean of {len(evs)} consecutive steps run right after the "

@@ -421,6 +421,52 @@ __global__ __launch_bounds__(128) void swa_decode_merge_balanced_kernel(const De
   if (d == 0 && p.lse) p.lse[rh] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
 }
 
+// Merge behind the stream form of the balanced split: the wavefront that ended a row has left the span of runs
+// (workgroups) holding the row's partials in ws_rows, so nothing has to be worked out from the other rows'
+// lengths here. Same arithmetic and order as swa_decode_merge_balanced_kernel.
+template <typename E>
+__global__ __launch_bounds__(128) void swa_decode_merge_rows_kernel(const DecodeParams p) {
+  const int64_t rh = blockIdx.x;  // r*Hq + hq
+  const int r = (int)(rh / p.Hq);
+  const int hq = (int)(rh - (int64_t)r * p.Hq);
+  const int d = threadIdx.x;
+  const int hi = p.seq_lens[r];
+  const int lo = p.window_left >= 0 ? max(0, hi - 1 - p.window_left) : 0;
+  float tot = 0.f, L = 0.f, M = kNegInf;
+  if (hi > lo) {
+    const int w_lo = p.ws_rows[2 * r], w_hi = p.ws_rows[2 * r + 1];
+    // eight partials per trip to memory, maxima, denominators and numerators together (a row cut into more
+    // than eight runs goes round again and rescales what it has): one trip for almost every row
+    for (int w = w_lo; w <= w_hi; w += 8) {
+      float ms[8], ls[8], av[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int64_t part = (int64_t)(min(w + j, w_hi) + r) * p.Hq + hq;
+        ms[j] = p.ws_ml[part * 2];
+        ls[j] = p.ws_ml[part * 2 + 1];
+        av[j] = p.ws_acc[part * 128 + d];
+      }
+      float Mn = M;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) Mn = fmaxf(Mn, ms[j]);
+      if (Mn != kNegInf) {
+        const float keep = (M == kNegInf) ? 0.f : fast_exp2(M - Mn);
+        tot *= keep;
+        L *= keep;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float f = (w + j > w_hi || ms[j] == kNegInf) ? 0.f : fast_exp2(ms[j] - Mn);
+          tot = fmaf(av[j], f, tot);
+          L = fmaf(ls[j], f, L);
+        }
+      }
+      M = Mn;
+    }
+  }
+  store_out<E>(p.out, (int64_t)r * p.o_sr + (int64_t)hq * p.o_sh + d, L > 0.f ? tot / L : 0.f);
+  if (d == 0 && p.lse) p.lse[rh] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
+}
+
 struct LseMergeParams {
   char *out;
   float *lse;
@@ -586,8 +632,8 @@ extern "C" int32_t sb_swa_decode_prefer_balanced(const int32_t *host_seq_lens, i
   const int64_t n_wg = balanced_workgroups(num_rows, n_split < 2 ? 2 : n_split);
   int64_t nonempty = 0;
   for (int64_t r = 0; r < num_rows; ++r) nonempty += chunks[r] > 0;
-  const int64_t laid_out = total + nonempty * kBalancedRowStartChunks;
-  const double balanced_end = (double)((laid_out + n_wg - 1) / n_wg) + kBalancedChunks + (double)num_rows / kBalancedRowsPerChunk;
+  (void)nonempty;  // (the stream kernel, which serves these calls, charges a row start nothing)
+  const double balanced_end = (double)((total + n_wg - 1) / n_wg) + kBalancedChunks + (double)num_rows / kBalancedRowsPerChunk;
   return balanced_end < fixed_end ? 1 : 0;
 }
 
@@ -595,7 +641,8 @@ extern "C" size_t sb_swa_decode_workspace_bytes(int64_t num_rows, int32_t num_q_
                                                 int32_t head_size, int32_t n_split) {
   if (n_split <= 1 || num_rows <= 0 || num_q_heads <= 0 || head_size <= 0) return 0;
   const int64_t parts = partial_slots(num_rows, n_split) * num_q_heads;
-  return (size_t)(kMergeCounterBytes + round_up(parts * head_size * 4, 256) + round_up(parts * 2 * 4, 256));
+  return (size_t)(kMergeCounterBytes + round_up(parts * head_size * 4, 256) + round_up(parts * 2 * 4, 256) +
+                  round_up(num_rows * 2 * 4, 256));  // ... + per row the span of runs holding its partials (balanced split)
 }
 
 extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
@@ -675,6 +722,8 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   p.Hkv = a->num_kv_heads;
   p.ws_acc = need ? (float *)((char *)a->workspace + kMergeCounterBytes) : nullptr;
   p.ws_ml = need ? (float *)((char *)a->workspace + kMergeCounterBytes + round_up(parts * 128 * 4, 256)) : nullptr;
+  p.ws_rows = need ? (int32_t *)((char *)a->workspace + kMergeCounterBytes + round_up(parts * 128 * 4, 256) +
+                                 round_up(parts * 2 * 4, 256)) : nullptr;
   p.Hq = a->num_q_heads; p.block_size = a->block_size > 0 ? a->block_size : 16;
   p.window_left = a->window_left; p.n_split = n_split;
   p.rows = (int)a->num_rows; p.n_wg = 0;
@@ -790,11 +839,14 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
       a->phases == 0 && ((a->flags >> 4) & 7) <= 1 && a->meta_len == 0 &&
       (a->num_rows + 7) / 8 * 8 * (int64_t)a->num_kv_heads <= kMergeCounters)
     p.merge_counter = (int *)a->workspace;
+  // the serving path (paged element cache, one query row per sequence, no key_lo, no meta rows) runs the
+  // split as one stream of chunks per wavefront
+  const bool stream = mfma && !int8_kv && !(a->flags & SB_DECODE_PER_SEGMENT) && a->block_table && !a->row_seq &&
+                      !a->key_lo && a->meta_len == 0 && !p.merge_counter && ((a->flags >> 4) & 7) <= 1 &&
+                      (int64_t)a->num_q_heads * a->q_stride_head * esz < (1LL << 31);
   if (a->phases != 2) {
     if (int8_kv) launch_swa_decode_split_i8(a->dtype, a->kv_quant, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p);
-    else if (mfma && !(a->flags & SB_DECODE_PER_SEGMENT) && a->block_table && !a->row_seq && !a->key_lo && a->meta_len == 0 &&
-             !p.merge_counter && ((a->flags >> 4) & 7) <= 1 &&
-             (int64_t)a->num_q_heads * a->q_stride_head * esz < (1LL << 31))
+    else if (stream)
       launch_swa_decode_stream(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split, st, p,
                                (hipEvent_t)a->profile_start_event, (hipEvent_t)a->profile_stop_event);
     else if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
@@ -808,6 +860,11 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   if (rc != SB_OK || n_split == 1 || a->phases == 1 || p.merge_counter) return rc;
 
   const dim3 mgrid((unsigned)(a->num_rows * a->num_q_heads));
+  if (p.n_wg > 0 && stream) {
+    if (a->dtype == SB_BF16) hipLaunchKernelGGL(swa_decode_merge_rows_kernel<BF16>, mgrid, dim3(128), 0, st, p);
+    else hipLaunchKernelGGL(swa_decode_merge_rows_kernel<F16>, mgrid, dim3(128), 0, st, p);
+    return check_launch("swa_decode_merge_rows_kernel");
+  }
   if (p.n_wg > 0) {
     if (a->dtype == SB_BF16) hipLaunchKernelGGL(swa_decode_merge_balanced_kernel<BF16>, mgrid, dim3(128), 0, st, p);
     else hipLaunchKernelGGL(swa_decode_merge_balanced_kernel<F16>, mgrid, dim3(128), 0, st, p);

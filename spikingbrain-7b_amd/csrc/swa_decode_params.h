@@ -14,10 +14,11 @@ constexpr int kMergeCounterBytes = 64 << 10;
 constexpr int kMergeCounters = kMergeCounterBytes / 4 - 1;
 constexpr int kMergeFaultWord = kMergeCounterBytes / 4 - 1;
 
-// Balanced split: on the common chunk axis every non-empty row is preceded by this many virtual chunks. A
-// workgroup whose run crosses into a new row drains and refills its load pipeline there (a round trip to
-// memory with nothing in flight); the virtual chunks charge that to its run, so it gets fewer real chunks
-// than a workgroup that stays inside one row. Split kernel, merge kernel and the host's cost model share it.
+// Balanced split of the per-segment kernel (swa_decode_mfma.hip): on the common chunk axis every non-empty row
+// is preceded by this many virtual chunks. A workgroup of that kernel whose run crosses into a new row drains
+// and refills its load pipeline there (a round trip to memory with nothing in flight); the virtual chunks
+// charge that to its run, so it gets fewer real chunks than a workgroup that stays inside one row. That split
+// kernel and its merge kernel share it. (The stream kernel crosses rows without a drain and has none.)
 constexpr int kBalancedRowStartChunks = SB_BALANCED_T;
 
 struct DecodeParams {
@@ -33,6 +34,7 @@ struct DecodeParams {
   const int32_t *key_lo;
   float *ws_acc;  // [rows, Hq, n_split, 128]
   float *ws_ml;   // [rows, Hq, n_split, 2]
+  int32_t *ws_rows;  // balanced split, stream kernel: per row the first and last run (workgroup) holding a partial of it
   int Hq, block_size, window_left, n_split;
   int rows, n_wg;  // balanced split: query rows, workgroups per kv-head group (0 = fixed split)
   // Merge inside the split kernel (matrix-core fixed split): arrival counters [rows, Hkv], zero before and after

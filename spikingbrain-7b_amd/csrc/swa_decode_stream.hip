@@ -26,10 +26,9 @@
 // chunk there, 3 % of its traffic at the 7B decode shape).
 //
 // Runs. Fixed split (kBalanced = false): grid = (rows, kv-head groups, splits), a workgroup's run is
-// chunks [cb, ce) of its row. Balanced split: the chunks of all rows are laid end to end (every non-empty
-// row preceded by kBalancedRowStartChunks virtual chunks, as the merge kernel and the host's cost model lay
-// them out), cut into gridDim.x equal runs; a run that covers several rows writes one partial per row,
-// numbered workgroup + row. Every wavefront derives its run from seq_lens by itself (lane i looks at row
+// chunks [cb, ce) of its row. Balanced split: the chunks of all rows are laid end to end and cut into
+// gridDim.x runs that differ by one chunk at most; a run that covers several rows writes one partial per
+// row, numbered workgroup + row, and the runs that start and end a row note their numbers for the merge. Every wavefront derives its run from seq_lens by itself (lane i looks at row
 // base + i, one wave-wide scan); the rows of a batch of 64 are then read back from those lanes, so walking
 // into the next row costs no memory access.
 //
@@ -42,32 +41,6 @@
 #include "common.h"
 #include "mfma_util.h"
 #include "swa_decode_params.h"
-
-#ifdef SB_STREAM_TRACE
-// (measurement builds only) per wavefront: start, first item computed, end (100 MHz clock), items, XCC
-__device__ unsigned long long sb_stream_trace[8192 * 8];
-__device__ unsigned long long sb_stream_trace_items[1024 * 64];  // time after every item of the first 1024 wavefronts
-extern "C" int sb_debug_stream_trace(void *dst, size_t bytes) {
-  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(sb_stream_trace), bytes, 0, hipMemcpyDeviceToHost);
-}
-extern "C" int sb_debug_stream_trace_items(void *dst, size_t bytes) {
-  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(sb_stream_trace_items), bytes, 0, hipMemcpyDeviceToHost);
-}
-#define SB_TRACE_ITEM(k)                                                                                               \
-  do {                                                                                                                 \
-    if (lane == 0 && (k) < 64)                                                                                         \
-      sb_stream_trace_items[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + (tid >> 6)) % 1024 * 64 + (k)] = \
-          wall_clock64();                                                                                              \
-  } while (0)
-#define SB_TRACE(slot, value)                                                                                          \
-  do {                                                                                                                 \
-    if (lane == 0)                                                                                                     \
-      sb_stream_trace[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + (tid >> 6)) % 8192 * 8 + (slot)] = \
-          (value);                                                                                                     \
-  } while (0)
-#else
-#define SB_TRACE(slot, value) do { } while (0)
-#endif
 
 namespace {
 
@@ -83,6 +56,7 @@ struct Slot {
 // What the computation of an item needs to know about it (wave-uniform).
 struct Rec {
   int r, lo, hi, cc;
+  bool row_first;  // the segment starts with the row's first chunk
   bool valid, edge, seg_last, row_last;
   int64_t part;  // index of the first head's partial of the segment (heads follow at part_hs)
 };
@@ -114,8 +88,6 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
   const int g = lane >> 4;
   const int c = lane & 15;
   const int w = blockIdx.x;
-  SB_TRACE(0, wall_clock64());
-  SB_TRACE(4, (unsigned long long)__builtin_amdgcn_s_getreg(20 | (3 << 11)));
 
   // ---- rows: lane i holds row batch0 + i ---------------------------------------------------------------
   int batch0 = 0;
@@ -132,7 +104,7 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
     v_n = hi > lo ? ((hi - 1) >> 5) - (lo >> 5) + 1 : 0;
     batch0 = base;
     if constexpr (kBalanced) {
-      const int incl = stream_wave_scan(v_n > 0 ? v_n + kBalancedRowStartChunks : 0, lane);
+      const int incl = stream_wave_scan(v_n, lane);
       v_own = before + incl - v_n;
       return before + __builtin_amdgcn_readlane(incl, 63);
     } else {
@@ -153,16 +125,18 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
         if (base + lane >= p.rows) hi = 0;
         const int lo = p.window_left >= 0 ? max(0, hi - 1 - p.window_left) : 0;
         const int nn = hi > lo ? ((hi - 1) >> 5) - (lo >> 5) + 1 : 0;
-        total += stream_wave_sum(nn > 0 ? nn + kBalancedRowStartChunks : 0);
+        total += stream_wave_sum(nn);
       }
       total = __builtin_amdgcn_readfirstlane(total);
     }
     axis_next = load_batch(0, 0);
     if (p.rows <= 64) total = axis_next;
+    // run w = chunks [w total / n, (w + 1) total / n) of the common axis: the runs differ by one chunk at most
     const int n_wg = gridDim.x;
-    const int per = (total + n_wg - 1) / n_wg;
-    const int c0 = w * per;
-    c1 = min(c0 + per, total);
+    // (fewer chunks than runs: one chunk each for the first `total` runs, so that no run in the middle of a row
+    // is empty: the merge reads a partial from every run between a row's first and last)
+    const int c0 = total < n_wg ? w : (int)((int64_t)w * total / n_wg);
+    c1 = total < n_wg ? min(w + 1, total) : (int)((int64_t)(w + 1) * total / n_wg);
     if (c0 >= c1) return;
     while (axis_next <= c0) axis_next = load_batch(batch0 + 64, axis_next);  // (c0 < total: ends inside the rows)
     const uint64_t cand = __builtin_amdgcn_ballot_w64(v_n > 0 && v_own + v_n > c0);
@@ -214,6 +188,7 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
   // ---- the front of the stream: the next item to be requested ---------------------------------------------
   bool f_valid = true;
   int f_i = i0, f_r, f_lo, f_hi, f_cc, f_ce, f_end;  // f_end: one past the last chunk of the row's window
+  bool f_row_first = false;
   int f_blk0 = 0, f_blk1 = 0, f_in0 = 0, f_in1 = 0;  // the item's two tiles: block-table entry, first row inside the block
   bool f_edge = false;
   // Looks the blocks of the front item's tiles up. Only the loads are issued here; the entries are first
@@ -240,6 +215,7 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
     f_lo = __builtin_amdgcn_readlane(v_lo, i);
     f_hi = __builtin_amdgcn_readlane(v_hi, i);
     f_end = (f_lo >> 5) + __builtin_amdgcn_readlane(v_n, i);
+    f_row_first = first == (f_lo >> 5);
     f_cc = first;
     f_ce = last;
     locate();
@@ -279,6 +255,7 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
   auto snapshot = [&]() {
     Rec x;
     x.r = f_r; x.lo = f_lo; x.hi = f_hi; x.cc = f_cc;
+    x.row_first = f_row_first;
     x.valid = f_valid;
     x.edge = f_edge;
     x.seg_last = f_cc + 1 == f_ce;
@@ -434,6 +411,14 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
         *reinterpret_cast<uint4 *>(const_cast<char *>(lane < 16 ? p.k : p.v) + dst) = fresh;
       }
     }
+    if constexpr (kBalanced) {
+      // the runs that start and end a row tell the merge which runs hold the row's partials: every run from
+      // the first to the last (rows without chunks have none; the merge sees that from the row's length)
+      if (any && kvh == 0 && lane == 0) {
+        if (x.row_first) p.ws_rows[2 * x.r] = w;
+        if (x.row_last) p.ws_rows[2 * x.r + 1] = w;
+      }
+    }
     float lt = l;
     lt += __shfl_xor(lt, 16);
     lt += __shfl_xor(lt, 32);
@@ -473,6 +458,7 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
   if (cb >= ce) {  // fixed split: a part of the row with no chunks still owes the merge its (empty) partial
     Rec x;
     x.r = batch0 + i0; x.lo = x.hi = x.cc = 0;
+    x.row_first = false;
     x.valid = true;
     x.edge = x.seg_last = x.row_last = false;
     x.part = part_of(x.r);
@@ -493,20 +479,11 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
   load_row(rec0.r);
   issue(ring[0]);
   advance();
-#ifdef SB_STREAM_TRACE
-  int n_items = 0;
-  SB_TRACE(5, wall_clock64());
-#endif
   do {
     rec1 = snapshot();
     issue(ring[1]);
     advance();
     compute(rec0, ring[0]);
-#ifdef SB_STREAM_TRACE
-    if (n_items == 0) SB_TRACE(1, wall_clock64());
-    SB_TRACE_ITEM(n_items);
-    n_items += 1 + (rec1.valid ? 1 : 0);
-#endif
     if (rec0.seg_last) finish(rec0, true, rec1);
     rec0 = snapshot();
     issue(ring[0]);
@@ -514,15 +491,8 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
     if (rec1.valid) {
       compute(rec1, ring[1]);
       if (rec1.seg_last) finish(rec1, true, rec0);
-#ifdef SB_STREAM_TRACE
-      SB_TRACE_ITEM(n_items - 1);
-#endif
     }
   } while (rec0.valid);
-#ifdef SB_STREAM_TRACE
-  SB_TRACE(2, wall_clock64());
-  SB_TRACE(3, (unsigned long long)n_items);
-#endif
 }
 
 }  // namespace
