@@ -100,6 +100,43 @@ class HybridDecodeCache:
         for s in self.seq_ids:
             self.manager.append_tokens(s, context_len, True)
 
+    _STAGES = 4   # staging sets: the host may run this many steps ahead of the GPU
+
+    def _staging(self):
+        """A ring of `_STAGES` staging sets, each a pair of pinned host buffers (the step's slots | lengths and
+        its block tables are written there, so that their uploads are truly asynchronous: from pageable
+        memory a `non_blocking` copy still waits for the stream, which lock-steps the host to the GPU) and
+        the device tensors they are uploaded into. The uploads run on a stream of their own, beside the
+        layers of the step before; the layers' stream waits for them. A set is rewritten only after the
+        layers of the step that used it have run (an event recorded behind them when the next step's
+        metadata is asked for), so the host runs at most `_STAGES` steps ahead."""
+        if not hasattr(self, "_stage_sets"):
+            B, width, dev = self.batch, self.manager.ring_blocks, self.device
+            self._stage_sets = [dict(packed=torch.empty(2 * B, dtype=torch.int64).pin_memory(),
+                                     tables=torch.empty(B * width, dtype=torch.int32).pin_memory(),
+                                     d_packed=torch.empty(2 * B, dtype=torch.int64, device=dev),
+                                     d_tables=torch.empty(B * width, dtype=torch.int32, device=dev),
+                                     uploaded=torch.cuda.Event(), used=None) for _ in range(self._STAGES)]
+            self._stage_next = 0
+            self._stage_last = None
+            self._upload_stream = torch.cuda.Stream(device=dev)
+            self.host_wait_s = 0.0   # time spent waiting for a staging set (the GPU is that far behind)
+        cur = torch.cuda.current_stream(self.device)
+        if self._stage_last is not None:   # the layers of the previous step are all enqueued by now
+            last = self._stage_sets[self._stage_last]
+            if last["used"] is None:
+                last["used"] = torch.cuda.Event()
+            last["used"].record(cur)
+        st = self._stage_sets[self._stage_next]
+        self._stage_last = self._stage_next
+        self._stage_next = (self._stage_next + 1) % self._STAGES
+        if st["used"] is not None and not st["used"].query():
+            import time
+            t0 = time.perf_counter()
+            st["used"].synchronize()
+            self.host_wait_s += time.perf_counter() - t0
+        return st
+
     def step_metadata(self) -> MetaAttentionMetadata:
         """Advance every sequence by one token (eviction + allocation) and build the decode-only
         metadata the SWA layers of this step share."""
@@ -107,13 +144,23 @@ class HybridDecodeCache:
         slots = mgr.decode_step(self.seq_ids)
         tables, seqlens, _ = mgr.kernel_view(self.seq_ids)
         dev = self.device
-        packed = torch.from_numpy(np.concatenate([slots, seqlens.astype(np.int64)])).to(dev, non_blocking=True)
-        B = self.batch
+        B, width = self.batch, tables.shape[1]
+        st = self._staging()
+        hp = st["packed"].numpy()
+        hp[:B] = slots
+        hp[B:] = seqlens
+        st["tables"][:B * width].view(B, width).numpy()[...] = tables
+        with torch.cuda.stream(self._upload_stream):
+            st["d_packed"].copy_(st["packed"], non_blocking=True)
+            st["d_tables"][:B * width].copy_(st["tables"][:B * width], non_blocking=True)
+            st["uploaded"].record(self._upload_stream)
+        torch.cuda.current_stream(dev).wait_event(st["uploaded"])
+        packed = st["d_packed"]
         return MetaAttentionMetadata(
             num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B,
             slot_mapping=packed[:B], seq_lens=None, seq_lens_tensor=packed[B:].to(torch.int32),
             max_prefill_seq_len=0, max_decode_seq_len=int(seqlens.max()), context_lens_tensor=None,
-            block_tables=torch.from_numpy(tables).to(dev, non_blocking=True), use_cuda_graph=False,
+            block_tables=st["d_tables"][:B * width].view(B, width), use_cuda_graph=False,
             max_query_len=1, max_decode_query_len=1)
 
     # -- device-side stepping: no host work between decode steps --------------------------------
