@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define SB_ABI_VERSION 2
+#define SB_ABI_VERSION 3
 
 enum sb_dtype { SB_BF16 = 0, SB_F16 = 1, SB_F32 = 2 };
 
@@ -199,7 +199,7 @@ typedef struct sb_swa_decode_args {
    * window and enter the same online softmax, so out and lse are those of ONE softmax over window
    * and meta keys (a row with an empty window attends to the meta rows alone). meta_len = 0 = off.
    * bf16/fp16 queries on the matrix-core kernels with the fixed split only (rejected with
-   * SB_DECODE_BALANCED, SB_DECODE_FORCE_VALU or fp32). Over a byte-code cache (kv_quant) the meta rows
+   * SB_DECODE_BALANCED, SB_DECODE_FORCE_VALU or fp32; soft cap / ALiBi: see below). Over a byte-code cache (kv_quant) the meta rows
    * are still elements of dtype: they are not quantised, and an fp8 cache's tensor scales do not apply
    * to them. */
   const void *meta_k;
@@ -216,10 +216,18 @@ typedef struct sb_swa_decode_args {
   /* The two score options the backend passes on to flash-attn (meta_attention.py:665-690, :965-981
    * alibi_slopes=..., softcap=...): softcap > 0 turns every scaled score x into softcap * tanh(x / softcap);
    * alibi_slopes ([num_q_heads] fp32, NULL = off) adds -slope[h] * (query position - key index), the query
-   * sitting at key index seq_lens[r]-1. Both are applied in front of the mask, the cap first. bf16/fp16
-   * queries on the matrix-core kernels (element, INT8 and fp8 caches); not together with meta tokens. */
+   * sitting at key index seq_lens[r]-1. Both are applied in front of the mask, the cap first. Any query
+   * type (the fp32 vector kernel takes them too); over element, INT8 and fp8 caches.
+   * Together with meta rows (bf16/fp16): the cap applies to their scores as to any other; their ALiBi term
+   * is the one flash-attn gives them in the reference's second attention call
+   * (fa_kernel_metatoken.py:169-188: all query rows of the call stacked as ONE sequence of
+   * meta_bias_rows queries against the meta_len meta keys, causal=False), i.e. for query row r and meta
+   * row j:  -slope[h] * |meta_bias_row0 + r + meta_len - meta_bias_rows - j|.  meta_bias_row0 is the
+   * index of this call's row 0 in that stacked sequence (0 when the call holds all of its rows),
+   * meta_bias_rows its length (0 = num_rows). */
   float softcap;
   const float *alibi_slopes;
+  int64_t meta_bias_row0, meta_bias_rows;
 } sb_swa_decode_args;
 
 /* Split count the auto rule (n_split = 0) would use for these shapes: the one with the lowest estimated
@@ -422,9 +430,13 @@ typedef struct sb_swa_prefill_args {
   int32_t meta_len;
   int64_t meta_stride_row, meta_stride_head;
   /* Score options as for sb_swa_decode (fa_kernel_metatoken.py:235-253 alibi_slopes=..., softcap=...): query j
-   * of a sequence sits at key index seq_lens_k - query_len + j. Not together with meta tokens. */
+   * of a sequence sits at key index seq_lens_k - query_len + j. Together with meta rows: as for
+   * sb_swa_decode, the stacked sequence of fa_kernel_metatoken.py:258-275 being the call's packed query rows:
+   * row t of q/out is its query meta_bias_row0 + t, and meta_bias_rows (required then: the kernel does not
+   * know the total) is that sequence's length: the packed query rows plus the meta tokens' own queries. */
   float softcap;
   const float *alibi_slopes;
+  int64_t meta_bias_row0, meta_bias_rows;
 } sb_swa_prefill_args;
 
 int sb_swa_prefill(const sb_swa_prefill_args *args);

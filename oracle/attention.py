@@ -192,14 +192,25 @@ def lse_merge(out_a: np.ndarray, lse_a: np.ndarray, out_b: np.ndarray, lse_b: np
 
 
 def metatoken_attention(q1: np.ndarray, q2: Optional[np.ndarray], k1: np.ndarray, k2: np.ndarray,
-                        v1: np.ndarray, v2: np.ndarray, scale: float, sliding_window: int) -> np.ndarray:
+                        v1: np.ndarray, v2: np.ndarray, scale: float, sliding_window: int,
+                        softcap: float = 0.0, alibi_slopes: Optional[Sequence[float]] = None,
+                        stack_row0: int = 0, stack_rows: Optional[int] = None) -> np.ndarray:
     """The dense masked-softmax statement of meta-token attention,
     vllm_hymeta/attention/fa_kernel_metatoken.py:372-405, for one sequence: ONE softmax per query
     over [k2 | k1]. Query i of q1 (Lq queries, bottom-right aligned on the Lk keys of k1) sees every
     meta token and the keys k with 0 <= pos_i - k < sliding_window (sliding_window <= 0: no window
     limit); the meta tokens' own queries q2 see the meta tokens only. q1 [Lq, Hq, D], q2 [M, Hq, D]
     or None, k1/v1 [Lk, Hkv, D], k2/v2 [M, Hkv, D]. Returns [Lq (+ M), Hq, D] float64, rows in the
-    order (q1, q2) as at :388 (the flash path moves the q2 rows to the front, :278-279)."""
+    order (q1, q2) as at :388 (the flash path moves the q2 rows to the front, :278-279).
+
+    softcap / alibi_slopes: what the flash path does with them (:157-194, :235-275). It runs two attentions
+    and merges them by log-sum-exp, which is one softmax over the union of their (capped, biased) scores. The
+    window attention biases key k of query i by -slope * (pos_i - k). The second attention stacks ALL query
+    rows of the call (every sequence's q1 rows, then the q2 rows) into one sequence of `stack_rows` queries
+    against the M meta keys with causal=False, for which flash-attn's ALiBi term is
+    -slope * |i + M - stack_rows - j| for stacked query i and meta key j. This function's q1 rows are stacked
+    queries stack_row0 .. stack_row0 + Lq - 1 and its q2 rows the last M ones (stack_rows defaults to
+    Lq (+ M): this sequence alone)."""
     Lq, Hq, D = q1.shape
     Lk, Hkv, _ = k1.shape
     M = k2.shape[0]
@@ -212,13 +223,22 @@ def metatoken_attention(q1: np.ndarray, q2: Optional[np.ndarray], k1: np.ndarray
         win &= (q_id[:, None] - k_id[None, :]) < sliding_window
     visible[:, M:] = win
     q = q1
+    n_stack = stack_rows if stack_rows is not None else Lq + (M if q2 is not None else 0)
+    stacked = stack_row0 + np.arange(Lq)                      # place of each row in the second attention's sequence
+    window_dist = (q_id[:, None] - k_id[None, :]).astype(np.float64)
     if q2 is not None:
         q = np.concatenate([q1, q2], 0)
         meta_rows = np.concatenate([np.ones((M, M), bool), np.zeros((M, Lk), bool)], 1)
         visible = np.concatenate([visible, meta_rows], 0)
+        stacked = np.concatenate([stacked, n_stack - M + np.arange(M)])
+        window_dist = np.concatenate([window_dist, np.zeros((M, Lk))], 0)
+    meta_dist = np.abs(stacked[:, None] + M - n_stack - np.arange(M)[None, :]).astype(np.float64)
+    dist = np.concatenate([meta_dist, window_dist], 1)        # [rows, M + Lk], what a slope multiplies
     k = np.concatenate([k2, k1], 0).astype(np.float64)
     v = np.concatenate([v2, v1], 0).astype(np.float64)
     out = np.zeros((q.shape[0], Hq, D))
     for h in range(Hq):
-        out[:, h] = masked_softmax_attention(q[:, h].astype(np.float64), k[:, h // G], v[:, h // G], ~visible, scale)
+        bias = None if alibi_slopes is None else -float(alibi_slopes[h]) * dist
+        out[:, h] = masked_softmax_attention(q[:, h].astype(np.float64), k[:, h // G], v[:, h // G], ~visible, scale,
+                                             softcap=softcap, bias=bias)
     return out

@@ -23,7 +23,7 @@ SB_DECODE_PER_SEGMENT = 8
 SB_KV_NONE, SB_KV_INT8, SB_KV_FP8 = 0, 1, 2
 SB_GLA_VECTOR_ONLY = 1
 SB_SWA_DECODE_STATIC_SCRATCH_BYTES = 8 << 20
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _DTYPES = {torch.bfloat16: SB_BF16, torch.float16: SB_F16, torch.float32: SB_F32}
 
@@ -62,7 +62,7 @@ class SwaDecodeArgs(C.Structure):
         ("k_scale_tensor", f32), ("v_scale_tensor", f32),
         ("meta_k", vp), ("meta_v", vp), ("meta_len", i32), ("meta_stride_row", i64), ("meta_stride_head", i64),
         ("profile_start_event", vp), ("profile_stop_event", vp),
-        ("softcap", f32), ("alibi_slopes", vp),
+        ("softcap", f32), ("alibi_slopes", vp), ("meta_bias_row0", i64), ("meta_bias_rows", i64),
     ]
 
 
@@ -106,7 +106,7 @@ class SwaPrefillArgs(C.Structure):
         ("stream", vp), ("lse", vp), ("k_scale", vp), ("v_scale", vp), ("kv_quant", i32),
         ("k_scale_tensor", f32), ("v_scale_tensor", f32),
         ("meta_k", vp), ("meta_v", vp), ("meta_len", i32), ("meta_stride_row", i64), ("meta_stride_head", i64),
-        ("softcap", f32), ("alibi_slopes", vp),
+        ("softcap", f32), ("alibi_slopes", vp), ("meta_bias_row0", i64), ("meta_bias_rows", i64),
     ]
 
 

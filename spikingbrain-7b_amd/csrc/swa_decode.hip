@@ -122,6 +122,10 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   for (int h = 0; h < G; ++h)
     qp[h] = load_pack<E>(p.q + (r * p.q_sr + (int64_t)(kvh * G + h) * p.q_sh + c * 8) * E::kBytes);
 
+  float slope[G];  // ALiBi slopes of the group's heads
+#pragma unroll
+  for (int h = 0; h < G; ++h) slope[h] = p.opt.slopes ? p.opt.slopes[kvh * G + h] : 0.f;
+
   float m[G], l[G], acc[G][8];
 #pragma unroll
   for (int h = 0; h < G; ++h) {
@@ -165,6 +169,13 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int h = 0; h < G; ++h) s[h][j] = row16_allreduce_sum(dot_pack<E>(qp[h], kb[j]));
+    if (p.opt.on) {  // soft cap / ALiBi (wave-uniform; the query sits at key index hi - 1)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int h = 0; h < G; ++h)
+          s[h][j] = adjust_score(p.opt, s[h][j], slope[h], (float)(i0 + 4 * j + g - (hi - 1)));
+    }
     if (i0 < lo || i0 + 16 > hi) {  // edge tile: mask keys outside [lo, hi)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -784,10 +795,16 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   p.opt.mult = p.scale_log2 / sb::kLog2e;  // what turns a raw dot product into the scaled score (K tensor scale included)
   p.opt.inv_mult = 1.f / p.opt.mult;
   if (a->softcap < 0.f || a->softcap != a->softcap) return fail(SB_ERR_INVALID, "sb_swa_decode: softcap must be >= 0");
+  p.meta_bias_off = 0;
   if (a->softcap > 0.f || a->alibi_slopes) {
-    if (!mfma)
-      return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: soft cap / ALiBi need bf16/fp16 queries on the matrix-core kernels");
-    if (a->meta_len > 0) return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: soft cap / ALiBi together with meta tokens");
+    if (a->meta_len > 0) {
+      const int64_t rows = a->meta_bias_rows > 0 ? a->meta_bias_rows : a->num_rows;
+      const int64_t off = a->meta_bias_row0 + a->meta_len - rows;
+      if (a->meta_bias_row0 < 0 || a->meta_bias_row0 + a->num_rows > rows || off > 0x3fffffffLL || off < -0x3fffffffLL)
+        return fail(SB_ERR_INVALID, "sb_swa_decode: meta_bias_row0 %lld / meta_bias_rows %lld do not hold this call's %lld rows",
+                    (long long)a->meta_bias_row0, (long long)a->meta_bias_rows, (long long)a->num_rows);
+      p.meta_bias_off = (int)off;
+    }
     p.opt.on = 1;
     p.opt.slopes = a->alibi_slopes;
     if (a->softcap > 0.f) {

@@ -230,8 +230,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     bool vis[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      vis[j] = i0 + ((j >> 2) << 4) + 4 * g + (j & 3) < p.meta_len;
-      sc[j] = vis[j] ? sc[j] * p.meta_k_mult : kNegInf;
+      const int key = i0 + ((j >> 2) << 4) + 4 * g + (j & 3);
+      vis[j] = key < p.meta_len;
+      float x = sc[j] * p.meta_k_mult;
+      // soft cap / ALiBi: the meta rows' distance is that of the stacked second attention of the reference
+      if (p.opt.on) x = adjust_score(p.opt, x, my_slope, -fabsf((float)(p.meta_bias_off + (int)r - key)));
+      sc[j] = vis[j] ? x : kNegInf;
     }
     float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
     mx = fmaxf(mx, __shfl_xor(mx, 16));

@@ -247,8 +247,9 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
 
   // One chunk of work: S^T = K Q^T, online softmax, O^T += V^T P^T. kMask = edge chunk (keys outside
   // [mlo, mhi) are masked by their true index).
-  auto compute_chunk = [&](int ch, const Chunk &ck, auto mask_tag, const int mlo, const int mhi) {
+  auto compute_chunk = [&](int ch, const Chunk &ck, auto mask_tag, const int mlo, const int mhi, auto meta_tag) {
     constexpr bool kMask = decltype(mask_tag)::value;
+    constexpr bool kMeta = decltype(meta_tag)::value;  // a chunk of meta rows: their ALiBi term has its own distance
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -258,8 +259,11 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
     float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
     if (p.opt.on) {  // soft cap / ALiBi (wave-uniform; the query sits at key index hi - 1)
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        sc[j] = adjust_score(p.opt, sc[j], my_slope, (float)((ch << 5) + ((j >> 2) << 4) + 4 * g + (j & 3) - (hi - 1)));
+      for (int j = 0; j < 8; ++j) {
+        const int key = (ch << 5) + ((j >> 2) << 4) + 4 * g + (j & 3);
+        const float dist = kMeta ? -fabsf((float)(p.meta_bias_off + (int)r - key)) : (float)(key - (hi - 1));
+        sc[j] = adjust_score(p.opt, sc[j], my_slope, dist);
+      }
     }
     if constexpr (kMask) {
       const int i0 = ch << 5;
@@ -361,7 +365,7 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
       if (e_head) load_edge(cb, hb0, hb1, head);
 #pragma unroll
       for (int u = 0; u < kDepth; ++u) issue(ch + u, ring[u]);
-      if (e_head) compute_chunk(cb, head, kMasked, lo, hi);
+      if (e_head) compute_chunk(cb, head, kMasked, lo, hi, kUnmasked);
       const int tail_at = e_tail ? max(ib, ie - 2) : -1;
       bool more = true;
       while (more) {
@@ -370,7 +374,7 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
           if (more) {
             if (ch == tail_at) load_edge(ce - 1, tb0, tb1, tail);
             issue(ch + kDepth, ring[(u + kDepth) % (kDepth + 1)]);
-            compute_chunk(ch, ring[u], kUnmasked, lo, hi);
+            compute_chunk(ch, ring[u], kUnmasked, lo, hi, kUnmasked);
             ++ch;
             more = ch < ie;
           }
@@ -379,16 +383,16 @@ __device__ __forceinline__ void split_segment(const DecodeParams &p, const int32
     } else {
       if (e_head) load_edge(cb, hb0, hb1, head);
       if (e_tail) load_edge(ce - 1, tb0, tb1, tail);
-      if (e_head) compute_chunk(cb, head, kMasked, lo, hi);
+      if (e_head) compute_chunk(cb, head, kMasked, lo, hi, kUnmasked);
     }
-    if (e_tail) compute_chunk(ce - 1, tail, kMasked, lo, hi);
+    if (e_tail) compute_chunk(ce - 1, tail, kMasked, lo, hi, kUnmasked);
   }
 
   if (has_meta) {
-    compute_chunk(meta_first, metac, kMasked, 0, p.meta_len);
+    compute_chunk(meta_first, metac, kMasked, 0, p.meta_len, kMasked);
     for (int cc = meta_first + meta_step; cc < meta_chunks; cc += meta_step) {
       load_meta(cc, metac);
-      compute_chunk(cc, metac, kMasked, 0, p.meta_len);
+      compute_chunk(cc, metac, kMasked, 0, p.meta_len, kMasked);
     }
   }
 

@@ -63,6 +63,9 @@ struct DecodeParams {
   // Over a byte-code cache the meta rows are still elements: their scores and probabilities are multiplied by
   // these so that the scales folded into scale_log2 and kv_out_scale (fp8 cache) cancel for them; else 1.
   float meta_k_mult, meta_v_mult;
+  // ALiBi term of meta row j for query row r: -slope * |meta_bias_off + r - j|, meta_bias_off = row0 + meta_len - rows
+  // (the position flash-attn gives row r of the reference's stacked second attention)
+  int meta_bias_off;
   // soft cap / ALiBi (matrix-core kernels): applied to every raw score in front of the mask
   ScoreOptions opt;
 };

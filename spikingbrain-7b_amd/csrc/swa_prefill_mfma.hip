@@ -81,6 +81,8 @@ struct PrefillParams {
   int meta_len;
   int64_t meta_sr, meta_sh;  // bytes
   ScoreOptions opt;          // soft cap / ALiBi slopes, applied to every raw score in front of the mask
+  // ALiBi term of meta row j for packed query row t: -slope * |meta_bias_off + t - j|, meta_bias_off = row0 + meta_len - rows
+  int meta_bias_off;
 };
 
 #ifndef SB_PREFILL_HEADS
@@ -481,6 +483,17 @@ void swa_prefill_kernel(const PrefillParams p) {
       }
       __syncthreads();
       first_half(0, sa, sa, kYes, kNo);
+      if (p.opt.on) {  // soft cap / ALiBi on the meta rows: the distance of the reference's stacked second attention
+        const int c0 = mc << 5;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          const int me = p.meta_bias_off + qrow0 + min(q0 + 16 * ts[b] + c, Lq - 1);
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            sa[b][j >> 2][j & 3] = adjust_score(p.opt, sa[b][j >> 2][j & 3], my_slope[b],
+                                                -fabsf((float)(me - (c0 + ((j >> 2) << 4) + 4 * g + (j & 3)))));
+        }
+      }
       {
         const int c0 = mc << 5;
         float t[NB];
@@ -673,8 +686,15 @@ extern "C" int sb_swa_prefill(const sb_swa_prefill_args *a) {
   p.opt.mult = a->scale;  // (byte-code rows are dequantised on their way into LDS: the scores are those of elements)
   p.opt.inv_mult = 1.f / p.opt.mult;
   if (a->softcap < 0.f || a->softcap != a->softcap) return fail(SB_ERR_INVALID, "sb_swa_prefill: softcap must be >= 0");
+  p.meta_bias_off = 0;
   if (a->softcap > 0.f || a->alibi_slopes) {
-    if (a->meta_len > 0) return fail(SB_ERR_UNSUPPORTED, "sb_swa_prefill: soft cap / ALiBi together with meta tokens");
+    if (a->meta_len > 0) {
+      if (a->meta_bias_row0 < 0 || a->meta_bias_rows <= 0 || a->meta_bias_rows > 0x3fffffffLL ||
+          a->meta_bias_row0 > a->meta_bias_rows)
+        return fail(SB_ERR_INVALID, "sb_swa_prefill: soft cap / ALiBi with meta tokens need meta_bias_rows (the query rows "
+                                    "of the reference's stacked second attention) and meta_bias_row0 inside it");
+      p.meta_bias_off = (int)(a->meta_bias_row0 + a->meta_len - a->meta_bias_rows);
+    }
     p.opt.on = 1;
     p.opt.slopes = a->alibi_slopes;
     if (a->softcap > 0.f) {

@@ -535,7 +535,15 @@ class MetaAttentionImpl:
             if query2.shape[0] != self.num_meta_tokens:
                 raise AssertionError(f"query2 must hold num_meta_tokens = {self.num_meta_tokens} rows")
             num_meta_prefill_tokens += self.num_meta_tokens
-            output[:self.num_meta_tokens] = ops.meta_token_attention(query2, key2, value2, self.scale)[0]
+            options = {}
+            if self.logits_soft_cap > 0 or self.alibi_slopes is not None:
+                # the meta tokens' own queries are the last rows of the prompt call's stacked second attention
+                # (fa_kernel_metatoken.py:258-275: q = cat(q1, q2))
+                if self.alibi_slopes is not None and self.alibi_slopes.device != query.device:
+                    self.alibi_slopes = self.alibi_slopes.to(query.device)
+                options = dict(softcap=self.logits_soft_cap, alibi_slopes=self.alibi_slopes,
+                               meta_bias=(num_prefill_query_tokens, num_prefill_query_tokens + self.num_meta_tokens))
+            output[:self.num_meta_tokens] = ops.meta_token_attention(query2, key2, value2, self.scale, **options)[0]
         prefill_output = output[num_meta_prefill_tokens - num_prefill_query_tokens:num_meta_prefill_tokens]
         decode_output = output[num_meta_prefill_tokens:]
 
@@ -547,12 +555,21 @@ class MetaAttentionImpl:
         want_lse = with_meta and not meta_inside
         # The two score options (:758-759, handed to every flash-attn call of the step) travel with the
         # meta rows' arguments to whichever kernel takes a piece of the step.
+        prefill_kv, decode_kv = meta_kv, meta_kv
         if self.logits_soft_cap > 0 or self.alibi_slopes is not None:
-            if with_meta:
-                raise NotImplementedError("meta tokens together with logits_soft_cap / alibi_slopes")
+            if with_meta and not meta_inside:
+                raise NotImplementedError("meta tokens together with logits_soft_cap / alibi_slopes need bf16/fp16 queries")
             if self.alibi_slopes is not None and self.alibi_slopes.device != query.device:
                 self.alibi_slopes = self.alibi_slopes.to(query.device)
-            meta_kv = dict(softcap=self.logits_soft_cap, alibi_slopes=self.alibi_slopes)
+            options = dict(softcap=self.logits_soft_cap, alibi_slopes=self.alibi_slopes)
+            # the meta rows' ALiBi term follows the reference's second attention call, which stacks the queries of
+            # the prompt call (prompt tokens, then the meta tokens' own queries) resp. of the decode call into
+            # one sequence (fa_kernel_metatoken.py:169-188, 258-275)
+            prefill_kv = dict(meta_kv, **options)
+            decode_kv = dict(meta_kv, **options)
+            if with_meta:
+                prefill_kv["meta_bias"] = (0, num_meta_prefill_tokens)
+                decode_kv["meta_bias"] = (0, num_decode_query_tokens)
 
         def merge_meta(q_part, out_part, lse_part):
             """out_part (attention over the window, log-sum-exp lse_part) takes in the meta tokens."""
@@ -574,7 +591,7 @@ class MetaAttentionImpl:
                 elif fp8_kv:  # scaled_fp8_quant of the prompt's keys and values (:853-869)
                     pk, pv = ops.fp8_round(pk.contiguous(), k_scale_f), ops.fp8_round(pv.contiguous(), v_scale_f)
                 lse = self._varlen_inflight(query, pk, pv, prefill_meta, prefill_output, window_left,
-                                            return_lse=want_lse, meta_kv=meta_kv)
+                                            return_lse=want_lse, meta_kv=prefill_kv)
             else:
                 # prefix hit / chunked prefill: keys and values come from the paged cache (:885-919)
                 assert prefill_meta.seq_lens is not None
@@ -582,7 +599,7 @@ class MetaAttentionImpl:
                 lse = self._varlen_paged(query, key_cache, value_cache, prefill_meta.query_start_loc,
                                          prefill_meta.seq_lens_tensor, prefill_meta.block_tables,
                                          max(prefill_meta.seq_lens), prefill_output, window_left,
-                                         meta=prefill_meta, return_lse=want_lse, scales=scales, meta_kv=meta_kv)
+                                         meta=prefill_meta, return_lse=want_lse, scales=scales, meta_kv=prefill_kv)
             merge_meta(query, prefill_output, lse)
         if decode_meta := attn_metadata.decode_metadata:
             assert decode_meta.max_decode_query_len is not None
@@ -592,7 +609,7 @@ class MetaAttentionImpl:
                 lse = self._varlen_paged(decode_query, key_cache, value_cache, decode_meta.query_start_loc,
                                          decode_meta.seq_lens_tensor, decode_meta.block_tables,
                                          decode_meta.max_decode_seq_len, decode_output, window_left,
-                                         meta=decode_meta, return_lse=want_lse, scales=scales, meta_kv=meta_kv)
+                                         meta=decode_meta, return_lse=want_lse, scales=scales, meta_kv=decode_kv)
             else:
                 # one query token per sequence (:954-981); K/V were appended above, or are appended
                 # by this very launch when the step is a pure decode step
@@ -612,7 +629,7 @@ class MetaAttentionImpl:
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
                     out=decode_output, return_lse=want_lse,
                     max_seq_len=decode_meta.max_decode_seq_len or None,
-                    balanced=False if byte_kv else decode_meta._decode_balanced, **scales, **fused, **meta_kv)
+                    balanced=False if byte_kv else decode_meta._decode_balanced, **scales, **fused, **decode_kv)
                 lse = res[1] if want_lse else None
             merge_meta(decode_query, decode_output, lse)
         return output

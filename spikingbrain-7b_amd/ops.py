@@ -156,13 +156,17 @@ def swa_decode_attention(
     profile_events=None,
     softcap: float = 0.0,
     alibi_slopes: Optional[torch.Tensor] = None,
+    meta_bias: Optional[Tuple[int, int]] = None,
 ):
     """Single-query window attention for each row of q [R, Hq, D].
 
     softcap > 0: every scaled score x becomes softcap * tanh(x / softcap); alibi_slopes [Hq] fp32 (device):
     -slope[h] * (query position - key index) is added, the query sitting at the row's last key. Both in front
-    of the mask, the cap first (what flash-attn does with the backend's logits_soft_cap / alibi_slopes);
-    bf16/fp16 queries only, not together with meta tokens.
+    of the mask, the cap first (what flash-attn does with the backend's logits_soft_cap / alibi_slopes).
+    With meta rows the cap applies to their scores too and their ALiBi term is -slope[h] * |row0 + r + M - rows - j|
+    for row r and meta row j, meta_bias = (row0, rows): the call's rows are queries row0 .. of the `rows` queries
+    the reference stacks into one sequence for its second attention (fa_kernel_metatoken.py:169-188); default
+    (0, R).
 
     profile_events: (start, stop) torch.cuda.Event pair made by `timing_events()`: attached to the split
     kernel's own dispatch, so start.elapsed_time(stop) is that kernel's duration alone (fixed-split
@@ -341,6 +345,7 @@ def swa_decode_attention(
         kv_quant=N.SB_KV_FP8 if fp8_kv else (N.SB_KV_INT8 if int8_kv else N.SB_KV_NONE),
         k_scale_tensor=float(fp8_scales[0]) if fp8_kv else 0.0, v_scale_tensor=float(fp8_scales[1]) if fp8_kv else 0.0,
         softcap=float(softcap), alibi_slopes=N.ptr(_slopes(alibi_slopes, Hq, dev)),
+        meta_bias_row0=int(meta_bias[0]) if meta_bias else 0, meta_bias_rows=int(meta_bias[1]) if meta_bias else 0,
         **fused, **_event_args(profile_events))
     N.check(L.sb_swa_decode(C.byref(a)), "swa_decode")
     return (out, lse) if return_lse else out
@@ -557,10 +562,11 @@ def swa_prefill_attention(
     meta_v: Optional[torch.Tensor] = None,
     softcap: float = 0.0,
     alibi_slopes: Optional[torch.Tensor] = None,
+    meta_bias: Optional[Tuple[int, int]] = None,
 ):
     """Causal sliding-window attention for q [total_q, Hq, D] packed sequence after sequence.
     softcap / alibi_slopes: as for swa_decode_attention; query j of a sequence sits at key position
-    seq_len_k - query_len + j.
+    seq_len_k - query_len + j. With meta rows: meta_bias = (row0, rows) as there (default (0, total_q)).
     With return_lse also the fp32 [total_q, Hq] natural-log log-sum-exp of each query's scores.
     meta_k/meta_v [M, Hkv, D]: meta (sink) tokens every query also attends to, unmasked, in the same
     softmax (not over byte-code caches).
@@ -680,7 +686,9 @@ def swa_prefill_attention(
         k_scale=N.ptr(k_scale), v_scale=N.ptr(v_scale), kv_quant=kv_quant,
         k_scale_tensor=float(fp8_scales[0]) if fp8_scales is not None else 0.0,
         v_scale_tensor=float(fp8_scales[1]) if fp8_scales is not None else 0.0,
-        softcap=float(softcap), alibi_slopes=N.ptr(_slopes(alibi_slopes, Hq, dev)), **meta)
+        softcap=float(softcap), alibi_slopes=N.ptr(_slopes(alibi_slopes, Hq, dev)),
+        meta_bias_row0=int(meta_bias[0]) if meta_bias else 0,
+        meta_bias_rows=int(meta_bias[1]) if meta_bias else int(q.shape[0]), **meta)
     N.check(N.lib().sb_swa_prefill(C.byref(a)), "swa_prefill")
     return (out, lse) if return_lse else out
 
@@ -705,11 +713,15 @@ def lse_merge(out: torch.Tensor, lse: torch.Tensor, block_out: torch.Tensor, blo
     N.check(N.lib().sb_lse_merge(C.byref(a)), "lse_merge")
 
 
-def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, scale: Optional[float] = None):
+def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, scale: Optional[float] = None,
+                         softcap: float = 0.0, alibi_slopes: Optional[torch.Tensor] = None,
+                         meta_bias: Optional[Tuple[int, int]] = None):
     """Non-causal attention of every query row over the same few cached meta tokens
     (k2, v2 [M, Hkv, D]), as the second attention of fa_kernel_metatoken.py:174-188 / 261-275.
     Returns (out [rows, Hq, D], lse fp32 [rows, Hq]). Runs on the single-query kernel: every row is
-    a query at position M-1 of one shared dense sequence."""
+    a query at position M-1 of one shared dense sequence. With softcap / alibi_slopes (bf16/fp16 only) the rows
+    are queries with an empty window that take the meta rows into their softmax; meta_bias = (row0, rows) places
+    them in the reference's stacked sequence (see swa_decode_attention)."""
     dev = N.require_gpu(q, k2, v2)
     R = q.shape[0]
     M, Hkv, D = k2.shape
@@ -720,6 +732,15 @@ def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, sc
     if k2.stride() != v2.stride():
         raise ValueError("k2 and v2 must share their strides")
     zeros32 = torch.zeros(R, dtype=torch.int32, device=dev)
+    if softcap > 0 or alibi_slopes is not None:
+        if q.dtype == torch.float32:
+            raise NotImplementedError("soft cap / ALiBi over meta tokens need bf16/fp16 queries")
+        # no window keys at all (a dense dummy sequence of length 0): the meta rows are the whole softmax
+        return swa_decode_attention(
+            q, k2, v2, zeros32, kv_start=torch.zeros(1, dtype=torch.int64, device=dev), row_seq=zeros32,
+            kv_strides=(0, k2.stride(0), k2.stride(1)), num_kv_heads=Hkv, window_left=-1, scale=scale,
+            return_lse=True, max_seq_len=1, n_split=1, balanced=False, meta_k=k2, meta_v=v2, softcap=softcap,
+            alibi_slopes=alibi_slopes, meta_bias=meta_bias)
     return swa_decode_attention(
         q, k2, v2, torch.full((R,), M, dtype=torch.int32, device=dev), kv_start=torch.zeros(1, dtype=torch.int64, device=dev),
         row_seq=zeros32, kv_strides=(0, k2.stride(0), k2.stride(1)), num_kv_heads=Hkv, window_left=-1, scale=scale,

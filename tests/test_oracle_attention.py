@@ -239,3 +239,58 @@ def test_flash_window_attention_is_W_plus_one_keys_and_unpads():
     q = r.standard_normal((B, 4, K, D)); k = r.standard_normal((B, 2, K, D)); v = r.standard_normal((B, 2, K, D))
     np.testing.assert_allclose(A.flash_window_attention(q, k, v, W, am), A.sdpa_window_attention(q, k, v, W + 1, am),
                                rtol=1e-12, atol=1e-12)
+
+
+def test_metatoken_attention_with_soft_cap_and_alibi_vs_torch_two_attention_form():
+    """Score options together with meta tokens, against torch running the flash path's own form
+    (fa_kernel_metatoken.py:235-279): a causal sliding-window attention per sequence with the ALiBi term
+    -slope * (pos_q - key) written out as an additive mask, a second NON-causal attention of all stacked query
+    rows (every sequence's tokens, then the meta tokens' own queries) over the meta keys whose ALiBi term is
+    flash-attn's -slope * |i + M - N - j| for stacked row i of N, both with the cap softcap * tanh(x / softcap)
+    on the scaled scores first, merged by log-sum-exp. Two sequences, so that the stacked index differs from
+    the index inside a sequence."""
+    import torch
+    r = rng(33)
+    Hq, Hkv, D, M, W, cap = 4, 2, 8, 5, 4, 1.7
+    G = Hq // Hkv
+    scale = 0.35
+    slopes = [0.5, 0.25, 0.125, 0.0625]
+    lens = [(3, 9), (4, 4)]                      # (new tokens, keys) of the two sequences
+    N = sum(lq for lq, _ in lens) + M            # rows of the stacked second attention
+    k2 = r.standard_normal((M, Hkv, D)); v2 = r.standard_normal((M, Hkv, D))
+    q2 = r.standard_normal((M, Hq, D))
+    seqs = [(r.standard_normal((lq, Hq, D)), r.standard_normal((lk, Hkv, D)), r.standard_normal((lk, Hkv, D))) for lq, lk in lens]
+
+    def attend(q, k, v, bias, masked):           # torch: capped, biased, masked scores -> (out, lse)
+        s = torch.tensor(q) @ torch.tensor(k).T * scale
+        s = cap * torch.tanh(s / cap) + torch.tensor(bias)
+        s = s.masked_fill(torch.tensor(masked), float("-inf"))
+        return (torch.softmax(s, -1) @ torch.tensor(v)).numpy(), torch.logsumexp(s, -1).numpy()
+
+    row0 = 0
+    for si, (q1, k1, v1) in enumerate(seqs):
+        lq, lk = lens[si]
+        got = A.metatoken_attention(q1, q2 if si == 0 else None, k1, k2, v1, v2, scale, W, softcap=cap, alibi_slopes=slopes,
+                                    stack_row0=row0, stack_rows=N)
+        pos = lk - lq + np.arange(lq)
+        keys = np.arange(lk)
+        dist = pos[:, None] - keys[None, :]
+        masked = (dist < 0) | (dist >= W)
+        stacked = row0 + np.arange(lq)
+        for h in range(Hq):
+            oa, la = attend(q1[:, h], k1[:, h // G], v1[:, h // G], -slopes[h] * dist, masked)
+            mb = -slopes[h] * np.abs(stacked[:, None] + M - N - np.arange(M)[None, :])
+            ob, lb = attend(q1[:, h], k2[:, h // G], v2[:, h // G], mb, np.zeros((lq, M), bool))
+            o, _ = A.lse_merge(oa, la, ob, lb)
+            np.testing.assert_allclose(got[:lq, h], o, rtol=1e-9, atol=1e-12)
+            if si == 0:                          # the meta tokens' own queries: the last M stacked rows, meta keys only
+                st2 = N - M + np.arange(M)
+                mb2 = -slopes[h] * np.abs(st2[:, None] + M - N - np.arange(M)[None, :])
+                o2, _ = attend(q2[:, h], k2[:, h // G], v2[:, h // G], mb2, np.zeros((M, M), bool))
+                np.testing.assert_allclose(got[lq:, h], o2, rtol=1e-9, atol=1e-12)
+        row0 += lq
+    # a slope of zero and a huge cap change nothing
+    q1, k1, v1 = seqs[0]
+    plain = A.metatoken_attention(q1, None, k1, k2, v1, v2, scale, W)
+    same = A.metatoken_attention(q1, None, k1, k2, v1, v2, scale, W, softcap=1e9, alibi_slopes=[0.0] * Hq, stack_rows=N)
+    np.testing.assert_allclose(same, plain, rtol=1e-9)
