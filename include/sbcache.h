@@ -198,10 +198,11 @@ typedef struct sb_swa_decode_args {
    * here the 32-row chunks of the meta rows are dealt round robin to the splits of each query row's
    * window and enter the same online softmax, so out and lse are those of ONE softmax over window
    * and meta keys (a row with an empty window attends to the meta rows alone). meta_len = 0 = off.
-   * bf16/fp16 queries on the matrix-core kernels with the fixed split only (rejected with
-   * SB_DECODE_BALANCED, SB_DECODE_FORCE_VALU or fp32; soft cap / ALiBi: see below). Over a byte-code cache (kv_quant) the meta rows
-   * are still elements of dtype: they are not quantised, and an fp8 cache's tensor scales do not apply
-   * to them. */
+   * Fixed split only (rejected with SB_DECODE_BALANCED on the matrix-core kernels). fp32 queries and
+   * SB_DECODE_FORCE_VALU take them in the vector kernel, whose wavefronts are dealt the meta rows 16 at a
+   * time; soft cap / ALiBi: see below. Over a byte-code cache (kv_quant; bf16/fp16 queries only) the meta
+   * rows are still elements of dtype: they are not quantised, and an fp8 cache's tensor scales do not
+   * apply to them. */
   const void *meta_k;
   const void *meta_v;
   int32_t meta_len;

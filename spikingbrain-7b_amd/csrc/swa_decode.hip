@@ -162,25 +162,30 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     }
   };
 
-  auto compute_tile = [&](int t, const Pack<E> (&kb)[4], const Pack<E> (&vb)[4]) {
+  // tile t of the window (keys [lo, hi) visible), or, with `meta`, of the meta rows (rows [0, meta_len) visible)
+  auto compute_tile = [&](int t, const Pack<E> (&kb)[4], const Pack<E> (&vb)[4], const bool meta) {
     const int i0 = t << 4;
+    const int vis_lo = meta ? 0 : lo, vis_hi = meta ? p.meta_len : hi;
     float s[G][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int h = 0; h < G; ++h) s[h][j] = row16_allreduce_sum(dot_pack<E>(qp[h], kb[j]));
-    if (p.opt.on) {  // soft cap / ALiBi (wave-uniform; the query sits at key index hi - 1)
+    if (p.opt.on) {  // soft cap / ALiBi (wave-uniform; the query sits at key index hi - 1; a meta row's distance
+                     // is that of the reference's stacked second attention)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j) {
+        const int key = i0 + 4 * j + g;
+        const float dist = meta ? -fabsf((float)(p.meta_bias_off + (int)r - key)) : (float)(key - (hi - 1));
 #pragma unroll
-        for (int h = 0; h < G; ++h)
-          s[h][j] = adjust_score(p.opt, s[h][j], slope[h], (float)(i0 + 4 * j + g - (hi - 1)));
+        for (int h = 0; h < G; ++h) s[h][j] = adjust_score(p.opt, s[h][j], slope[h], dist);
+      }
     }
-    if (i0 < lo || i0 + 16 > hi) {  // edge tile: mask keys outside [lo, hi)
+    if (i0 < vis_lo || i0 + 16 > vis_hi) {  // edge tile: mask keys outside the visible range
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int i = i0 + 4 * j + g;
-        if (i < lo || i >= hi) {
+        if (i < vis_lo || i >= vis_hi) {
 #pragma unroll
           for (int h = 0; h < G; ++h) s[h][j] = kNegInf;
         }
@@ -236,7 +241,7 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
         const int64_t base2 = tile_base(min(t + 8, last));
         Pack<E> kn[4], vn[4];
         load_tile(min(t + 4, last), base1, kn, vn);
-        compute_tile(t, kb, vb);
+        compute_tile(t, kb, vb, false);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           kb[j] = kn[j];
@@ -249,7 +254,23 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     for (; t < te; t += 4) {
       Pack<E> kb[4], vb[4];
       load_tile(t, tile_base(t), kb, vb);
-      compute_tile(t, kb, vb);
+      compute_tile(t, kb, vb, false);
+    }
+  }
+  // Meta tokens: 16-row tiles of the shared meta rows, dealt to the wavefronts of all splits in turn, go into the
+  // same softmax (rows past the last one repeat it and are masked).
+  if (p.meta_len > 0) {
+    const int meta_tiles = (p.meta_len + 15) >> 4;
+    const char *mk = p.meta_k + (int64_t)kvh * p.meta_sh + c * kPackBytes, *mv = p.meta_v + (int64_t)kvh * p.meta_sh + c * kPackBytes;
+    for (int mt = split * 4 + wave; mt < meta_tiles; mt += 4 * p.n_split) {
+      Pack<E> kb[4], vb[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t off = (int64_t)min((mt << 4) + 4 * j + g, p.meta_len - 1) * p.meta_sr;
+        kb[j] = load_pack<E>(mk + off);
+        vb[j] = load_pack<E>(mv + off);
+      }
+      compute_tile(mt, kb, vb, true);
     }
   }
 
@@ -774,9 +795,9 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   if (a->meta_len < 0) return fail(SB_ERR_INVALID, "sb_swa_decode: negative meta_len");
   if (a->meta_len > 0) {
     if (!a->meta_k || !a->meta_v) return fail(SB_ERR_INVALID, "sb_swa_decode: meta_len without meta_k / meta_v");
-    if (!mfma || (a->flags & SB_DECODE_BALANCED))
+    if ((mfma && (a->flags & SB_DECODE_BALANCED)) || (!mfma && int8_kv))
       return fail(SB_ERR_UNSUPPORTED,
-                  "sb_swa_decode: meta tokens need bf16/fp16 queries on the matrix-core kernel with the fixed split");
+                  "sb_swa_decode: meta tokens go with the fixed split (and, over a byte-code cache, with bf16/fp16 queries)");
     if (((reinterpret_cast<uintptr_t>(a->meta_k) | reinterpret_cast<uintptr_t>(a->meta_v)) & 15u) ||
         (a->meta_stride_row * esz) % 16 || (a->meta_stride_head * esz) % 16 || a->meta_stride_row <= 0)
       return fail(SB_ERR_INVALID, "sb_swa_decode: meta rows must be 16-byte aligned");
@@ -848,7 +869,13 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
       if (arc != SB_OK) return arc;
     }
   }
-  if (mfma && !int8_kv && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED))
+  // (the balanced kernels number the chunks of all rows on one 32-bit axis: a row holds at most its table's
+  // or its window's keys)
+  int64_t row_chunks_max = (int64_t)1 << 26;
+  if (a->block_table) row_chunks_max = std::min<int64_t>(row_chunks_max, a->block_table_stride * (int64_t)a->block_size / 32 + 2);
+  if (a->window_left >= 0) row_chunks_max = std::min<int64_t>(row_chunks_max, (int64_t)a->window_left / 32 + 3);
+  if (mfma && !int8_kv && n_split > 1 && a->num_rows <= kBalancedMaxRows && (a->flags & SB_DECODE_BALANCED) &&
+      a->num_rows * row_chunks_max < ((int64_t)1 << 30))
     p.n_wg = (int)balanced_workgroups(a->num_rows, n_split);
   // On request the fixed split of the matrix-core kernel merges in the same launch (the last wavefront of a
   // row to finish does it), where the arrival counters fit; otherwise the merge kernel follows as usual.

@@ -28,9 +28,10 @@
 // Runs. Fixed split (kBalanced = false): grid = (rows, kv-head groups, splits), a workgroup's run is
 // chunks [cb, ce) of its row. Balanced split: the chunks of all rows are laid end to end and cut into
 // gridDim.x runs that differ by one chunk at most; a run that covers several rows writes one partial per
-// row, numbered workgroup + row, and the runs that start and end a row note their numbers for the merge. Every wavefront derives its run from seq_lens by itself (lane i looks at row
-// base + i, one wave-wide scan); the rows of a batch of 64 are then read back from those lanes, so walking
-// into the next row costs no memory access.
+// row, numbered workgroup + row, and the runs that start and end a row note their numbers for the merge.
+// Every wavefront derives its run from seq_lens by itself (lane i looks at row base + i, one wave-wide
+// scan); the rows of a batch of 64 are then read back from those lanes, so walking into the next row costs
+// no memory access.
 //
 // Built for the serving path: paged cache, one query row per sequence, no key_lo, no meta rows. Everything
 // else stays on the per-segment kernels of swa_decode_mfma.hip.
@@ -92,8 +93,7 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
   // ---- rows: lane i holds row batch0 + i ---------------------------------------------------------------
   int batch0 = 0;
   int v_lo = 0, v_hi = 0, v_n = 0, v_own = 0;
-  // loads the 64 rows from `base` on; `before` = chunks (virtual ones included) of the rows below; returns
-  // the same for the next batch
+  // loads the 64 rows from `base` on; `before` = chunks of the rows below; returns the same for the next batch
   auto load_batch = [&](int base, int before) {
     const int rr = min(base + lane, p.rows - 1);
     int hi = seq_lens[rr];
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
     const uint64_t cand = __builtin_amdgcn_ballot_w64(v_n > 0 && v_own + v_n > c0);
     i0 = __builtin_ctzll(cand);
     const int own = __builtin_amdgcn_readlane(v_own, i0);
-    if (own >= c1) return;  // the run holds nothing but virtual chunks
+    if (own >= c1) return;  // (cannot happen: the row that holds chunk c0 starts at or below it)
     const int fc = __builtin_amdgcn_readlane(v_lo, i0) >> 5, n = __builtin_amdgcn_readlane(v_n, i0);
     cb = fc + max(c0 - own, 0);
     ce = fc + min(c1 - own, n);
@@ -325,8 +325,6 @@ __global__ __launch_bounds__(256, 1) void swa_decode_stream_kernel(const DecodeP
       opaque(pv0[j]);
       opaque(pv1[j]);
     }
-    // (first, so that every wait for the item's operands covers it too; without a fused append: any valid
-    // address, the value is never used)
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
       s.k0[st] = stream16(pk0 + st * 64);

@@ -547,18 +547,13 @@ class MetaAttentionImpl:
         prefill_output = output[num_meta_prefill_tokens - num_prefill_query_tokens:num_meta_prefill_tokens]
         decode_output = output[num_meta_prefill_tokens:]
 
-        # With bf16/fp16 queries the kernels take the meta rows into their own softmax (meta_k/meta_v), over
-        # element and byte-code caches alike; fp32 queries run a second attention over the meta rows that is
-        # merged by log-sum-exp, the reference's own form.
-        meta_inside = with_meta and query.dtype in (torch.bfloat16, torch.float16)
-        meta_kv = dict(meta_k=key2, meta_v=value2) if meta_inside else {}
-        want_lse = with_meta and not meta_inside
+        # The kernels take the meta rows into their own softmax (meta_k/meta_v), over element and byte-code
+        # caches alike (the reference runs a second attention over them and merges by log-sum-exp).
+        meta_kv = dict(meta_k=key2, meta_v=value2) if with_meta else {}
         # The two score options (:758-759, handed to every flash-attn call of the step) travel with the
         # meta rows' arguments to whichever kernel takes a piece of the step.
         prefill_kv, decode_kv = meta_kv, meta_kv
         if self.logits_soft_cap > 0 or self.alibi_slopes is not None:
-            if with_meta and not meta_inside:
-                raise NotImplementedError("meta tokens together with logits_soft_cap / alibi_slopes need bf16/fp16 queries")
             if self.alibi_slopes is not None and self.alibi_slopes.device != query.device:
                 self.alibi_slopes = self.alibi_slopes.to(query.device)
             options = dict(softcap=self.logits_soft_cap, alibi_slopes=self.alibi_slopes)
@@ -570,12 +565,6 @@ class MetaAttentionImpl:
             if with_meta:
                 prefill_kv["meta_bias"] = (0, num_meta_prefill_tokens)
                 decode_kv["meta_bias"] = (0, num_decode_query_tokens)
-
-        def merge_meta(q_part, out_part, lse_part):
-            """out_part (attention over the window, log-sum-exp lse_part) takes in the meta tokens."""
-            if want_lse and q_part.shape[0] > 0:
-                meta_out, meta_lse = ops.meta_token_attention(q_part, key2, value2, self.scale)
-                ops.lse_merge(out_part, lse_part, meta_out, meta_lse)
 
         decode_query = query[num_prefill_query_tokens:]
         query = query[:num_prefill_query_tokens]
@@ -590,26 +579,24 @@ class MetaAttentionImpl:
                     pk, pv = ops.quantize_sym(pk), ops.quantize_sym(pv)
                 elif fp8_kv:  # scaled_fp8_quant of the prompt's keys and values (:853-869)
                     pk, pv = ops.fp8_round(pk.contiguous(), k_scale_f), ops.fp8_round(pv.contiguous(), v_scale_f)
-                lse = self._varlen_inflight(query, pk, pv, prefill_meta, prefill_output, window_left,
-                                            return_lse=want_lse, meta_kv=prefill_kv)
+                self._varlen_inflight(query, pk, pv, prefill_meta, prefill_output, window_left, meta_kv=prefill_kv)
             else:
                 # prefix hit / chunked prefill: keys and values come from the paged cache (:885-919)
                 assert prefill_meta.seq_lens is not None
                 assert prefill_meta.query_start_loc is not None
-                lse = self._varlen_paged(query, key_cache, value_cache, prefill_meta.query_start_loc,
-                                         prefill_meta.seq_lens_tensor, prefill_meta.block_tables,
-                                         max(prefill_meta.seq_lens), prefill_output, window_left,
-                                         meta=prefill_meta, return_lse=want_lse, scales=scales, meta_kv=prefill_kv)
-            merge_meta(query, prefill_output, lse)
+                self._varlen_paged(query, key_cache, value_cache, prefill_meta.query_start_loc,
+                                   prefill_meta.seq_lens_tensor, prefill_meta.block_tables,
+                                   max(prefill_meta.seq_lens), prefill_output, window_left,
+                                   meta=prefill_meta, scales=scales, meta_kv=prefill_kv)
         if decode_meta := attn_metadata.decode_metadata:
             assert decode_meta.max_decode_query_len is not None
             if decode_meta.max_decode_query_len > 1:
                 # several query tokens per decoding sequence (:924-953)
                 assert decode_meta.query_start_loc is not None
-                lse = self._varlen_paged(decode_query, key_cache, value_cache, decode_meta.query_start_loc,
-                                         decode_meta.seq_lens_tensor, decode_meta.block_tables,
-                                         decode_meta.max_decode_seq_len, decode_output, window_left,
-                                         meta=decode_meta, return_lse=want_lse, scales=scales, meta_kv=decode_kv)
+                self._varlen_paged(decode_query, key_cache, value_cache, decode_meta.query_start_loc,
+                                   decode_meta.seq_lens_tensor, decode_meta.block_tables,
+                                   decode_meta.max_decode_seq_len, decode_output, window_left,
+                                   meta=decode_meta, scales=scales, meta_kv=decode_kv)
             else:
                 # one query token per sequence (:954-981); K/V were appended above, or are appended
                 # by this very launch when the step is a pure decode step
@@ -624,14 +611,11 @@ class MetaAttentionImpl:
                         host_lens is not None and len(host_lens) >= n and
                         ops.plan_decode_split(n, self.num_kv_heads, decode_meta.max_decode_seq_len or max(host_lens[:n]),
                                               window_left, host_lens[:n]))
-                res = ops.swa_decode_attention(
+                ops.swa_decode_attention(
                     decode_query, key_cache, value_cache, decode_meta.seq_lens_tensor[:n],
                     block_table=decode_meta.block_tables, window_left=window_left, scale=self.scale,
-                    out=decode_output, return_lse=want_lse,
-                    max_seq_len=decode_meta.max_decode_seq_len or None,
+                    out=decode_output, max_seq_len=decode_meta.max_decode_seq_len or None,
                     balanced=False if byte_kv else decode_meta._decode_balanced, **scales, **fused, **decode_kv)
-                lse = res[1] if want_lse else None
-            merge_meta(decode_query, decode_output, lse)
         return output
 
     # -- multi-query forms: every query token becomes one row of the single-query kernel ----

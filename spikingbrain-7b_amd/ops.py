@@ -174,7 +174,7 @@ def swa_decode_attention(
 
     meta_k/meta_v [M, Hkv, D]: meta (sink) tokens every row also attends to, unmasked, inside the same
     softmax (key2/value2 of vllm_hymeta/attention/fa_kernel_metatoken.py:110-194, there a second
-    attention merged by log-sum-exp). bf16/fp16 caches with the fixed split only.
+    attention merged by log-sum-exp). Fixed split only; over a byte-code cache bf16/fp16 queries only.
 
     new_key/new_value [R, Hkv, D] + new_slot_mapping [R] int64 (all three or none): the newest key
     of each row (index seq_lens[r]-1) is taken from these tensors and stored into the paged cache
@@ -286,9 +286,8 @@ def swa_decode_attention(
         if meta_k is None or meta_v is None:
             raise ValueError("meta_k and meta_v go together")
         N.require_gpu(q, meta_k, meta_v)
-        if force_valu or q.dtype not in (torch.bfloat16, torch.float16):
-            raise NotImplementedError("meta tokens inside the decode launch need bf16/fp16 queries on the matrix-core "
-                                      "kernel (merge a separate meta_token_attention with lse_merge instead)")
+        if int8_kv and (force_valu or q.dtype not in (torch.bfloat16, torch.float16)):
+            raise NotImplementedError("meta tokens over a byte-code cache need bf16/fp16 queries on the matrix-core kernel")
         if meta_k.dim() != 3 or meta_k.shape[1:] != (Hkv, D) or meta_v.shape != meta_k.shape or \
                 meta_k.dtype != q.dtype or meta_v.dtype != q.dtype or meta_k.stride() != meta_v.stride():
             raise ValueError(f"meta_k and meta_v must be [meta_tokens, {Hkv}, {D}] of q's dtype with equal strides")
@@ -719,9 +718,9 @@ def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, sc
     """Non-causal attention of every query row over the same few cached meta tokens
     (k2, v2 [M, Hkv, D]), as the second attention of fa_kernel_metatoken.py:174-188 / 261-275.
     Returns (out [rows, Hq, D], lse fp32 [rows, Hq]). Runs on the single-query kernel: every row is
-    a query at position M-1 of one shared dense sequence. With softcap / alibi_slopes (bf16/fp16 only) the rows
-    are queries with an empty window that take the meta rows into their softmax; meta_bias = (row0, rows) places
-    them in the reference's stacked sequence (see swa_decode_attention)."""
+    a query at position M-1 of one shared dense sequence. With softcap / alibi_slopes the rows are queries with
+    an empty window that take the meta rows into their softmax; meta_bias = (row0, rows) places them in the
+    reference's stacked sequence (see swa_decode_attention)."""
     dev = N.require_gpu(q, k2, v2)
     R = q.shape[0]
     M, Hkv, D = k2.shape
@@ -733,8 +732,6 @@ def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, sc
         raise ValueError("k2 and v2 must share their strides")
     zeros32 = torch.zeros(R, dtype=torch.int32, device=dev)
     if softcap > 0 or alibi_slopes is not None:
-        if q.dtype == torch.float32:
-            raise NotImplementedError("soft cap / ALiBi over meta tokens need bf16/fp16 queries")
         # no window keys at all (a dense dummy sequence of length 0): the meta rows are the whole softmax
         return swa_decode_attention(
             q, k2, v2, zeros32, kv_start=torch.zeros(1, dtype=torch.int64, device=dev), row_seq=zeros32,

@@ -146,14 +146,16 @@ def test_meta_token_argument_errors(sb, dev):
         sb.ops.lse_merge(out, torch.zeros(8, HQ, device=dev), out[:4], torch.zeros(8, HQ, device=dev))
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("n_split,M", [(1, 128), (4, 128), (3, 100), (4, 1), (2, 33), (5, 200), (0, 128)])
 def test_decode_launch_takes_meta_tokens_into_its_softmax(sb, dev, dtype, n_split, M):
     """meta_k/meta_v inside sb_swa_decode: the meta rows' chunks are dealt to the splits of each row's
     window. Against the one-softmax oracle; and against the two-attention form the reference uses
     (window attention, meta attention, log-sum-exp merge) computed by this library's own ops. Rows:
     short, window-saturated, one with an empty window (key_lo past its keys: the meta rows alone);
-    with and without the fused append."""
+    with and without the fused append. fp32 queries run the vector kernel, which takes the meta rows the same way
+    (tolerance 1e-4 there)."""
+    tol = 1e-4 if dtype == torch.float32 else TOL
     bs, wl = 16, 300
     lens = [1, 17, 300, 301, 640, 1000, 33]
     R = len(lens)
@@ -195,12 +197,12 @@ def test_decode_launch_takes_meta_tokens_into_its_softmax(sb, dev, dtype, n_spli
     args = dict(block_table=tables.to(dev), window_left=wl, key_lo=key_lo.to(dev), n_split=n_split, max_seq_len=max(lens))
     out = sb.ops.swa_decode_attention(q.to(dev), kc.to(dev), vc.to(dev), seq.to(dev), meta_k=k2.to(dev), meta_v=v2.to(dev), **args)
     got = out.float().cpu().numpy()
-    assert np.abs(got - ref).max() <= TOL
+    assert np.abs(got - ref).max() <= tol
     # the reference's form: two attentions merged by their log-sum-exp
     o1, l1 = sb.ops.swa_decode_attention(q.to(dev), kc.to(dev), vc.to(dev), seq.to(dev), return_lse=True, **args)
     o2, l2 = sb.ops.meta_token_attention(q.to(dev), k2.to(dev), v2.to(dev))
     sb.ops.lse_merge(o1, l1, o2, l2)
-    assert np.abs(got - o1.float().cpu().numpy()).max() <= TOL
+    assert np.abs(got - o1.float().cpu().numpy()).max() <= tol
     # the log-sum-exp of the one softmax equals the merged one
     _, lse = sb.ops.swa_decode_attention(q.to(dev), kc.to(dev), vc.to(dev), seq.to(dev), meta_k=k2.to(dev), meta_v=v2.to(dev),
                                          return_lse=True, **args)
@@ -208,6 +210,7 @@ def test_decode_launch_takes_meta_tokens_into_its_softmax(sb, dev, dtype, n_spli
 
 
 def test_meta_tokens_with_fused_append_and_rejections(sb, dev):
+    """Meta rows together with the fused append (bf16 on the matrix cores, fp32 on the vector kernel), and what is refused."""
     bs, wl, M, R = 16, 64, 128, 5
     g = torch.Generator().manual_seed(5)
     lens = [1, 16, 65, 100, 129]
@@ -237,9 +240,16 @@ def test_meta_tokens_with_fused_append_and_rejections(sb, dev):
     got = sb.ops.swa_decode_attention(q, kd, vd, seq, new_key=newk, new_value=newv, new_slot_mapping=slots.to(dev), **args)
     assert (got.float() - want.float()).abs().max().item() <= TOL
     assert torch.equal(kd.cpu(), kc) and torch.equal(vd.cpu(), vc)
-    with pytest.raises(NotImplementedError):
-        sb.ops.swa_decode_attention(q.float(), kc.float().to(dev), vc.float().to(dev), seq, block_table=tables.to(dev),
-                                    window_left=wl, meta_k=k2.float(), meta_v=v2.float())
+    # fp32 queries (vector kernel): the meta rows go into the same launch there too, the append in front of it
+    kf, vf = kc.float(), vc.float()
+    kf.view(-1, HKV, D)[slots] = float("nan")
+    vf.view(-1, HKV, D)[slots] = float("nan")
+    kf, vf = kf.to(dev), vf.to(dev)
+    args32 = dict(args, meta_k=k2.float(), meta_v=v2.float())
+    got32 = sb.ops.swa_decode_attention(q.float(), kf, vf, seq, new_key=newk.float(), new_value=newv.float(),
+                                        new_slot_mapping=slots.to(dev), **args32)
+    assert (got32 - want.float()).abs().max().item() <= TOL
+    assert torch.equal(kf.cpu(), kc.float()) and torch.equal(vf.cpu(), vc.float())
     with pytest.raises(ValueError):
         sb.ops.swa_decode_attention(q, kc.to(dev), vc.to(dev), seq, block_table=tables.to(dev), window_left=wl,
                                     meta_k=k2[:, :2], meta_v=v2[:, :2])

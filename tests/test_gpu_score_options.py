@@ -3,8 +3,8 @@ kernel): the two options the backend hands to every flash-attn call
 (vllm_hymeta/attention/meta_attention.py:665-690, :758-759, :882-883, :916-918, :950-952, :978-980), in the
 decode kernels (element, INT8 and fp8 caches; fixed and balanced split), the many-query kernel (in-flight and
 paged keys) and through MetaAttentionImpl.forward, against the float64 oracle.
-Tolerance: max-abs 2e-2 (bf16), 5e-3 (fp16), against fp64 mathematics on the same (for byte-code caches:
-dequantised) rows."""
+Tolerance: max-abs 2e-2 (bf16), 5e-3 (fp16), 1e-4 (fp32), against fp64 mathematics on the same (for byte-code
+caches: dequantised) rows."""
 import numpy as np
 import pytest
 import torch
@@ -15,7 +15,7 @@ from oracle import quant as Q
 pytestmark = pytest.mark.gpu
 
 D = 128
-TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3}
+TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3, torch.float32: 1e-4}
 OPTIONS = [dict(softcap=0.0, alibi=True), dict(softcap=3.0, alibi=False), dict(softcap=1.5, alibi=True)]
 
 
@@ -143,7 +143,7 @@ def test_many_query_kernel_with_soft_cap_and_alibi(sb, dev, dtype, Hq, Hkv, opt,
     assert np.abs(plain - ref).max() > 5 * TOL[dtype]
 
 
-def test_backend_passes_the_options_on_and_rejects_what_no_kernel_takes(sb, dev):
+def test_backend_passes_the_options_on(sb, dev):
     """MetaAttentionImpl(alibi_slopes=..., logits_soft_cap=...): a prompt step over the in-flight keys, then
     decode steps through the paged cache, against the oracle with the same options."""
     Hq, Hkv, bs, wl, nb = 28, 4, 16, 40, 32
@@ -179,15 +179,6 @@ def test_backend_passes_the_options_on_and_rejects_what_no_kernel_takes(sb, dev)
         sb.MetaAttentionImpl(Hq, D, 1.0, Hkv, [0.5] * 3, wl + 1, "auto")
     with pytest.raises(ValueError, match="logits_soft_cap"):
         sb.MetaAttentionImpl(Hq, D, 1.0, Hkv, None, wl + 1, "auto", logits_soft_cap=-1.0)
-    # meta tokens with fp32 queries go through a second attention and a merge, which take neither option: refused
-    impl32 = sb.MetaAttentionImpl(Hq, D, D ** -0.5, Hkv, slopes, wl + 1, "auto", logits_soft_cap=2.5, num_meta_tokens=4)
-    runner32 = sb.runner.SwaCacheRunner(1, nb, bs, wl, Hkv, D, torch.float32, dev, max_seqs=1, max_chunk_tokens=64)
-    runner32.add_seq(0)
-    meta = runner32.build_step([(0, 8)], [])
-    q32 = torch.randn(8, Hq, D, device=dev); k32 = torch.randn(8, Hkv, D, device=dev)
-    with pytest.raises(NotImplementedError, match="bf16/fp16"):
-        impl32.forward(None, q32, k32, k32, None, torch.randn(4, Hkv, D, device=dev), torch.randn(4, Hkv, D, device=dev),
-                       runner32.kv_caches[0], meta, output=torch.empty_like(q32))
 
 
 @pytest.mark.parametrize("dtype,force_valu,G", [(torch.float32, False, 7), (torch.float32, False, 1), (torch.bfloat16, True, 7),
@@ -220,13 +211,15 @@ def _gather(kv, tables, b, n, bs):
             np.stack([kv[1][int(tables[b, i // bs]), i % bs].float().numpy() for i in range(n)]) if n else np.zeros((0,) + tuple(kv.shape[3:])))
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("opt", OPTIONS)
+@pytest.mark.parametrize("dtype,force_valu", [(torch.bfloat16, False), (torch.float16, False), (torch.float32, False),
+                                              (torch.bfloat16, True)])
+@pytest.mark.parametrize("opt", OPTIONS + [dict(softcap=0.0, alibi=False)])
 @pytest.mark.parametrize("M,n_split,stack", [(1, 1, None), (40, 3, None), (100, 2, (7, 50))])
-def test_decode_with_meta_rows_and_options(sb, dev, dtype, opt, M, n_split, stack):
+def test_decode_with_meta_rows_and_options(sb, dev, dtype, force_valu, opt, M, n_split, stack):
     """Meta rows inside the decode launch together with the score options: the cap on their scores, and the
     ALiBi term of the reference's stacked second attention, -slope |row0 + r + M - rows - j| (fa_kernel_metatoken.py:
-    169-188), against the one-softmax oracle."""
+    169-188), against the one-softmax oracle; on the matrix-core kernel and on the vector kernel (fp32 queries, or
+    forced)."""
     Hq, Hkv, bs, wl = 28, 4, 16, 70
     lens = [1, 17, 0, 65, 129, 300]
     R = len(lens)
@@ -239,7 +232,7 @@ def test_decode_with_meta_rows_and_options(sb, dev, dtype, opt, M, n_split, stac
     out = sb.ops.swa_decode_attention(
         q.to(dev), kv[0].to(dev), kv[1].to(dev), torch.tensor(lens, dtype=torch.int32, device=dev),
         block_table=tables.to(dev), window_left=wl, scale=D ** -0.5, n_split=n_split, balanced=False,
-        meta_k=k2.to(dev), meta_v=v2.to(dev), softcap=opt["softcap"],
+        meta_k=k2.to(dev), meta_v=v2.to(dev), softcap=opt["softcap"], force_valu=force_valu,
         alibi_slopes=None if slopes is None else torch.tensor(slopes, device=dev), **kw).float().cpu().numpy()
     row0, rows = stack if stack else (0, R)
     for r, n in enumerate(lens):
@@ -336,27 +329,29 @@ def test_many_query_kernel_with_meta_rows_and_options(sb, dev, dtype, opt, paged
         assert np.abs(out[qs] - ref).max() <= TOL[dtype], s_
 
 
-def test_backend_with_meta_tokens_and_options(sb, dev):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_backend_with_meta_tokens_and_options(sb, dev, dtype):
     """MetaAttentionImpl.forward with key2/value2/query2 AND logits_soft_cap / alibi_slopes: a prompt step (meta
-    queries in front of the output), then decode steps, against the oracle's stacked-sequence convention."""
+    queries in front of the output), then decode steps, against the oracle's stacked-sequence convention. fp32
+    queries take every piece of the step through the vector kernel."""
     Hq, Hkv, bs, wl, nb, M = 28, 4, 16, 40, 32, 12
     slopes = slopes_for(Hq)
     impl = sb.MetaAttentionImpl(Hq, D, D ** -0.5, Hkv, slopes, wl + 1, "auto", logits_soft_cap=2.5, num_meta_tokens=M)
-    runner = sb.runner.SwaCacheRunner(1, nb, bs, wl, Hkv, D, torch.bfloat16, dev, max_seqs=2, max_chunk_tokens=128)
+    runner = sb.runner.SwaCacheRunner(1, nb, bs, wl, Hkv, D, dtype, dev, max_seqs=2, max_chunk_tokens=128)
     g = torch.Generator().manual_seed(2)
-    k2 = torch.randn(M, Hkv, D, generator=g).bfloat16(); v2 = torch.randn(M, Hkv, D, generator=g).bfloat16()
-    q2 = (2.0 * torch.randn(M, Hq, D, generator=g)).bfloat16()
+    k2 = torch.randn(M, Hkv, D, generator=g).to(dtype); v2 = torch.randn(M, Hkv, D, generator=g).to(dtype)
+    q2 = (2.0 * torch.randn(M, Hq, D, generator=g)).to(dtype)
     hist_k = {0: [], 1: []}; hist_v = {0: [], 1: []}
     for sid in (0, 1):
         runner.add_seq(sid)
 
     def step(prompts, decodes):
         T = sum(n for _, n in prompts) + len(decodes)
-        q = (2.0 * torch.randn(T, Hq, D, generator=g)).bfloat16()
-        k = torch.randn(T, Hkv, D, generator=g).bfloat16(); v = torch.randn(T, Hkv, D, generator=g).bfloat16()
+        q = (2.0 * torch.randn(T, Hq, D, generator=g)).to(dtype)
+        k = torch.randn(T, Hkv, D, generator=g).to(dtype); v = torch.randn(T, Hkv, D, generator=g).to(dtype)
         meta = runner.build_step(prompts, decodes)
         with_q2 = bool(prompts)
-        out = torch.empty(T + (M if with_q2 else 0), Hq, D, dtype=torch.bfloat16, device=dev)
+        out = torch.empty(T + (M if with_q2 else 0), Hq, D, dtype=dtype, device=dev)
         impl.forward(None, q.to(dev), k.to(dev), v.to(dev), q2.to(dev) if with_q2 else None, k2.to(dev), v2.to(dev),
                      runner.kv_caches[0], meta, output=out)
         o = out.float().cpu().numpy()
@@ -369,9 +364,9 @@ def test_backend_with_meta_tokens_and_options(sb, dev):
             ref = A.metatoken_attention(q[t:t + n].float().numpy(), q2.float().numpy() if first else None, np.stack(hist_k[sid]),
                                         k2.float().numpy(), np.stack(hist_v[sid]), v2.float().numpy(), D ** -0.5, wl + 1,
                                         softcap=2.5, alibi_slopes=slopes, stack_row0=t, stack_rows=n_prompt + M)
-            assert np.abs(o[base + t:base + t + n] - ref[:n]).max() <= 2e-2
+            assert np.abs(o[base + t:base + t + n] - ref[:n]).max() <= TOL[dtype]
             if first:
-                assert np.abs(o[:M] - ref[n:]).max() <= 2e-2       # the meta tokens' own outputs come first
+                assert np.abs(o[:M] - ref[n:]).max() <= TOL[dtype]       # the meta tokens' own outputs come first
             first = False
             t += n
         for i, sid in enumerate(decodes):
@@ -379,7 +374,7 @@ def test_backend_with_meta_tokens_and_options(sb, dev):
             ref = A.metatoken_attention(q[t:t + 1].float().numpy(), None, np.stack(hist_k[sid]), k2.float().numpy(),
                                         np.stack(hist_v[sid]), v2.float().numpy(), D ** -0.5, wl + 1, softcap=2.5,
                                         alibi_slopes=slopes, stack_row0=i, stack_rows=len(decodes))
-            assert np.abs(o[base + t] - ref[0]).max() <= 2e-2
+            assert np.abs(o[base + t] - ref[0]).max() <= TOL[dtype]
             t += 1
 
     step([(0, 30), (1, 75)], [])
