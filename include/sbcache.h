@@ -219,7 +219,7 @@ typedef struct sb_swa_decode_args {
    * alibi_slopes ([num_q_heads] fp32, NULL = off) adds -slope[h] * (query position - key index), the query
    * sitting at key index seq_lens[r]-1. Both are applied in front of the mask, the cap first. Any query
    * type (the fp32 vector kernel takes them too); over element, INT8 and fp8 caches.
-   * Together with meta rows (bf16/fp16): the cap applies to their scores as to any other; their ALiBi term
+   * Together with meta rows (any query type): the cap applies to their scores as to any other; their ALiBi term
    * is the one flash-attn gives them in the reference's second attention call
    * (fa_kernel_metatoken.py:169-188: all query rows of the call stacked as ONE sequence of
    * meta_bias_rows queries against the meta_len meta keys, causal=False), i.e. for query row r and meta
