@@ -14,6 +14,9 @@
 //   (registers -> LDS), then either normalised and stored (n_split == 1) or written as an
 //   fp32 partial (m, l, acc) that swa_decode_merge_kernel combines.
 //   Scores are kept in log2 units: p = exp2(s*scale*log2e - m).
+//   Head sizes other than 128 (the reference's backend lists 32 .. 256 in steps of 32,
+//   vllm_hymeta/attention/meta_attention.py:57-59) run this kernel with LPR = 8 or 32 lanes per row instead of
+//   16 (a load instruction then covers 8 or 2 rows); lanes past the head's last dim carry zeros.
 #include <algorithm>
 #include <functional>
 #include <mutex>
@@ -91,10 +94,24 @@ __device__ __forceinline__ void store_out(char *out, int64_t idx, float x) {
 
 constexpr float kNegInf = -__builtin_inff();
 
-template <typename E, int G>
+// sum over each aligned group of LPR lanes
+template <int LPR>
+__device__ __forceinline__ float row_allreduce_sum(float v) {
+  if constexpr (LPR == 16) {
+    return row16_allreduce_sum(v);
+  } else {
+#pragma unroll
+    for (int o = 1; o < LPR; o <<= 1) v += __shfl_xor(v, o);
+    return v;
+  }
+}
+
+// LPR: lanes per key row (8 dims each; head sizes up to 8 LPR). NJ load instructions of 64 / LPR rows cover a tile.
+template <typename E, int G, int LPR>
 __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParams p) {
   constexpr int kPackBytes = 8 * E::kBytes;
   constexpr bool kPrefetch = (E::kBytes == 2);
+  constexpr int RPL = 64 / LPR, NJ = 16 / RPL;
 
   const int64_t r = blockIdx.x;
   const int kvh = blockIdx.y;
@@ -102,8 +119,12 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
-  const int g = lane >> 4;
-  const int c = lane & 15;
+  const int g = lane / LPR;
+  const int c_lane = lane % LPR;
+  // lanes past the head's last dim (head sizes that do not fill the LPR lanes) work on the last 8 dims with a zero
+  // query: their scores add nothing and their outputs are not stored
+  const bool live = c_lane * 8 < p.D;
+  const int c = live ? c_lane : p.D / 8 - 1;
 
   const int64_t seq = p.row_seq ? (int64_t)p.row_seq[r] : r;
   const int hi = p.seq_lens[r];
@@ -119,8 +140,13 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   // query vectors of the group, this lane's 8 dims
   Pack<E> qp[G];
 #pragma unroll
-  for (int h = 0; h < G; ++h)
+  for (int h = 0; h < G; ++h) {
     qp[h] = load_pack<E>(p.q + (r * p.q_sr + (int64_t)(kvh * G + h) * p.q_sh + c * 8) * E::kBytes);
+    if (!live) {
+#pragma unroll
+      for (int i = 0; i < E::kPackWords; ++i) qp[h].w[i] = 0u;
+    }
+  }
 
   float slope[G];  // ALiBi slopes of the group's heads
 #pragma unroll
@@ -151,11 +177,11 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   };
   // rows outside [lo, hi) are clamped onto the nearest visible key: nothing outside the window
   // is ever read, so stale or uninitialised rows cannot leak in through 0 * NaN
-  auto load_tile = [&](int t, int64_t base, Pack<E> (&kb)[4], Pack<E> (&vb)[4]) {
+  auto load_tile = [&](int t, int64_t base, Pack<E> (&kb)[NJ], Pack<E> (&vb)[NJ]) {
     const int i0 = t << 4;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int row = min(max(4 * j + g, lo - i0), hi - 1 - i0);
+    for (int j = 0; j < NJ; ++j) {
+      const int row = min(max(RPL * j + g, lo - i0), hi - 1 - i0);
       const int64_t off = base + (int64_t)row * p.kv_sr + lane_off;
       kb[j] = load_pack<E>(p.k + off);
       vb[j] = load_pack<E>(p.v + off);
@@ -163,19 +189,19 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   };
 
   // tile t of the window (keys [lo, hi) visible), or, with `meta`, of the meta rows (rows [0, meta_len) visible)
-  auto compute_tile = [&](int t, const Pack<E> (&kb)[4], const Pack<E> (&vb)[4], const bool meta) {
+  auto compute_tile = [&](int t, const Pack<E> (&kb)[NJ], const Pack<E> (&vb)[NJ], const bool meta) {
     const int i0 = t << 4;
     const int vis_lo = meta ? 0 : lo, vis_hi = meta ? p.meta_len : hi;
-    float s[G][4];
+    float s[G][NJ];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-      for (int h = 0; h < G; ++h) s[h][j] = row16_allreduce_sum(dot_pack<E>(qp[h], kb[j]));
+      for (int h = 0; h < G; ++h) s[h][j] = row_allreduce_sum<LPR>(dot_pack<E>(qp[h], kb[j]));
     if (p.opt.on) {  // soft cap / ALiBi (wave-uniform; the query sits at key index hi - 1; a meta row's distance
                      // is that of the reference's stacked second attention)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int key = i0 + 4 * j + g;
+      for (int j = 0; j < NJ; ++j) {
+        const int key = i0 + RPL * j + g;
         const float dist = meta ? -fabsf((float)(p.meta_bias_off + (int)r - key)) : (float)(key - (hi - 1));
 #pragma unroll
         for (int h = 0; h < G; ++h) s[h][j] = adjust_score(p.opt, s[h][j], slope[h], dist);
@@ -183,8 +209,8 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     }
     if (i0 < vis_lo || i0 + 16 > vis_hi) {  // edge tile: mask keys outside the visible range
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = i0 + 4 * j + g;
+      for (int j = 0; j < NJ; ++j) {
+        const int i = i0 + RPL * j + g;
         if (i < vis_lo || i >= vis_hi) {
 #pragma unroll
           for (int h = 0; h < G; ++h) s[h][j] = kNegInf;
@@ -195,14 +221,22 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     bool grew = false;
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-      const float mx = fmaxf(fmaxf(s[h][0], s[h][1]), fmaxf(s[h][2], s[h][3])) * p.scale_log2;
+      float mx;
+      if constexpr (NJ == 4) {
+        mx = fmaxf(fmaxf(s[h][0], s[h][1]), fmaxf(s[h][2], s[h][3]));
+      } else {
+        mx = s[h][0];
+#pragma unroll
+        for (int j = 1; j < NJ; ++j) mx = fmaxf(mx, s[h][j]);
+      }
+      mx *= p.scale_log2;
       const float m_new = fmaxf(m[h], mx);
       const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
       grew |= (m_new > m[h]);
       alpha[h] = fast_exp2(m[h] - m_safe);
       float psum = 0.f;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         s[h][j] = fast_exp2(fmaf(s[h][j], p.scale_log2, -m_safe));
         psum += s[h][j];
       }
@@ -216,7 +250,7 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
         for (int d = 0; d < 8; ++d) acc[h][d] *= alpha[h];
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       float vf[8];
       unpack<E>(vb[j], vf);
 #pragma unroll
@@ -234,16 +268,16 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     // path and the wait before the compute only covers the current tile's loads.
     if (t < te) {
       const int last = te - 1;
-      Pack<E> kb[4], vb[4];
+      Pack<E> kb[NJ], vb[NJ];
       load_tile(t, tile_base(t), kb, vb);
       int64_t base1 = tile_base(min(t + 4, last));
       for (; t < te; t += 4) {
         const int64_t base2 = tile_base(min(t + 8, last));
-        Pack<E> kn[4], vn[4];
+        Pack<E> kn[NJ], vn[NJ];
         load_tile(min(t + 4, last), base1, kn, vn);
         compute_tile(t, kb, vb, false);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NJ; ++j) {
           kb[j] = kn[j];
           vb[j] = vn[j];
         }
@@ -252,7 +286,7 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     }
   } else {
     for (; t < te; t += 4) {
-      Pack<E> kb[4], vb[4];
+      Pack<E> kb[NJ], vb[NJ];
       load_tile(t, tile_base(t), kb, vb);
       compute_tile(t, kb, vb, false);
     }
@@ -263,10 +297,10 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     const int meta_tiles = (p.meta_len + 15) >> 4;
     const char *mk = p.meta_k + (int64_t)kvh * p.meta_sh + c * kPackBytes, *mv = p.meta_v + (int64_t)kvh * p.meta_sh + c * kPackBytes;
     for (int mt = split * 4 + wave; mt < meta_tiles; mt += 4 * p.n_split) {
-      Pack<E> kb[4], vb[4];
+      Pack<E> kb[NJ], vb[NJ];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int64_t off = (int64_t)min((mt << 4) + 4 * j + g, p.meta_len - 1) * p.meta_sr;
+      for (int j = 0; j < NJ; ++j) {
+        const int64_t off = (int64_t)min((mt << 4) + RPL * j + g, p.meta_len - 1) * p.meta_sr;
         kb[j] = load_pack<E>(mk + off);
         vb[j] = load_pack<E>(mv + off);
       }
@@ -274,31 +308,32 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     }
   }
 
-  // ---- merge the 4 row groups of this wavefront ------------------------------------
+  // ---- merge the row groups of this wavefront ----------------------------------------
 #pragma unroll
   for (int h = 0; h < G; ++h) {
     const float mo = m[h];
-    float M = fmaxf(mo, __shfl_xor(mo, 16));
-    M = fmaxf(M, __shfl_xor(M, 32));
+    float M = mo;
+#pragma unroll
+    for (int o = LPR; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o));
     const float f = (mo == kNegInf) ? 0.f : fast_exp2(mo - M);
     float lv = l[h] * f;
-    lv += __shfl_xor(lv, 16);
-    lv += __shfl_xor(lv, 32);
+#pragma unroll
+    for (int o = LPR; o < 64; o <<= 1) lv += __shfl_xor(lv, o);
     l[h] = lv;
     m[h] = M;
 #pragma unroll
     for (int d = 0; d < 8; ++d) {
       float a = acc[h][d] * f;
-      a += __shfl_xor(a, 16);
-      a += __shfl_xor(a, 32);
+#pragma unroll
+      for (int o = LPR; o < 64; o <<= 1) a += __shfl_xor(a, o);
       acc[h][d] = a;
     }
   }
 
   // ---- merge the 4 wavefronts through LDS ---------------------------------------------
   __shared__ float s_m[4][G], s_l[4][G];
-  __shared__ __attribute__((aligned(16))) float s_acc[4][G][128];
-  if (g == 0) {
+  __shared__ __attribute__((aligned(16))) float s_acc[4][G][8 * LPR];
+  if (g == 0 && live) {
 #pragma unroll
     for (int h = 0; h < G; ++h) {
       if (c == 0) {
@@ -311,8 +346,8 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
     }
   }
   __syncthreads();
-  for (int idx = tid; idx < G * 128; idx += 256) {
-    const int h = idx >> 7, d = idx & 127;
+  for (int idx = tid; idx < G * p.D; idx += 256) {
+    const int h = p.D == 128 ? idx >> 7 : idx / p.D, d = idx - h * p.D;
     const float M = fmaxf(fmaxf(s_m[0][h], s_m[1][h]), fmaxf(s_m[2][h], s_m[3][h]));
     float tot = 0.f, L = 0.f;
     if (M != kNegInf) {
@@ -330,7 +365,7 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
       if (d == 0 && p.lse) p.lse[r * p.Hq + hq] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
     } else {
       const int64_t part = (r * p.Hq + hq) * p.n_split + split;
-      p.ws_acc[part * 128 + d] = tot;
+      p.ws_acc[part * p.D + d] = tot;
       if (d == 0) {
         p.ws_ml[part * 2] = M;
         p.ws_ml[part * 2 + 1] = L;
@@ -339,15 +374,15 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   }
 }
 
-// One 128-thread workgroup per (query row, query head): log-sum-exp merge of the splits.
+// One workgroup of head_size threads per (query row, query head): log-sum-exp merge of the splits.
 template <typename E>
-__global__ __launch_bounds__(128) void swa_decode_merge_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(256) void swa_decode_merge_kernel(const DecodeParams p) {
   const int64_t rh = blockIdx.x;  // r*Hq + hq
   const int64_t r = rh / p.Hq;
   const int hq = (int)(rh - r * p.Hq);
   const int d = threadIdx.x;
   const float *ml = p.ws_ml + rh * p.n_split * 2;
-  const float *acc = p.ws_acc + rh * p.n_split * 128 + d;
+  const float *acc = p.ws_acc + rh * p.n_split * p.D + d;
   // Four splits per trip, every load of a trip issued before any is used: with the usual split counts
   // the kernel is one round trip to memory. Across trips the running sums are rescaled to the new maximum.
   float tot = 0.f, L = 0.f, M = kNegInf;
@@ -358,7 +393,7 @@ __global__ __launch_bounds__(128) void swa_decode_merge_kernel(const DecodeParam
       const int s = min(s0 + j, p.n_split - 1);
       ms[j] = ml[2 * s];
       ls[j] = ml[2 * s + 1];
-      av[j] = acc[(int64_t)s * 128];
+      av[j] = acc[(int64_t)s * p.D];
     }
     float Mn = M;
 #pragma unroll
@@ -543,16 +578,23 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const LseMergeParams p) 
   }
 }
 
-template <typename E>
-int launch_for_group(int G, dim3 grid, hipStream_t st, const DecodeParams &p) {
+template <typename E, int LPR>
+int launch_for_group_lanes(int G, dim3 grid, hipStream_t st, const DecodeParams &p) {
   switch (G) {
-    case 1: hipLaunchKernelGGL((swa_decode_split_kernel<E, 1>), grid, dim3(256), 0, st, p); return 0;
-    case 2: hipLaunchKernelGGL((swa_decode_split_kernel<E, 2>), grid, dim3(256), 0, st, p); return 0;
-    case 4: hipLaunchKernelGGL((swa_decode_split_kernel<E, 4>), grid, dim3(256), 0, st, p); return 0;
-    case 7: hipLaunchKernelGGL((swa_decode_split_kernel<E, 7>), grid, dim3(256), 0, st, p); return 0;
-    case 8: hipLaunchKernelGGL((swa_decode_split_kernel<E, 8>), grid, dim3(256), 0, st, p); return 0;
+    case 1: hipLaunchKernelGGL((swa_decode_split_kernel<E, 1, LPR>), grid, dim3(256), 0, st, p); return 0;
+    case 2: hipLaunchKernelGGL((swa_decode_split_kernel<E, 2, LPR>), grid, dim3(256), 0, st, p); return 0;
+    case 4: hipLaunchKernelGGL((swa_decode_split_kernel<E, 4, LPR>), grid, dim3(256), 0, st, p); return 0;
+    case 7: hipLaunchKernelGGL((swa_decode_split_kernel<E, 7, LPR>), grid, dim3(256), 0, st, p); return 0;
+    case 8: hipLaunchKernelGGL((swa_decode_split_kernel<E, 8, LPR>), grid, dim3(256), 0, st, p); return 0;
     default: return -1;
   }
+}
+// lanes per key row by head size: 8 (up to 64 dims), 16 (up to 128), 32 (up to 256)
+template <typename E>
+int launch_for_group(int G, dim3 grid, hipStream_t st, const DecodeParams &p) {
+  if (p.D <= 64) return launch_for_group_lanes<E, 8>(G, grid, st, p);
+  if (p.D <= 128) return launch_for_group_lanes<E, 16>(G, grid, st, p);
+  return launch_for_group_lanes<E, 32>(G, grid, st, p);
 }
 
 inline int64_t round_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
@@ -684,8 +726,12 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   if (a->num_rows == 0) return SB_OK;
   if (!a->q || !a->k_cache || !a->v_cache || !a->out || !a->seq_lens)
     return fail(SB_ERR_INVALID, "sb_swa_decode: null tensor pointer");
-  if (a->head_size != 128)
-    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: head_size %d (only 128 is built)", a->head_size);
+  // (vllm_hymeta/attention/meta_attention.py:57-59 lists 32 .. 256 in steps of 32; the matrix-core and byte-code
+  // kernels are built for 128, the other sizes run on the vector kernel)
+  if (a->head_size < 32 || a->head_size > 256 || a->head_size % 32 != 0)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: head_size %d (built: 32 to 256 in steps of 32)", a->head_size);
+  if (a->head_size != 128 && a->kv_quant != SB_KV_NONE)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: byte-code caches are built for head_size 128 only");
   if (a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_q_heads % a->num_kv_heads != 0)
     return fail(SB_ERR_INVALID, "sb_swa_decode: num_q_heads must be a positive multiple of num_kv_heads");
   if (!(a->scale > 0.f)) return fail(SB_ERR_INVALID, "sb_swa_decode: scale must be positive");
@@ -736,7 +782,7 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   if (n_split == 0)
     n_split = sb_swa_decode_auto_split(a->num_rows, a->num_kv_heads, a->max_seq_len, a->window_left);
   if (n_split > 65535) return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: n_split > 65535");
-  const size_t need = sb_swa_decode_workspace_bytes(a->num_rows, a->num_q_heads, 128, n_split);
+  const size_t need = sb_swa_decode_workspace_bytes(a->num_rows, a->num_q_heads, a->head_size, n_split);
   if (need > 0 && (!a->workspace || a->workspace_bytes < need))
     return fail(SB_ERR_WORKSPACE, "sb_swa_decode: workspace of %zu bytes needed for n_split=%d, got %zu",
                 need, n_split, a->workspace ? a->workspace_bytes : (size_t)0);
@@ -748,13 +794,14 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   p.out = (char *)a->out; p.lse = a->lse;
   p.block_table = a->block_table; p.kv_start = a->kv_start; p.row_seq = a->row_seq;
   p.seq_lens = a->seq_lens; p.key_lo = a->key_lo;
+  p.D = a->head_size;
   const int64_t parts = partial_slots(a->num_rows, n_split) * a->num_q_heads;
   // workspace = [arrival counters of the in-kernel merge | partial numerators | partial (max, denominator)]
   p.merge_counter = nullptr;
   p.Hkv = a->num_kv_heads;
   p.ws_acc = need ? (float *)((char *)a->workspace + kMergeCounterBytes) : nullptr;
-  p.ws_ml = need ? (float *)((char *)a->workspace + kMergeCounterBytes + round_up(parts * 128 * 4, 256)) : nullptr;
-  p.ws_rows = need ? (int32_t *)((char *)a->workspace + kMergeCounterBytes + round_up(parts * 128 * 4, 256) +
+  p.ws_ml = need ? (float *)((char *)a->workspace + kMergeCounterBytes + round_up(parts * a->head_size * 4, 256)) : nullptr;
+  p.ws_rows = need ? (int32_t *)((char *)a->workspace + kMergeCounterBytes + round_up(parts * a->head_size * 4, 256) +
                                  round_up(parts * 2 * 4, 256)) : nullptr;
   p.Hq = a->num_q_heads; p.block_size = a->block_size > 0 ? a->block_size : 16;
   p.window_left = a->window_left; p.n_split = n_split;
@@ -777,7 +824,7 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   int rc = 0;
   if (a->phases < 0 || a->phases > 2) return fail(SB_ERR_INVALID, "sb_swa_decode: phases must be 0, 1 or 2");
   // bf16/fp16 run on the matrix cores (any group size up to 16); fp32 runs on the vector ALUs
-  const bool mfma = (a->dtype != SB_F32) && !(a->flags & SB_DECODE_FORCE_VALU);
+  const bool mfma = (a->dtype != SB_F32) && !(a->flags & SB_DECODE_FORCE_VALU) && a->head_size == 128;
   if (mfma ? (G > 16) : (G != 1 && G != 2 && G != 4 && G != 7 && G != 8))
     return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: GQA group size %d (built: up to 16 for bf16/fp16; 1, 2, 4, 7, 8 for fp32)", G);
   if (mfma && (a->kv_stride_row <= 0 || a->kv_stride_row * kv_esz * 16 >= (1LL << 31)))
@@ -914,9 +961,10 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
     else hipLaunchKernelGGL(swa_decode_merge_balanced_kernel<F16>, mgrid, dim3(128), 0, st, p);
     return check_launch("swa_decode_merge_balanced_kernel");
   }
-  if (a->dtype == SB_BF16) hipLaunchKernelGGL(swa_decode_merge_kernel<BF16>, mgrid, dim3(128), 0, st, p);
-  else if (a->dtype == SB_F16) hipLaunchKernelGGL(swa_decode_merge_kernel<F16>, mgrid, dim3(128), 0, st, p);
-  else hipLaunchKernelGGL(swa_decode_merge_kernel<F32>, mgrid, dim3(128), 0, st, p);
+  const dim3 mblock((unsigned)a->head_size);
+  if (a->dtype == SB_BF16) hipLaunchKernelGGL(swa_decode_merge_kernel<BF16>, mgrid, mblock, 0, st, p);
+  else if (a->dtype == SB_F16) hipLaunchKernelGGL(swa_decode_merge_kernel<F16>, mgrid, mblock, 0, st, p);
+  else hipLaunchKernelGGL(swa_decode_merge_kernel<F32>, mgrid, mblock, 0, st, p);
   return check_launch("swa_decode_merge_kernel");
 }
 
@@ -942,7 +990,7 @@ extern "C" int sb_swa_decode_static(const sb_swa_decode_args *a) {
   if (n_split < 0) return fail(SB_ERR_INVALID, "sb_swa_decode_static: negative n_split");
   if (n_split == 0)
     n_split = sb_swa_decode_auto_split(a->num_rows, a->num_kv_heads, a->max_seq_len, a->window_left);
-  const size_t need = sb_swa_decode_workspace_bytes(a->num_rows, a->num_q_heads, 128, n_split);
+  const size_t need = sb_swa_decode_workspace_bytes(a->num_rows, a->num_q_heads, a->head_size, n_split);
   if (need > (size_t)SB_SWA_DECODE_STATIC_SCRATCH_BYTES)
     return fail(SB_ERR_WORKSPACE,
                 "sb_swa_decode_static: %lld rows x %d heads in %d splits need %zu bytes of partial results, the "

@@ -66,8 +66,9 @@ struct DecodeParams {
   // ALiBi term of meta row j for query row r: -slope * |meta_bias_off + r - j|, meta_bias_off = row0 + meta_len - rows
   // (the position flash-attn gives row r of the reference's stacked second attention)
   int meta_bias_off;
-  // soft cap / ALiBi (matrix-core kernels): applied to every raw score in front of the mask
+  // soft cap / ALiBi: applied to every raw score in front of the mask
   ScoreOptions opt;
+  int D;  // head size (vector kernel and its merge; the matrix-core kernels are built for 128)
 };
 
 }  // namespace sb

@@ -48,11 +48,10 @@ class MetaAttentionBackend:
 
     @staticmethod
     def get_supported_head_sizes() -> List[int]:
-        """The reference lists 32 .. 256 in steps of 32 (meta_attention.py:57-59: what flash-attn builds);
-        the gfx950 kernels here are built for head_dim 128, the 7B model's, and the list says so, so that an
-        unsupported size is refused when the layer is constructed (`MetaAttentionImpl.__init__`, the
-        reference's own check at :694-699) and not at the first launch."""
-        return [128]
+        """The reference's list (meta_attention.py:57-59: what flash-attn builds). The matrix-core and byte-code
+        kernels here are built for head_dim 128, the 7B model's; the other sizes run every piece of a step on the
+        vector kernel (one row per query token), with element caches only."""
+        return [32, 64, 96, 128, 160, 192, 224, 256]
 
     @staticmethod
     def get_name() -> str:
@@ -440,6 +439,8 @@ class MetaAttentionImpl:
         if self.head_size not in support_head_sizes:
             raise ValueError(f"Head size {head_size} is not supported by MetaAttention. "
                              f"Supported head sizes are {support_head_sizes}.")
+        if self.head_size != 128 and self.kv_cache_dtype.startswith("fp8"):
+            raise NotImplementedError(f"MetaAttention: the fp8 kv-cache kernels are built for head size 128, not {head_size}")
         self.attn_type = attn_type
 
     def forward(
@@ -632,8 +633,8 @@ class MetaAttentionImpl:
     @staticmethod
     def _plan_for(meta, q):
         """Tile plan for the many-query matrix-core kernel, or None when it cannot take the step
-        (fp32, host lengths unknown, rows padded beyond the sequences' tokens)."""
-        if q.dtype not in (torch.bfloat16, torch.float16):
+        (fp32, a head size other than 128, host lengths unknown, rows padded beyond the sequences' tokens)."""
+        if q.dtype not in (torch.bfloat16, torch.float16) or q.shape[-1] != 128:
             return None
         plan = meta.prefill_plan(q.device)
         if plan is None or plan.total_q != q.shape[0]:

@@ -160,7 +160,7 @@ def test_backend_static_interface(sb, dev):
         B.get_kv_cache_shape(10, 8, 4, 128)
     assert B.get_impl_cls() is sb.MetaAttentionImpl and B.get_metadata_cls() is sb.MetaAttentionMetadata
     assert B.get_builder_cls() is sb.MetaAttentionMetadataBuilder
-    assert B.get_supported_head_sizes() == [128]           # what the kernels are built for: refused at construction otherwise
+    assert B.get_supported_head_sizes() == [32, 64, 96, 128, 160, 192, 224, 256]   # the reference's list (meta_attention.py:57-59)
     # copy_blocks: copy-on-write inside each layer's cache, both halves
     g = torch.Generator().manual_seed(0)
     caches = [torch.randn(2, 6, 16, 4, 128, generator=g).bfloat16().to(dev) for _ in range(2)]
@@ -210,7 +210,7 @@ def test_profile_run_and_errors(sb, dev):
         impl.forward(None, q, k, v, None, None, None, torch.empty(0), meta, output=out, output_scale=torch.ones(1))
     with pytest.raises(ValueError, match="blocksparse"):
         sb.MetaAttentionImpl(HQ, D, 1.0, HKV, None, 65, "auto", blocksparse_params={})
-    for bad in (100, 64, 256):                             # sizes the reference's list holds but no kernel here is built for
+    for bad in (100, 16, 512):                             # sizes outside the list
         with pytest.raises(ValueError, match="Head size"):
             sb.MetaAttentionImpl(HQ, bad, 1.0, HKV, None, 65, "auto")
     with pytest.raises(NotImplementedError, match="KV sharing"):
