@@ -41,8 +41,12 @@ def test_bad_shapes_rejected_before_launch(sb):
     N = sb._native
     L = N.lib()
     a = N.SwaDecodeArgs(q=16, k_cache=16, v_cache=16, out=16, seq_lens=16, num_rows=1, num_q_heads=28,
-                        num_kv_heads=4, head_size=64, block_size=16, scale=1.0, dtype=0)
-    assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_UNSUPPORTED  # head_size 64 is not built
+                        num_kv_heads=4, head_size=48, block_size=16, scale=1.0, dtype=0)
+    assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_UNSUPPORTED  # head sizes go from 32 to 256 in steps of 32
+    a.head_size = 64
+    a.kv_quant = N.SB_KV_INT8
+    assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_UNSUPPORTED  # byte-code caches: 128 only
+    a.kv_quant = N.SB_KV_NONE
     a.head_size = 128
     a.num_q_heads = 27
     assert L.sb_swa_decode(C.byref(a)) == N.SB_ERR_INVALID
