@@ -110,8 +110,9 @@ int sb_kv_append(const sb_kv_append_args *args);
  * stays zero.) Without the flag the region is not touched.
  * head_size: 32 to 256 in steps of 32, the list of vllm_hymeta/attention/meta_attention.py:57-59. At 128
  * bf16/fp16 run on the matrix cores with any GQA group size num_q_heads/num_kv_heads <= 16; fp32,
- * SB_DECODE_FORCE_VALU and every other head size run on the vector ALUs with group sizes {1,2,4,7,8}
- * (8, 16 or 32 lanes per key row). Byte-code caches (kv_quant) are built for 128 only.
+ * SB_DECODE_FORCE_VALU, larger groups and every other head size run on the vector ALUs (8, 16 or 32
+ * lanes per key row; built for 1, 2, 4, 7 or 8 query heads per workgroup, any other group size is cut
+ * into parts of one of these). Byte-code caches (kv_quant) are built for 128 and groups <= 16 only.
  * ------------------------------------------------------------------------------------ */
 #define SB_KV_NONE 0
 #define SB_KV_INT8 1

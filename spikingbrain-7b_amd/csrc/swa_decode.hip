@@ -114,7 +114,9 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   constexpr int RPL = 64 / LPR, NJ = 16 / RPL;
 
   const int64_t r = blockIdx.x;
-  const int kvh = blockIdx.y;
+  // a GQA group of p.group_parts * G query heads is served by p.group_parts workgroups of G heads each
+  const int kvh = blockIdx.y / p.group_parts;
+  const int head0 = kvh * (p.group_parts * G) + (blockIdx.y - kvh * p.group_parts) * G;
   const int split = blockIdx.z;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
   Pack<E> qp[G];
 #pragma unroll
   for (int h = 0; h < G; ++h) {
-    qp[h] = load_pack<E>(p.q + (r * p.q_sr + (int64_t)(kvh * G + h) * p.q_sh + c * 8) * E::kBytes);
+    qp[h] = load_pack<E>(p.q + (r * p.q_sr + (int64_t)(head0 + h) * p.q_sh + c * 8) * E::kBytes);
     if (!live) {
 #pragma unroll
       for (int i = 0; i < E::kPackWords; ++i) qp[h].w[i] = 0u;
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
 
   float slope[G];  // ALiBi slopes of the group's heads
 #pragma unroll
-  for (int h = 0; h < G; ++h) slope[h] = p.opt.slopes ? p.opt.slopes[kvh * G + h] : 0.f;
+  for (int h = 0; h < G; ++h) slope[h] = p.opt.slopes ? p.opt.slopes[head0 + h] : 0.f;
 
   float m[G], l[G], acc[G][8];
 #pragma unroll
@@ -359,7 +361,7 @@ __global__ __launch_bounds__(256) void swa_decode_split_kernel(const DecodeParam
         L = fmaf(s_l[w][h], f, L);
       }
     }
-    const int hq = kvh * G + h;
+    const int hq = head0 + h;
     if (p.n_split == 1) {
       store_out<E>(p.out, r * p.o_sr + (int64_t)hq * p.o_sh + d, L > 0.f ? tot / L : 0.f);
       if (d == 0 && p.lse) p.lse[r * p.Hq + hq] = L > 0.f ? (M + log2f(L)) * kLn2 : kNegInf;
@@ -823,10 +825,17 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
   hipStream_t st = (hipStream_t)a->stream;
   int rc = 0;
   if (a->phases < 0 || a->phases > 2) return fail(SB_ERR_INVALID, "sb_swa_decode: phases must be 0, 1 or 2");
-  // bf16/fp16 run on the matrix cores (any group size up to 16); fp32 runs on the vector ALUs
-  const bool mfma = (a->dtype != SB_F32) && !(a->flags & SB_DECODE_FORCE_VALU) && a->head_size == 128;
-  if (mfma ? (G > 16) : (G != 1 && G != 2 && G != 4 && G != 7 && G != 8))
-    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: GQA group size %d (built: up to 16 for bf16/fp16; 1, 2, 4, 7, 8 for fp32)", G);
+  // bf16/fp16 at head size 128 run on the matrix cores (up to 16 query heads per kv head); everything else on the vector ALUs
+  const bool mfma = (a->dtype != SB_F32) && !(a->flags & SB_DECODE_FORCE_VALU) && a->head_size == 128 && G <= 16;
+  if (int8_kv && G > 16)
+    return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: GQA group size %d over a byte-code cache (the matrix-core kernels take up to 16 query heads per kv head)", G);
+  if (a->num_q_heads > 65535) return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: grid too large");
+  // The vector kernel is built for 1, 2, 4, 7 and 8 query heads per workgroup; any other group size is cut
+  // into parts of the largest of these that divides it (the parts read the same K/V rows).
+  int vec_g = 1;
+  for (int cand : {8, 7, 4, 2})
+    if (G % cand == 0) { vec_g = cand; break; }
+  p.group_parts = mfma ? 1 : G / vec_g;
   if (mfma && (a->kv_stride_row <= 0 || a->kv_stride_row * kv_esz * 16 >= (1LL << 31)))
     return fail(SB_ERR_UNSUPPORTED, "sb_swa_decode: kv row stride %lld does not fit the kernel's 32-bit in-tile offsets",
                 (long long)a->kv_stride_row);
@@ -943,9 +952,12 @@ extern "C" int sb_swa_decode(const sb_swa_decode_args *a) {
     else if (mfma) launch_swa_decode_split_mfma(a->dtype, G, a->num_kv_heads, (unsigned)a->num_rows, (unsigned)n_split,
                                            (a->flags >> 4) & 7, st, p, (hipEvent_t)a->profile_start_event,
                                            (hipEvent_t)a->profile_stop_event);
-    else if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(G, grid, st, p);
-    else if (a->dtype == SB_F16) rc = launch_for_group<F16>(G, grid, st, p);
-    else rc = launch_for_group<F32>(G, grid, st, p);
+    else {
+      const dim3 vgrid((unsigned)a->num_rows, (unsigned)(a->num_kv_heads * p.group_parts), (unsigned)n_split);
+      if (a->dtype == SB_BF16) rc = launch_for_group<BF16>(vec_g, vgrid, st, p);
+      else if (a->dtype == SB_F16) rc = launch_for_group<F16>(vec_g, vgrid, st, p);
+      else rc = launch_for_group<F32>(vec_g, vgrid, st, p);
+    }
     if (rc == SB_OK) rc = check_launch("swa_decode_split_kernel");
   }
   if (rc != SB_OK || n_split == 1 || a->phases == 1 || p.merge_counter) return rc;

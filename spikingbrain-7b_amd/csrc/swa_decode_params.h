@@ -69,6 +69,7 @@ struct DecodeParams {
   // soft cap / ALiBi: applied to every raw score in front of the mask
   ScoreOptions opt;
   int D;  // head size (vector kernel and its merge; the matrix-core kernels are built for 128)
+  int group_parts;  // vector kernel: workgroups that share a kv head (each takes its share of the group's query heads)
 };
 
 }  // namespace sb

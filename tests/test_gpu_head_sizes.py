@@ -1,6 +1,7 @@
 """Head sizes other than 128: the backend's list is the reference's (32 .. 256 in steps of 32,
 vllm_hymeta/attention/meta_attention.py:57-59). The matrix-core kernels are built for 128; the other sizes run
-every piece of a step on the vector kernel (8, 16 or 32 lanes per key row). Against the float64 oracle.
+every piece of a step on the vector kernel (8, 16 or 32 lanes per key row). Likewise any GQA group size: the
+vector kernel cuts a group it is not built for into parts. Against the float64 oracle.
 Tolerance: max-abs 2e-2 (bf16), 5e-3 (fp16), 1e-5 (fp32; 1e-4 with soft cap / ALiBi)."""
 import numpy as np
 import pytest
@@ -121,6 +122,26 @@ def test_backend_forward_at_other_head_sizes(sb, dev, dtype, D):
     step([(2, 50)], [0, 1], chunked=True)
     for _ in range(bs + 2):
         step([], [0, 1, 2])
+
+
+@pytest.mark.parametrize("dtype,D,Hq,Hkv", [(torch.float32, 128, 12, 4), (torch.bfloat16, 128, 68, 4), (torch.float32, 128, 6, 1),
+                                             (torch.float16, 64, 9, 3), (torch.float32, 96, 15, 3), (torch.float32, 128, 28, 2),
+                                             (torch.bfloat16, 256, 22, 2)])
+def test_any_gqa_group_size(sb, dev, dtype, D, Hq, Hkv):
+    """Groups of 3, 17, 6, 3, 5, 14 and 11 query heads per kv head: beyond the matrix-core kernels' 16, or not among
+    the vector kernel's built sizes (1, 2, 4, 7, 8), a group is served as several workgroups of a built size."""
+    bs, wl = 16, 90
+    lens = [1, 16, 17, 65, 129, 300]
+    kv, tables = paged_problem(lens, bs, Hkv, D, dtype, seed=Hq)
+    q = torch.randn(len(lens), Hq, D, generator=torch.Generator().manual_seed(3)).to(dtype)
+    slopes = [2.0 ** (-8.0 * (h + 1) / Hq) for h in range(Hq)]
+    for n_split, opts in ((1, {}), (3, dict(alibi_slopes=torch.tensor(slopes, device=dev)))):
+        out = sb.ops.swa_decode_attention(q.to(dev), kv[0].to(dev), kv[1].to(dev), torch.tensor(lens, dtype=torch.int32, device=dev),
+                                          block_table=tables.to(dev), window_left=wl, scale=D ** -0.5, n_split=n_split, **opts)
+        ref = A.paged_decode_attention(q.float().numpy(), kv[0].float().numpy(), kv[1].float().numpy(), tables.numpy(), lens,
+                                       D ** -0.5, wl, alibi_slopes=slopes if opts else None)
+        tol = 1e-4 if (dtype == torch.float32 and opts) else TOL[dtype]
+        assert np.abs(out.float().cpu().numpy() - ref).max() <= tol, (n_split, bool(opts))
 
 
 def test_what_stays_at_128(sb, dev):

@@ -239,10 +239,8 @@ def test_argument_errors(sb, dev):
         sb.ops.swa_decode_attention(q, kv[0], kv[1], sl.long(), block_table=bt)
     with pytest.raises(ValueError, match="share one dtype"):
         sb.ops.swa_decode_attention(q.float(), kv[0], kv[1], sl, block_table=bt)
-    with pytest.raises(NotImplementedError, match="group size"):      # fp32 (vector-ALU kernel): group of 3 is not built
-        sb.ops.swa_decode_attention(torch.zeros(2, 12, 128, device=dev), kv[0].float(), kv[1].float(), sl, block_table=bt)
-    with pytest.raises(NotImplementedError, match="group size"):      # bf16 (matrix-core kernel): group of 17 > 16
-        sb.ops.swa_decode_attention(torch.zeros(2, 68, 128, device=dev, dtype=torch.bfloat16), kv[0], kv[1], sl, block_table=bt)
+    with pytest.raises(ValueError, match="multiple"):                 # 27 query heads over 4 kv heads
+        sb.ops.swa_decode_attention(torch.zeros(2, 27, 128, device=dev, dtype=torch.bfloat16), kv[0], kv[1], sl, block_table=bt)
     with pytest.raises(ValueError, match="dense mode"):
         sb.ops.swa_decode_attention(q, kv[0], kv[1], sl)
 
