@@ -288,6 +288,7 @@ int sb_swa_decode_static(const sb_swa_decode_args *args);
  *   out    [B, H, T, 128] dtype `dtype`
  * ------------------------------------------------------------------------------------ */
 #define SB_GLA_VECTOR_ONLY 1
+#define SB_GLA_CHECK_GATES 2 /* matrix-core block form: count gates beyond its range (see flags, sb_gla_gate_range_hits) */
 
 typedef struct sb_gla_recurrent_args {
   const void *q, *k, *v, *g;
@@ -319,9 +320,11 @@ typedef struct sb_gla_recurrent_args {
    * Gate range of the block form: inside a pair of blocks it forms exp(-(g_1 + .. + g_s)) per key dim, with
    * the exponent clamped at 80, so it is exact only while the gates of any 32 consecutive tokens sum to
    * more than -80 per key dim (|g| up to 2.5 per token, sustained; the model's log-sigmoid(x) / 16 gates
-   * reach that only for x < -40). Beyond it near-diagonal q.k terms are under-weighted without an error;
-   * callers whose gates can be that negative set SB_GLA_VECTOR_ONLY, which has no such limit (fla's
-   * fused_chunk_gla, which this path replaces, divides by the same cumulative decays inside its chunks). */
+   * reach that only for x < -40). Beyond it near-diagonal q.k terms are under-weighted; the call itself
+   * returns no error (it does not wait for the kernel); with SB_GLA_CHECK_GATES every such event adds to
+   * a device counter that sb_gla_gate_range_hits reads (a build of the kernel of its own, 0-4 % slower). Callers whose gates can be that negative
+   * set SB_GLA_VECTOR_ONLY, which has no such limit (fla's fused_chunk_gla, which this path replaces,
+   * divides by the same cumulative decays inside its chunks). */
   int32_t flags;
   /* Shared states, 0 or 1 = off. The reference computes k, v and the gate for the 4 kv heads and
    * repeats them to the 28 query heads (hf_7B_model/gla_attention.py:147-149,
@@ -338,6 +341,14 @@ typedef struct sb_gla_recurrent_args {
 } sb_gla_recurrent_args;
 
 int sb_gla_recurrent(const sb_gla_recurrent_args *args);
+
+/* Gate range check of the block form above. No counterpart in the reference (fla's kernel gives no such
+ * signal). *hits = number of times the matrix-core GLA launches made with SB_GLA_CHECK_GATES on the current
+ * device met gates beyond the range stated at `flags` (one per prompt, head, 32 key dims and pair of 16-token blocks concerned), since
+ * the counter was last cleared; reset != 0 clears it. Waits for the device (a blocking copy): call it where a synchronisation is
+ * acceptable, e.g. once after the prompts of a batch, not under stream capture. 0 hits = every block-form
+ * result so far is exact in the sense stated there. */
+int sb_gla_gate_range_hits(int64_t *hits, int32_t reset);
 
 /* ------------------------------------------------------------------------------------
  * Block copy inside one device (copy-on-write of cache blocks).

@@ -22,6 +22,7 @@ SB_DECODE_MERGE_IN_KERNEL = 4
 SB_DECODE_PER_SEGMENT = 8
 SB_KV_NONE, SB_KV_INT8, SB_KV_FP8 = 0, 1, 2
 SB_GLA_VECTOR_ONLY = 1
+SB_GLA_CHECK_GATES = 2
 SB_SWA_DECODE_STATIC_SCRATCH_BYTES = 8 << 20
 ABI_VERSION = 3
 
@@ -173,6 +174,7 @@ EXPORTS = {
     "sb_swa_decode": (C.c_int, [C.POINTER(SwaDecodeArgs)]),
     "sb_swa_decode_static": (C.c_int, [C.POINTER(SwaDecodeArgs)]),
     "sb_gla_recurrent": (C.c_int, [C.POINTER(GlaRecurrentArgs)]),
+    "sb_gla_gate_range_hits": (C.c_int, [C.POINTER(C.c_int64), C.c_int32]),
     "sb_copy_blocks": (C.c_int, [vp, vp, i64, i64, i64, vp]),
     "sb_window_shift": (C.c_int, [C.POINTER(WindowShiftArgs)]),
     "sb_swa_prefill": (C.c_int, [C.POINTER(SwaPrefillArgs)]),

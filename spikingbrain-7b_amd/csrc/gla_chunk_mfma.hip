@@ -29,14 +29,22 @@
 // the output path rounds its operands (q*exp(B), k*exp(-B), S_0) to bf16 like any bf16 GEMM.
 // exp(-(B_s + L)) grows with the gates of at most two blocks: 32 * max|g| stays far below the fp32/bf16
 // exponent range for any log-sigmoid gate (|g| up to 2.5 per token, sustained); the exponent is clamped at
-// 80 as a guard.
+// 80 as a guard. A wavefront whose gates reach the clamp in a pair of blocks (results then under-weight
+// near-diagonal terms) adds one to a device counter that sb_gla_gate_range_hits reads.
 //
 // Tile row order: accumulator tile rt of the state holds rows 32*(rt/2) + 8*(m/4) + 4*(rt%2) + m%4
 // (m = tile row), so that the 8 consecutive rows a lane needs as the B operand of q S_0 are exactly
 // the rows it already holds in tiles 2*st and 2*st+1: no cross-lane movement between the update
 // and the next block's read of the state.
+#include <mutex>
+
 #include "common.h"
 #include "mfma_util.h"
+
+// Events of gla_chunk_kernel meeting gates beyond the block form's range (one per wavefront and pair of blocks
+// concerned) since the counter was last cleared; one copy per GPU (the name is only the host's handle for
+// hipGetSymbolAddress).
+static __device__ unsigned int gla_range_hits;
 
 namespace {
 
@@ -57,6 +65,7 @@ struct GlaChunkParams {
   // stands for state head hh / jn and query head (hh / jn) * G + j0 + hh % jn; write_state: store the
   // final state. One state per head: G = jn = 1, j0 = 0, write_state = 1.
   int G, jn, j0, write_state;
+  unsigned int *range_hits;  // device counter of (wavefront, pair of blocks) events whose gates reached the exponent clamp
 };
 
 constexpr int kCB = 16;      // tokens per block
@@ -106,7 +115,9 @@ __device__ __forceinline__ float row_shr(float x) {
 __device__ __forceinline__ float bf16_to_f32(uint16_t x) { return __uint_as_float((uint32_t)x << 16); }
 __device__ __forceinline__ uint16_t f32_to_bf16(float x) { return __builtin_bit_cast(uint16_t, (__bf16)x); }  // v_cvt_pk_bf16_f32
 
-template <bool kStateF32, int GDT>
+// kCheck: report gates beyond the block form's range (SB_GLA_CHECK_GATES); a build of its own, because even this
+// little extra work shifts the register allocation of a kernel that runs at the edge of its budget (0-4 % slower).
+template <bool kStateF32, int GDT, bool kCheck>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gla_chunk_kernel(const GlaChunkParams p) {
   const int b = blockIdx.x / p.H;
   const int hh = blockIdx.x - b * p.H;
@@ -205,6 +216,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if constexpr (kSecond) x += carry[i];
       B[i] = x;
       tot[i] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane | 15) << 2, __builtin_bit_cast(int, x)));
+    }
+    // Gate range: the largest exponent formed inside a pair of blocks is minus its total log-decay. Checked where
+    // the pair ends, and reported on the spot (a flag carried through the loop costs this kernel 6 %: it runs at
+    // the edge of its register budget).
+    if constexpr (kSecond && kCheck) {
+      const float worst = fminf(fminf(fminf(tot[0], tot[1]), fminf(tot[2], tot[3])), fminf(fminf(tot[4], tot[5]), fminf(tot[6], tot[7])));
+      if (__builtin_amdgcn_ballot_w64(worst < -kMaxExp * kLog2e) != 0 && lane == 0) atomicAdd(p.range_hits, 1u);
     }
     float qf[8], kf[8];
 #pragma unroll
@@ -352,15 +370,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if (blk < n_blocks) {
     __syncthreads();
     multiply(blk * kCB, stage[0], kFirst);
+    float worst = 0.f;  // (a last block without a partner: its own total is the exponent range it used)
 #pragma unroll
     for (int rt = 0; rt < 8; ++rt) {
       const float4 dc = *reinterpret_cast<const float4 *>(&stage[0].dec[32 * (rt >> 1) + 8 * g + 4 * (rt & 1)]);
+      if constexpr (kCheck) worst = fminf(worst, fminf(fminf(dc.x, dc.y), fminf(dc.z, dc.w)));
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
         S[rt][nt][0] *= fast_exp2(dc.x); S[rt][nt][1] *= fast_exp2(dc.y);
         S[rt][nt][2] *= fast_exp2(dc.z); S[rt][nt][3] *= fast_exp2(dc.w);
       }
     }
+    if constexpr (kCheck)
+      if (__builtin_amdgcn_ballot_w64(worst < -kMaxExp * kLog2e) != 0 && tid == 0) atomicAdd(p.range_hits, 1u);
   }
 
   if (!p.write_state) return;
@@ -378,11 +400,58 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 }  // namespace
 
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_hits_mu;
+unsigned int *g_hits_ptr[kMaxDevices];  // per device: address of that device's copy of gla_range_hits
+
+// Address of the current device's counter (looked up once per device), or null with the error set.
+unsigned int *range_hits_ptr() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    sb_host::set_error("gla_chunk: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_hits_mu);
+  if (!g_hits_ptr[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(gla_range_hits));
+    if (e != hipSuccess || !ptr) {
+      sb_host::set_error("gla_chunk: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_hits_ptr[dev] = (unsigned int *)ptr;
+  }
+  return g_hits_ptr[dev];
+}
+}  // namespace
+
+extern "C" int sb_gla_gate_range_hits(int64_t *hits, int32_t reset) {
+  using namespace sb_host;
+  if (!hits) return fail(SB_ERR_INVALID, "sb_gla_gate_range_hits: null pointer");
+  unsigned int *ptr = range_hits_ptr();
+  if (!ptr) return SB_ERR_INVALID;
+  unsigned int h = 0;
+  hipError_t e = hipMemcpy(&h, ptr, sizeof(h), hipMemcpyDeviceToHost);  // waits for the work queued before it
+  if (e != hipSuccess) return fail((int)e, "sb_gla_gate_range_hits: hipMemcpy: %s", hipGetErrorString(e));
+  if (reset) {
+    e = hipMemset(ptr, 0, sizeof(h));
+    if (e != hipSuccess) return fail((int)e, "sb_gla_gate_range_hits: hipMemset: %s", hipGetErrorString(e));
+  }
+  *hits = (int64_t)h;
+  return SB_OK;
+}
+
 namespace sb_host {
 
 // Launch for bf16 q/k/v/out; g of any built type. Grid: one workgroup per (row, head).
-void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads, int G, int jn, int j0, int write_state) {
+// Returns SB_OK, or an error when the device's hit counter cannot be located (nothing is launched then).
+int launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads, int G, int jn, int j0, int write_state) {
   GlaChunkParams p;
+  const bool check = (a->flags & SB_GLA_CHECK_GATES) != 0;
+  p.range_hits = check ? range_hits_ptr() : nullptr;
+  if (check && !p.range_hits) return SB_ERR_INVALID;
   p.q = (const uint16_t *)a->q; p.k = (const uint16_t *)a->k; p.v = (const uint16_t *)a->v; p.g = a->g;
   p.state = a->state; p.out = (uint16_t *)a->out; p.slot_idx = a->slot_idx; p.cu = a->cu_seqlens;
   p.H = heads; p.T = a->seq_len; p.scale = a->scale;
@@ -395,7 +464,11 @@ void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads,
   p.s_slot = a->state_stride_slot; p.s_head = a->state_stride_head;
   const dim3 grid((unsigned)groups), block(256);
   hipStream_t st = (hipStream_t)a->stream;
-#define SB_LAUNCH(F32S, GDT) hipLaunchKernelGGL((gla_chunk_kernel<F32S, GDT>), grid, block, 0, st, p)
+#define SB_LAUNCH(F32S, GDT)                                                                     \
+  do {                                                                                           \
+    if (check) hipLaunchKernelGGL((gla_chunk_kernel<F32S, GDT, true>), grid, block, 0, st, p);   \
+    else hipLaunchKernelGGL((gla_chunk_kernel<F32S, GDT, false>), grid, block, 0, st, p);        \
+  } while (0)
   if (a->state_dtype == SB_F32) {
     if (a->g_dtype == SB_F32) SB_LAUNCH(true, SB_F32);
     else if (a->g_dtype == SB_BF16) SB_LAUNCH(true, SB_BF16);
@@ -406,6 +479,7 @@ void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads,
     else SB_LAUNCH(false, SB_F16);
   }
 #undef SB_LAUNCH
+  return SB_OK;
 }
 
 }  // namespace sb_host

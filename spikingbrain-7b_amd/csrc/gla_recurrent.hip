@@ -500,7 +500,7 @@ void launch_sequence(const GlaParams &p, dim3 grid, hipStream_t st) {
 }  // namespace
 
 namespace sb_host {
-void launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads, int G, int jn, int j0, int write_state);
+int launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads, int G, int jn, int j0, int write_state);
 }
 
 // Calls of this many steps or more (and every packed call) with bf16 q, k, v run on the matrix cores.
@@ -573,9 +573,11 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
     // one workgroup per query head busy), all reading the group's state. The group's first head stores
     // the final state, in a launch of its own behind the others so that no head reads a state already
     // advanced.
-    if (G > 1) launch_gla_chunk(a, a->batch * (int64_t)Hk * (G - 1), Hk * (G - 1), G, G - 1, 1, 0);
-    if (G > 1) launch_gla_chunk(a, a->batch * (int64_t)Hk, Hk, G, 1, 0, 1);
-    else launch_gla_chunk(a, groups, a->num_heads, 1, 1, 0, 1);
+    int rc = SB_OK;
+    if (G > 1) rc = launch_gla_chunk(a, a->batch * (int64_t)Hk * (G - 1), Hk * (G - 1), G, G - 1, 1, 0);
+    if (G > 1 && rc == SB_OK) rc = launch_gla_chunk(a, a->batch * (int64_t)Hk, Hk, G, 1, 0, 1);
+    else if (G <= 1) rc = launch_gla_chunk(a, groups, a->num_heads, 1, 1, 0, 1);
+    if (rc != SB_OK) return rc;
     return check_launch("gla_chunk_kernel");
   }
   if (a->cu_seqlens && !vectors_ok)

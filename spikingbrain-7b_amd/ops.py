@@ -744,15 +744,27 @@ def meta_token_attention(q: torch.Tensor, k2: torch.Tensor, v2: torch.Tensor, sc
         return_lse=True, max_seq_len=M, n_split=1)
 
 
+def gla_gate_range_hits(reset: bool = False) -> int:
+    """How often the matrix-core GLA launches made with check_gates=True on the current device met gates beyond the block form's range (a
+    pair of 16-token blocks whose log-gates sum below -80 for some key dim: results there under-weight
+    near-diagonal terms; `vector_only=True` has no such limit) since the counter was last cleared: one count per
+    prompt, head, 32 key dims and pair of blocks concerned. Waits for the device."""
+    hits = C.c_int64(0)
+    N.check(N.lib().sb_gla_gate_range_hits(C.byref(hits), 1 if reset else 0), "gla_gate_range_hits")
+    return int(hits.value)
+
+
 def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
                   slot_idx: Optional[torch.Tensor] = None, scale: Optional[float] = None,
-                  out: Optional[torch.Tensor] = None, vector_only: bool = False, profile_events=None) -> torch.Tensor:
+                  out: Optional[torch.Tensor] = None, vector_only: bool = False, profile_events=None,
+                  check_gates: bool = False) -> torch.Tensor:
     """q, k, v, g [B, H, T, D] (any batch/head/time strides, contiguous D); state
     [slots, H, D, D] fp32 or bf16, updated in place; returns o [B, H, T, D] in q's dtype.
     Rows with slot_idx == -1 are skipped (state and output untouched).
     Calls of 32 steps or more with bf16 q/k/v run 16 tokens at a time on the matrix cores (state, gates
     and accumulation in fp32, bf16 operand rounding on the output path); vector_only=True keeps them on
-    the step-by-step fp32 kernel.
+    the step-by-step fp32 kernel. check_gates=True: the block form counts gates beyond its range (see
+    gla_gate_range_hits).
     Shared states: k, v, g may come with Hkv < H heads (H a multiple of Hkv, up to 8 query heads per kv
     head) and state as [slots, Hkv, D, D]: query head h then works on head h // (H // Hkv) of them, which is
     the reference's repeat_kv of k, v and the gate (hf_7B_model/gla_attention.py:147-149) without the
@@ -796,7 +808,8 @@ def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
         g_stride_b=g.stride(0), g_stride_h=g.stride(1), g_stride_t=g.stride(2),
         out_stride_b=out.stride(0), out_stride_h=out.stride(1), out_stride_t=out.stride(2),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
-        num_slots=state.shape[0], stream=N.stream_ptr(dev), flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0,
+        num_slots=state.shape[0], stream=N.stream_ptr(dev),
+        flags=(N.SB_GLA_VECTOR_ONLY if vector_only else 0) | (N.SB_GLA_CHECK_GATES if check_gates else 0),
         q_heads_per_state=H // Hk, **_event_args(profile_events))
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
@@ -813,7 +826,8 @@ def _state_heads(num_q_heads: int, num_k_heads: int) -> int:
 def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
                          cu_seqlens: torch.Tensor, slot_idx: Optional[torch.Tensor] = None,
                          scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
-                         max_seq_len: Optional[int] = None, vector_only: bool = False) -> torch.Tensor:
+                         max_seq_len: Optional[int] = None, vector_only: bool = False,
+                         check_gates: bool = False) -> torch.Tensor:
     """The same recurrence over packed prompts: q, k, v, g [total_tokens, H, D] (token/head strides
     free, contiguous D), sequence b owning tokens cu_seqlens[b] .. cu_seqlens[b+1]-1 (int32 device
     vector [B+1]); its state is state[slot_idx[b]] (default b), advanced in place. One launch for
@@ -859,7 +873,8 @@ def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: t
         out_stride_b=0, out_stride_h=out.stride(1), out_stride_t=out.stride(0),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
         num_slots=state.shape[0], stream=N.stream_ptr(dev), cu_seqlens=N.ptr(cu_seqlens),
-        flags=N.SB_GLA_VECTOR_ONLY if vector_only else 0, q_heads_per_state=H // Hk)
+        flags=(N.SB_GLA_VECTOR_ONLY if vector_only else 0) | (N.SB_GLA_CHECK_GATES if check_gates else 0),
+        q_heads_per_state=H // Hk)
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
 

@@ -283,9 +283,40 @@ def test_block_form_strong_gates_and_gate_dtypes(sb, dev, gdtype, strength):
     ref_o, ref_S = G.gla_recurrent(q.float().numpy(), k.float().numpy(), v.float().numpy(), gate.float().numpy(), None)
     fd = fused.to(dev)
     qd, kd, vd = (fd[..., i * D:(i + 1) * D].transpose(1, 2) for i in range(3))
+    sb.ops.gla_gate_range_hits(reset=True)
     o, S = sb.fused_recurrent_gla(qd, kd, vd, gate.to(dev), output_final_state=True)
     assert rel(S.double().cpu().numpy(), ref_S) <= STATE_RTOL
     assert out_close(o.float().cpu().numpy(), ref_o)
+    # the same call with the range check on: same results, nothing counted (inside the block form's range)
+    st = torch.zeros(B, H, D, D, device=dev)
+    o2 = sb.ops.gla_recurrent(qd, kd, vd, gate.to(dev), st, check_gates=True)
+    assert torch.equal(o2, o) and torch.equal(st, S)
+    assert sb.ops.gla_gate_range_hits() == 0
+
+
+def test_gates_beyond_the_block_forms_range_are_counted(sb, dev):
+    """32 consecutive log-gates summing below -80 for some key dim put exp(-(cumulative gate)) beyond the exponent
+    the block form allows itself: every (prompt, head) workgroup that meets such gates counts itself in the
+    device counter that sb_gla_gate_range_hits reads when the call asks for the check (the call itself cannot
+    report it: it does not wait for the kernel). Two prompts of a packed launch, one with strong gates in one head only; vector_only has no such
+    range and counts nothing."""
+    H, D = 2, 128
+    lens = [64, 48]
+    T = sum(lens)
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(T, H, D, generator=g).bfloat16().to(dev) for _ in range(3))
+    gate = -0.5 * torch.rand(T, H, D, generator=g)
+    gate[64:112, 1, 5] = -3.0                              # prompt 1, head 1, one key dim: 32 tokens x -3 per pair of blocks
+    cu = torch.tensor([0, lens[0], T], dtype=torch.int32, device=dev)
+    sb.ops.gla_gate_range_hits(reset=True)
+    for vector_only, expect in ((False, 1), (True, 0)):
+        state = torch.zeros(2, H, D, D, device=dev)
+        sb.ops.gla_recurrent_packed(q, k, v, gate.to(dev), state, cu, max_seq_len=max(lens), vector_only=vector_only,
+                                    check_gates=True)
+        assert sb.ops.gla_gate_range_hits(reset=True) == expect, vector_only
+    # without the flag the kernel is the unchecked build: nothing is counted
+    sb.ops.gla_recurrent_packed(q, k, v, gate.to(dev), torch.zeros(2, H, D, D, device=dev), cu, max_seq_len=max(lens))
+    assert sb.ops.gla_gate_range_hits() == 0
 
 
 @pytest.mark.parametrize("gdtype", [torch.float32, torch.float16, torch.bfloat16])
