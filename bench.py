@@ -299,6 +299,34 @@ def bench_gla_prompt(sb, dev, S=16, L=8192, H=28, iters=3):
             "vector_only_kernel_ms": round(times["vector_only"], 3)}
 
 
+def bench_gla_prompt_shared(sb, dev, H=28, Hk=4, iters=3):
+    """The same 131 072 prompt tokens through a GLA layer that keeps one state per kv head (k, v and the gate with
+    4 heads, q with 28), as 16 long and as 64 shorter prompts: one workgroup per query head (two ordered
+    launches) against one workgroup per group of 7 query heads (one launch, the state advanced once)."""
+    res = {"workload": f"GLA layer with one state per kv head, 131 072 prompt tokens, {H} q / {Hk} kv heads, bf16 q/k/v, fp32 gate and state"}
+    for S, L in ((16, 8192), (64, 2048)):
+        g = torch.Generator().manual_seed(0)
+        tokens = S * L
+        q = torch.randn(tokens, H, D, generator=g).bfloat16().to(dev)
+        k, v = (torch.randn(tokens, Hk, D, generator=g).bfloat16().to(dev) for _ in range(2))
+        gate = (torch.nn.functional.logsigmoid(torch.randn(tokens, Hk, D, generator=g)) / 16).to(dev)
+        cache = torch.zeros(S, Hk, D, D, device=dev)
+        cu = torch.arange(0, tokens + 1, L, dtype=torch.int32, device=dev)
+        out = torch.empty_like(q)
+        entry = {}
+        for name, per_head in (("per_query_head_ms", True), ("per_group_ms", False), ("as_dispatched_ms", None)):
+            sb.ops.gla_recurrent_packed(q, k, v, gate, cache, cu, out=out, max_seq_len=L, per_head=per_head)
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+            for a, b in evs:
+                a.record()
+                sb.ops.gla_recurrent_packed(q, k, v, gate, cache, cu, out=out, max_seq_len=L, per_head=per_head)
+                b.record()
+            torch.cuda.synchronize()
+            entry[name] = round(statistics.mean(a.elapsed_time(b) for a, b in evs), 3)
+        res[f"{S}x{L}"] = entry
+    return res
+
+
 def bench_hybrid(sb, dev, B=256, steps=128, warmup=4, kv_quant=None, gla_state_dtype=torch.float32,
                  gla_shared_states=False):
     """BASELINE config 5: the cache work of 128 consecutive decode steps of the 28-layer stack
@@ -399,7 +427,7 @@ def main():
     ap.add_argument("--extras", action="store_true", help="also time the GLA state update (config 3), chunked prefill (config 4) and the "
                                                     "28-layer hybrid decode step (config 5)")
     ap.add_argument("--only", choices=("prefill", "hybrid", "hybrid_int8", "hybrid_fp8", "hybrid_lean", "hybrid_shared",
-                                       "hybrid_leanest", "gla_prompt", "gla_step", "decode_sweep"), default=None,
+                                       "hybrid_leanest", "gla_prompt", "gla_prompt_shared", "gla_step", "decode_sweep"), default=None,
                     help="run just that section and print its JSON (short runs for profiling one kernel)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -418,6 +446,9 @@ def main():
         return
     if args.only == "gla_prompt":
         print(json.dumps({"gla_prompt": bench_gla_prompt(sb, dev)}))
+        return
+    if args.only == "gla_prompt_shared":
+        print(json.dumps({"gla_prompt_shared_states": bench_gla_prompt_shared(sb, dev)}))
         return
     if args.only == "gla_step":
         print(json.dumps({"gla_state_update": bench_gla_step(sb, dev), "gla_state_update_b256": bench_gla_step(sb, dev, B3=256, iters=40)}))
@@ -585,6 +616,7 @@ def main():
         line["prefill"] = bench_prefill(sb, dev)
         torch.cuda.empty_cache()
         line["gla_prompt"] = bench_gla_prompt(sb, dev)
+        line["gla_prompt_shared_states"] = bench_gla_prompt_shared(sb, dev)
         torch.cuda.empty_cache()
         line["hybrid_decode_int8_kv"] = bench_hybrid(sb, dev, kv_quant="int8")
         torch.cuda.empty_cache()

@@ -289,6 +289,8 @@ int sb_swa_decode_static(const sb_swa_decode_args *args);
  * ------------------------------------------------------------------------------------ */
 #define SB_GLA_VECTOR_ONLY 1
 #define SB_GLA_CHECK_GATES 2 /* matrix-core block form: count gates beyond its range (see flags, sb_gla_gate_range_hits) */
+#define SB_GLA_PER_HEAD 4 /* shared states, matrix-core block form: one workgroup per query head (two launches), whatever the batch */
+#define SB_GLA_GROUP_PASS 8 /* ... one workgroup per group of query heads (one launch), whatever the batch; default: by batch size */
 
 typedef struct sb_gla_recurrent_args {
   const void *q, *k, *v, *g;
@@ -333,6 +335,12 @@ typedef struct sb_gla_recurrent_args {
    * q_heads_per_state = G > 1, k, v, g and state have num_heads / G heads (query head h uses head
    * h / G of them), q and out keep num_heads heads, and every state is read and written once per
    * step for its whole group: the state traffic of a decode step drops G-fold, results unchanged.
+   * Prompts on the matrix cores (the block form above) come in two shapes with the same bits: one workgroup
+   * per query head, each carrying the recurrence for its own outputs (two ordered launches, the group's
+   * first head stores the state), or one workgroup per group, which advances the state once and forms all
+   * G outputs against it (vllm_hymeta/model_for_7B/gla_attention.py:264-267 "can be optimised later"); the
+   * second where batch x (num_heads / G) >= 112 groups fill the machine by themselves, SB_GLA_PER_HEAD /
+   * SB_GLA_GROUP_PASS to choose by hand.
    * num_heads must be a multiple of G, G <= 8. */
   int32_t q_heads_per_state;
   /* Optional timing of the decode-step kernel (one token, one state per head), as for sb_swa_decode. */

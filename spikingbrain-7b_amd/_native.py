@@ -23,6 +23,8 @@ SB_DECODE_PER_SEGMENT = 8
 SB_KV_NONE, SB_KV_INT8, SB_KV_FP8 = 0, 1, 2
 SB_GLA_VECTOR_ONLY = 1
 SB_GLA_CHECK_GATES = 2
+SB_GLA_PER_HEAD = 4
+SB_GLA_GROUP_PASS = 8
 SB_SWA_DECODE_STATIC_SCRATCH_BYTES = 8 << 20
 ABI_VERSION = 3
 

@@ -398,6 +398,306 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
 }
 
+
+// ---- one pass for a whole GQA group (shared states) -----------------------------------------------------------
+// One workgroup per (sequence, state head): the state is advanced ONCE per block and the outputs of all G query
+// heads of the group are formed against it, instead of one workgroup per query head each carrying the whole
+// recurrence (G - 1 of them only for their outputs). Per head the arithmetic and its order are those of
+// gla_chunk_kernel (same operands, same matrix instructions in the same sequence), so the results are the same
+// bits. The q operands of the G heads sit side by side in LDS; k-hat, v and the decays are prepared once.
+constexpr int kMaxGroup = 8;
+
+struct GroupStage {
+  uint16_t qs[kMaxGroup][kCB][kRow];
+  uint16_t ks[kCB][kRow];
+  uint16_t kl[kCB][kRow];
+  uint16_t vs[kCB][kRow];
+  float dec[128];
+};
+
+template <bool kStateF32, int GDT>
+__global__ __launch_bounds__(256) void gla_chunk_group_kernel(const GlaChunkParams p) {
+  const int b = blockIdx.x / p.H;   // p.H: state heads here
+  const int hk = blockIdx.x - b * p.H;
+  const int G = p.G;
+  const int64_t slot = p.slot_idx ? (int64_t)p.slot_idx[b] : (int64_t)b;
+  if (slot < 0) return;
+  int T = p.T;
+  int64_t qo, ko, vo, go, oo;
+  if (p.cu) {
+    const int64_t t0 = p.cu[b];
+    T = p.cu[b + 1] - (int)t0;
+    qo = t0 * p.q_st; ko = t0 * p.k_st; vo = t0 * p.v_st; go = t0 * p.g_st; oo = t0 * p.o_st;
+  } else {
+    qo = b * p.q_sb; ko = b * p.k_sb; vo = b * p.v_sb; go = b * p.g_sb; oo = b * p.o_sb;
+  }
+  if (T <= 0) return;
+  qo += (int64_t)hk * G * p.q_sh; ko += hk * p.k_sh; vo += hk * p.v_sh; go += hk * p.g_sh; oo += (int64_t)hk * G * p.o_sh;
+
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int g = lane >> 4, c = lane & 15;
+  const int r = tid >> 4;
+
+  extern __shared__ __attribute__((aligned(16))) char group_smem[];
+  GroupStage *const stage = reinterpret_cast<GroupStage *>(group_smem);
+
+  char *sbase = reinterpret_cast<char *>(p.state) + (slot * p.s_slot + (int64_t)hk * p.s_head) * (kStateF32 ? 4 : 2);
+  f32x4_t S[8][2];
+  auto state_index = [&](int rt, int nt, int i) {
+    return (32 * (rt >> 1) + 8 * g + 4 * (rt & 1) + i) * 128 + 32 * w + 16 * nt + c;
+  };
+#pragma unroll
+  for (int rt = 0; rt < 8; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int idx = state_index(rt, nt, i);
+        S[rt][nt][i] = kStateF32 ? reinterpret_cast<const float *>(sbase)[idx]
+                                 : bf16_to_f32(reinterpret_cast<const uint16_t *>(sbase)[idx]);
+      }
+
+  constexpr int kGateBytes = GDT == SB_F32 ? 4 : 2;
+  const char *gb = reinterpret_cast<const char *>(p.g) + go * kGateBytes;
+  const char *qb = reinterpret_cast<const char *>(p.q + qo), *kb = reinterpret_cast<const char *>(p.k + ko),
+             *vb_ = reinterpret_cast<const char *>(p.v + vo);
+  const int64_t g_row = p.g_st * kGateBytes, q_row = p.q_st * 2, k_row = p.k_st * 2, v_row = p.v_st * 2, o_row = p.o_st * 2;
+  const int q_head = (int)(p.q_sh * 2), o_head = (int)(p.o_sh * 2);  // bytes between the group's heads (host-checked to fit)
+  struct BlockIn {
+    uint4 q[kMaxGroup], k, v;
+    uint4 g[kGateBytes / 2];
+  };
+  auto fetch = [&](int t0, BlockIn &in) {
+    const int tok = min(c, T - 1 - t0);
+    const __amdgpu_buffer_rsrc_t qr = rows_from(qb + t0 * q_row);
+#pragma unroll
+    for (int h = 0; h < kMaxGroup; ++h)
+      if (h < G) in.q[h] = load16(qr, tok * (int)q_row + h * q_head + r * 16);
+    in.k = load16(rows_from(kb + t0 * k_row), tok * (int)k_row + r * 16);
+    in.v = load16(rows_from(vb_ + t0 * v_row), tok * (int)v_row + r * 16);
+    const __amdgpu_buffer_rsrc_t gr = rows_from(gb + t0 * g_row);
+#pragma unroll
+    for (int j = 0; j < kGateBytes / 2; ++j) in.g[j] = load16(gr, tok * (int)g_row + r * 8 * kGateBytes + 16 * j);
+  };
+  auto fix_tail = [&](BlockIn &in, int t0) {
+    if (t0 + kCB > T && t0 + c >= T) {
+#pragma unroll
+      for (int h = 0; h < kMaxGroup; ++h) in.q[h] = make_uint4(0u, 0u, 0u, 0u);
+      in.k = in.v = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int j = 0; j < kGateBytes / 2; ++j) in.g[j] = make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+  float carry[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) carry[i] = 0.f;
+  auto prepare = [&](const BlockIn &in, GroupStage &st, auto second_tag) {
+    constexpr bool kSecond = decltype(second_tag)::value;
+    const uint4 rk = in.k, rv = in.v;
+    float B[8], tot[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float x;
+      if constexpr (GDT == SB_F32) x = __uint_as_float(word(in.g[i >> 2], i & 3));
+      else if constexpr (GDT == SB_BF16) x = (i & 1) ? bf16_hi(word(in.g[0], i >> 1)) : bf16_lo(word(in.g[0], i >> 1));
+      else x = (i & 1) ? f16_hi(word(in.g[0], i >> 1)) : f16_lo(word(in.g[0], i >> 1));
+      x *= kLog2e;
+      x += row_shr<1>(x);
+      x += row_shr<2>(x);
+      x += row_shr<4>(x);
+      x += row_shr<8>(x);
+      if constexpr (kSecond) x += carry[i];
+      B[i] = x;
+      tot[i] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane | 15) << 2, __builtin_bit_cast(int, x)));
+    }
+    float eq[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) eq[i] = fast_exp2(B[i]);
+#pragma unroll
+    for (int h = 0; h < kMaxGroup; ++h)
+      if (h < G) {
+        const uint4 rq = in.q[h];
+        uint32_t qs[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          qs[i] = Mma<BF16>::pack(bf16_lo(word(rq, i)) * p.scale * eq[2 * i], bf16_hi(word(rq, i)) * p.scale * eq[2 * i + 1]);
+        *reinterpret_cast<uint4 *>(&st.qs[h][c][8 * r]) = make_uint4(qs[0], qs[1], qs[2], qs[3]);
+      }
+    float kf[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      kf[2 * i] = bf16_lo(word(rk, i));
+      kf[2 * i + 1] = bf16_hi(word(rk, i));
+    }
+    uint32_t ks[4], kl[4];
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      const float x0 = kf[i] * fast_exp2(fminf(-B[i], kMaxExp * kLog2e)), x1 = kf[i + 1] * fast_exp2(fminf(-B[i + 1], kMaxExp * kLog2e));
+      const uint32_t h = Mma<BF16>::pack(x0, x1);
+      const uint32_t l = Mma<BF16>::pack(x0 - __uint_as_float(h << 16), x1 - __uint_as_float(h & 0xffff0000u));
+      ks[i / 2] = h;
+      kl[i / 2] = l;
+    }
+    *reinterpret_cast<uint4 *>(&st.ks[c][8 * r]) = make_uint4(ks[0], ks[1], ks[2], ks[3]);
+    *reinterpret_cast<uint4 *>(&st.kl[c][8 * r]) = make_uint4(kl[0], kl[1], kl[2], kl[3]);
+    *reinterpret_cast<uint4 *>(&st.vs[c][8 * r]) = rv;
+    if constexpr (kSecond) {
+      *reinterpret_cast<float4 *>(&st.dec[8 * r]) = make_float4(fast_exp2(tot[0]), fast_exp2(tot[1]), fast_exp2(tot[2]), fast_exp2(tot[3]));
+      *reinterpret_cast<float4 *>(&st.dec[8 * r + 4]) = make_float4(fast_exp2(tot[4]), fast_exp2(tot[5]), fast_exp2(tot[6]), fast_exp2(tot[7]));
+    } else {
+      *reinterpret_cast<float4 *>(&st.dec[8 * r]) = make_float4(tot[0], tot[1], tot[2], tot[3]);
+      *reinterpret_cast<float4 *>(&st.dec[8 * r + 4]) = make_float4(tot[4], tot[5], tot[6], tot[7]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) carry[i] = tot[i];
+    }
+  };
+
+  auto multiply = [&](int t0, const GroupStage &st, auto second_tag) {
+    constexpr bool kSecond = decltype(second_tag)::value;
+    // what every head of the group shares: k-hat as the score operand, v, and the state before the block as
+    // the operand of q S_0
+    uint4 ka[4];
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) ka[s4] = *reinterpret_cast<const uint4 *>(&st.ks[c][32 * s4 + 8 * g]);
+    uint4 vb[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const uint2 x = load_transposed(&st.vs[4 * g + (c >> 2)][32 * w + 16 * nt + 4 * (c & 3)]);
+      vb[nt] = make_uint4(x.x, x.y, x.x, x.y);
+    }
+    uint4 sb16[4][2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) {
+        const f32x4_t &a = S[2 * s4][nt], &bb = S[2 * s4 + 1][nt];
+        sb16[s4][nt] = make_uint4(Mma<BF16>::pack(a[0], a[1]), Mma<BF16>::pack(a[2], a[3]),
+                                  Mma<BF16>::pack(bb[0], bb[1]), Mma<BF16>::pack(bb[2], bb[3]));
+      }
+    // NP heads at a time, their chains of dependent matrix instructions taken in turn (a head alone is one
+    // chain: four instructions for its scores, then five per output tile)
+    auto heads = [&](int h0, auto np_tag) __attribute__((always_inline)) {
+      constexpr int NP = decltype(np_tag)::value;
+      uint4 qa[NP][4];
+      f32x4_t at[NP];
+#pragma unroll
+      for (int u = 0; u < NP; ++u) at[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+          qa[u][s4] = *reinterpret_cast<const uint4 *>(&st.qs[h0 + u][c][32 * s4 + 8 * g]);
+          at[u] = Mma<BF16>::run(ka[s4], qa[u][s4], at[u]);
+        }
+      uint4 pa[NP];
+#pragma unroll
+      for (int u = 0; u < NP; ++u) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (4 * g + i > c) at[u][i] = 0.f;
+        const uint32_t h01 = Mma<BF16>::pack(at[u][0], at[u][1]), h23 = Mma<BF16>::pack(at[u][2], at[u][3]);
+        pa[u] = make_uint4(h01, h23,
+                           Mma<BF16>::pack(at[u][0] - __uint_as_float(h01 << 16), at[u][1] - __uint_as_float(h01 & 0xffff0000u)),
+                           Mma<BF16>::pack(at[u][2] - __uint_as_float(h23 << 16), at[u][3] - __uint_as_float(h23 & 0xffff0000u)));
+      }
+      f32x4_t o[NP][2];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int u = 0; u < NP; ++u) o[u][nt] = Mma<BF16>::run(vb[nt], pa[u], f32x4_t{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int u = 0; u < NP; ++u) o[u][nt] = Mma<BF16>::run(sb16[s4][nt], qa[u][s4], o[u][nt]);
+#pragma unroll
+      for (int u = 0; u < NP; ++u) {
+        // (a descriptor per head: its bound drops the rows past the end of the prompt, whatever the head stride)
+        const __amdgpu_buffer_rsrc_t orows = __builtin_amdgcn_make_buffer_rsrc(
+            reinterpret_cast<char *>(p.out + oo) + t0 * o_row + (int64_t)(h0 + u) * o_head, 0, min(kCB, T - t0) * (int)o_row,
+            0x00020000);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+          typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+          u32x2_t val;
+          val.x = Mma<BF16>::pack(o[u][nt][0], o[u][nt][1]);
+          val.y = Mma<BF16>::pack(o[u][nt][2], o[u][nt][3]);
+          __builtin_amdgcn_raw_buffer_store_b64(val, orows, c * (int)o_row + (32 * w + 16 * nt + 4 * g) * 2, 0, 0);
+        }
+      }
+    };
+    {
+      int h = 0;
+      for (; h + 2 <= G; h += 2) heads(h, std::integral_constant<int, 2>{});
+      if (h < G) heads(h, std::integral_constant<int, 1>{});
+    }
+#pragma unroll
+    for (int rt = 0; rt < 8; ++rt) {
+      const int tok = 4 * g + (c >> 2), dims = 32 * (rt >> 1) + 8 * (c & 3) + 4 * (rt & 1);
+      const uint2 h2 = load_transposed(&st.ks[tok][dims]);
+      const uint2 l2 = load_transposed(&st.kl[tok][dims]);
+      const uint4 kt = make_uint4(h2.x, h2.y, l2.x, l2.y);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) S[rt][nt] = Mma<BF16>::run(kt, vb[nt], S[rt][nt]);
+      if constexpr (kSecond) {
+        const float4 dc = *reinterpret_cast<const float4 *>(&st.dec[32 * (rt >> 1) + 8 * g + 4 * (rt & 1)]);
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+          S[rt][nt][0] *= dc.x; S[rt][nt][1] *= dc.y; S[rt][nt][2] *= dc.z; S[rt][nt][3] *= dc.w;
+        }
+      }
+    }
+  };
+
+  const int n_blocks = (T + kCB - 1) / kCB;
+  const std::false_type kFirst{};
+  const std::true_type kSecond{};
+  BlockIn in;
+  fetch(0, in);
+  fix_tail(in, 0);
+  prepare(in, stage[0], kFirst);
+  fetch(min(1, n_blocks - 1) * kCB, in);
+  int blk = 0;
+  for (; blk + 1 < n_blocks; blk += 2) {
+    __syncthreads();
+    fix_tail(in, (blk + 1) * kCB);
+    multiply(blk * kCB, stage[0], kFirst);
+    prepare(in, stage[1], kSecond);
+    fetch(min(blk + 2, n_blocks - 1) * kCB, in);
+    __syncthreads();
+    fix_tail(in, (blk + 2) * kCB);
+    multiply((blk + 1) * kCB, stage[1], kSecond);
+    prepare(in, stage[0], kFirst);
+    fetch(min(blk + 3, n_blocks - 1) * kCB, in);
+  }
+  if (blk < n_blocks) {
+    __syncthreads();
+    multiply(blk * kCB, stage[0], kFirst);
+#pragma unroll
+    for (int rt = 0; rt < 8; ++rt) {
+      const float4 dc = *reinterpret_cast<const float4 *>(&stage[0].dec[32 * (rt >> 1) + 8 * g + 4 * (rt & 1)]);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        S[rt][nt][0] *= fast_exp2(dc.x); S[rt][nt][1] *= fast_exp2(dc.y);
+        S[rt][nt][2] *= fast_exp2(dc.z); S[rt][nt][3] *= fast_exp2(dc.w);
+      }
+    }
+  }
+#pragma unroll
+  for (int rt = 0; rt < 8; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int idx = state_index(rt, nt, i);
+        if (kStateF32) reinterpret_cast<float *>(sbase)[idx] = S[rt][nt][i];
+        else reinterpret_cast<uint16_t *>(sbase)[idx] = f32_to_bf16(S[rt][nt][i]);
+      }
+}
+
 }  // namespace
 
 namespace {
@@ -468,6 +768,49 @@ int launch_gla_chunk(const sb_gla_recurrent_args *a, int64_t groups, int heads, 
   do {                                                                                           \
     if (check) hipLaunchKernelGGL((gla_chunk_kernel<F32S, GDT, true>), grid, block, 0, st, p);   \
     else hipLaunchKernelGGL((gla_chunk_kernel<F32S, GDT, false>), grid, block, 0, st, p);        \
+  } while (0)
+  if (a->state_dtype == SB_F32) {
+    if (a->g_dtype == SB_F32) SB_LAUNCH(true, SB_F32);
+    else if (a->g_dtype == SB_BF16) SB_LAUNCH(true, SB_BF16);
+    else SB_LAUNCH(true, SB_F16);
+  } else {
+    if (a->g_dtype == SB_F32) SB_LAUNCH(false, SB_F32);
+    else if (a->g_dtype == SB_BF16) SB_LAUNCH(false, SB_BF16);
+    else SB_LAUNCH(false, SB_F16);
+  }
+#undef SB_LAUNCH
+  return SB_OK;
+}
+
+// Shared states, one pass: grid = one workgroup per (row, state head), each forming the outputs of its G query
+// heads. SB_ERR_UNSUPPORTED (nothing launched) where the group's head offsets do not fit the kernel's 32-bit
+// in-block offsets; the caller then takes the launches per query head.
+int launch_gla_chunk_group(const sb_gla_recurrent_args *a, int state_heads, int G) {
+  if (G < 2 || G > kMaxGroup) return SB_ERR_UNSUPPORTED;
+  if ((int64_t)G * a->q_stride_h * 2 >= (1LL << 30) || (int64_t)G * a->out_stride_h * 2 >= (1LL << 30) ||
+      a->q_stride_h < 0 || a->out_stride_h < 0)
+    return SB_ERR_UNSUPPORTED;
+  GlaChunkParams p;
+  p.range_hits = nullptr;
+  p.q = (const uint16_t *)a->q; p.k = (const uint16_t *)a->k; p.v = (const uint16_t *)a->v; p.g = a->g;
+  p.state = a->state; p.out = (uint16_t *)a->out; p.slot_idx = a->slot_idx; p.cu = a->cu_seqlens;
+  p.H = state_heads; p.T = a->seq_len; p.scale = a->scale;
+  p.G = G; p.jn = 1; p.j0 = 0; p.write_state = 1;
+  p.q_sb = a->q_stride_b; p.q_sh = a->q_stride_h; p.q_st = a->q_stride_t;
+  p.k_sb = a->k_stride_b; p.k_sh = a->k_stride_h; p.k_st = a->k_stride_t;
+  p.v_sb = a->v_stride_b; p.v_sh = a->v_stride_h; p.v_st = a->v_stride_t;
+  p.g_sb = a->g_stride_b; p.g_sh = a->g_stride_h; p.g_st = a->g_stride_t;
+  p.o_sb = a->out_stride_b; p.o_sh = a->out_stride_h; p.o_st = a->out_stride_t;
+  p.s_slot = a->state_stride_slot; p.s_head = a->state_stride_head;
+  const dim3 grid((unsigned)(a->batch * (int64_t)state_heads)), block(256);
+  hipStream_t st = (hipStream_t)a->stream;
+  constexpr int kLds = 2 * (int)sizeof(GroupStage);
+#define SB_LAUNCH(F32S, GDT)                                                                                  \
+  do {                                                                                                        \
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gla_chunk_group_kernel<F32S, GDT>),    \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);                     \
+    if (e != hipSuccess) return fail((int)e, "gla_chunk_group_kernel: %s", hipGetErrorString(e));             \
+    hipLaunchKernelGGL((gla_chunk_group_kernel<F32S, GDT>), grid, block, kLds, st, p);                        \
   } while (0)
   if (a->state_dtype == SB_F32) {
     if (a->g_dtype == SB_F32) SB_LAUNCH(true, SB_F32);

@@ -757,14 +757,16 @@ def gla_gate_range_hits(reset: bool = False) -> int:
 def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
                   slot_idx: Optional[torch.Tensor] = None, scale: Optional[float] = None,
                   out: Optional[torch.Tensor] = None, vector_only: bool = False, profile_events=None,
-                  check_gates: bool = False) -> torch.Tensor:
+                  check_gates: bool = False, per_head: Optional[bool] = None) -> torch.Tensor:
     """q, k, v, g [B, H, T, D] (any batch/head/time strides, contiguous D); state
     [slots, H, D, D] fp32 or bf16, updated in place; returns o [B, H, T, D] in q's dtype.
     Rows with slot_idx == -1 are skipped (state and output untouched).
     Calls of 32 steps or more with bf16 q/k/v run 16 tokens at a time on the matrix cores (state, gates
     and accumulation in fp32, bf16 operand rounding on the output path); vector_only=True keeps them on
     the step-by-step fp32 kernel. check_gates=True: the block form counts gates beyond its range (see
-    gla_gate_range_hits).
+    gla_gate_range_hits). per_head (shared states, block form): True = one workgroup per query head, False = one
+    per group of query heads (the state advanced once for the group), None = chosen by the number of groups; the
+    results are the same bits either way.
     Shared states: k, v, g may come with Hkv < H heads (H a multiple of Hkv, up to 8 query heads per kv
     head) and state as [slots, Hkv, D, D]: query head h then works on head h // (H // Hkv) of them, which is
     the reference's repeat_kv of k, v and the gate (hf_7B_model/gla_attention.py:147-149) without the
@@ -809,7 +811,8 @@ def gla_recurrent(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
         out_stride_b=out.stride(0), out_stride_h=out.stride(1), out_stride_t=out.stride(2),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
         num_slots=state.shape[0], stream=N.stream_ptr(dev),
-        flags=(N.SB_GLA_VECTOR_ONLY if vector_only else 0) | (N.SB_GLA_CHECK_GATES if check_gates else 0),
+        flags=(N.SB_GLA_VECTOR_ONLY if vector_only else 0) | (N.SB_GLA_CHECK_GATES if check_gates else 0)
+        | (0 if per_head is None else (N.SB_GLA_PER_HEAD if per_head else N.SB_GLA_GROUP_PASS)),
         q_heads_per_state=H // Hk, **_event_args(profile_events))
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
@@ -827,7 +830,7 @@ def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: t
                          cu_seqlens: torch.Tensor, slot_idx: Optional[torch.Tensor] = None,
                          scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
                          max_seq_len: Optional[int] = None, vector_only: bool = False,
-                         check_gates: bool = False) -> torch.Tensor:
+                         check_gates: bool = False, per_head: Optional[bool] = None) -> torch.Tensor:
     """The same recurrence over packed prompts: q, k, v, g [total_tokens, H, D] (token/head strides
     free, contiguous D), sequence b owning tokens cu_seqlens[b] .. cu_seqlens[b+1]-1 (int32 device
     vector [B+1]); its state is state[slot_idx[b]] (default b), advanced in place. One launch for
@@ -873,7 +876,8 @@ def gla_recurrent_packed(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: t
         out_stride_b=0, out_stride_h=out.stride(1), out_stride_t=out.stride(0),
         state_stride_slot=state.stride(0), state_stride_head=state.stride(1),
         num_slots=state.shape[0], stream=N.stream_ptr(dev), cu_seqlens=N.ptr(cu_seqlens),
-        flags=(N.SB_GLA_VECTOR_ONLY if vector_only else 0) | (N.SB_GLA_CHECK_GATES if check_gates else 0),
+        flags=(N.SB_GLA_VECTOR_ONLY if vector_only else 0) | (N.SB_GLA_CHECK_GATES if check_gates else 0)
+        | (0 if per_head is None else (N.SB_GLA_PER_HEAD if per_head else N.SB_GLA_GROUP_PASS)),
         q_heads_per_state=H // Hk)
     N.check(N.lib().sb_gla_recurrent(C.byref(a)), "gla_recurrent")
     return out
