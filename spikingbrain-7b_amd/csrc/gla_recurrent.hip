@@ -581,7 +581,8 @@ extern "C" int sb_gla_recurrent(const sb_gla_recurrent_args *a) {
     // One pass per group (the state advanced once, the outputs of all its query heads formed against it) where
     // the groups alone fill the machine: one workgroup per group does 0.4 x the work of one per query head but
     // runs a single wavefront per SIMD; measured on 131 072 prompt tokens, 28 : 4 heads: 16 / 24 / 32 / 64 / 256
-    // prompts 2.22 / 1.20 / 1.19 / 0.75 / 0.79 ms against 1.78 / 1.24 / 1.39 / 1.17 / 1.23. SB_GLA_GROUP_PASS /
+    // prompts 2.22 / 1.20 / 1.19 / 0.75 / 0.79 ms against 1.78 / 1.24 / 1.39 / 1.17 / 1.23; groups of 2 / 3 / 4 / 8
+    // heads at 64 prompts 0.33 / 0.40 / 0.45 / 0.80 ms against 0.49 / 0.60 / 0.77 / 1.33. SB_GLA_GROUP_PASS /
     // SB_GLA_PER_HEAD choose by hand; the gate check exists only per head.
     const bool group_pass = (a->flags & SB_GLA_GROUP_PASS) ||
                             (!(a->flags & SB_GLA_PER_HEAD) && a->batch * (int64_t)Hk >= kGroupPassMinGroups);
