@@ -70,8 +70,10 @@ static std::vector<uint16_t> random_bf16(size_t n, Lcg &g, float scale = 1.f) {
 }
 
 // ---- paged window attention: sb_kv_append + sb_swa_decode (two splits, so workspace and merge run too) ----
-static int check_attention() {
-  const int B = 3, Hq = 28, Hkv = 4, D = 128, bs = 16, wl = 64, nb = 32, G = Hq / Hkv, width = 8;
+// (D = 128 with 28 : 4 heads is the 7B shape on the matrix cores; another head size or a group the vector kernel is
+// not built for goes through the same entry points)
+static int check_attention(const int D, const int Hq, const int Hkv) {
+  const int B = 3, bs = 16, wl = 64, nb = 32, G = Hq / Hkv, width = 8;
   const int lens[B] = {40, 100, 17};  // keys of each sequence once this step's token is appended
   Lcg g{1};
   std::vector<uint16_t> kc = random_bf16((size_t)nb * bs * Hkv * D, g), vc = random_bf16((size_t)nb * bs * Hkv * D, g);
@@ -151,7 +153,7 @@ static int check_attention() {
       for (int d = 0; d < D; ++d)
         worst = std::max(worst, std::fabs(o[d] / den - from_bf16(out[((size_t)b * Hq + h) * D + d])));
     }
-  std::printf("attention: max abs error %.3e (bound 2e-2)\n", worst);
+  std::printf("attention (head size %d, %d : %d heads): max abs error %.3e (bound 2e-2)\n", D, Hq, Hkv, worst);
   HIP_OK(hipFree(d_k)); HIP_OK(hipFree(d_v)); HIP_OK(hipFree(d_q)); HIP_OK(hipFree(d_nk)); HIP_OK(hipFree(d_nv));
   HIP_OK(hipFree(d_table)); HIP_OK(hipFree(d_lens)); HIP_OK(hipFree(d_slots)); HIP_OK(hipFree(d_out)); HIP_OK(hipFree(d_ws));
   return worst <= 2e-2 ? 0 : 1;
@@ -230,7 +232,7 @@ int main() {
     return 4;
   }
   HIP_OK(hipSetDevice(0));
-  const int bad = check_attention() + check_gla();
+  const int bad = check_attention(128, 28, 4) + check_attention(64, 12, 4) + check_gla();
   std::printf(bad ? "FAILED\n" : "ok\n");
   return bad ? 1 : 0;
 }

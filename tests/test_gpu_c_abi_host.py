@@ -19,4 +19,6 @@ def test_cpp_host_program_drives_the_library():
     run = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     assert run.returncode == 0, run.stdout + run.stderr
     assert run.stdout.strip().endswith("ok"), run.stdout
-    assert "attention: max abs error" in run.stdout and "gla: state max abs error" in run.stdout
+    assert "attention (head size 128, 28 : 4 heads): max abs error" in run.stdout
+    assert "attention (head size 64, 12 : 4 heads): max abs error" in run.stdout
+    assert "gla: state max abs error" in run.stdout
